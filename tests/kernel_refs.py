@@ -1,0 +1,159 @@
+"""Plain PyTorch counterparts of the HIP kernels, one function per kernel, with the
+same call signatures as ``yalis_amd.ops.hip.HipOps``.
+
+Two uses: the GPU tests compare each kernel with its counterpart here at sizes of
+their own; and ``RefOps`` lets the CPU tests run the framework's host logic (batching,
+paging, scheduling) without a GPU.  It is test equipment: the framework never imports
+it.  Everything is computed in float32 and rounded once to the output dtype.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+
+def embed(token_ids, table):
+    return table[token_ids.long()].to(torch.float32)
+
+
+def add_rmsnorm(residual, delta, weight, eps, unit_offset, out_dtype):
+    """residual += delta in place (float32); returns the normalised rows."""
+    if delta is not None:
+        residual += delta.to(torch.float32)
+    return _rmsnorm(residual, weight, eps, unit_offset).to(out_dtype)
+
+
+def gather_add_rmsnorm(residual, delta, rows, weight, eps, unit_offset, out_dtype):
+    v = residual[rows.long()]
+    if delta is not None:
+        v = v + delta[rows.long()].to(torch.float32)
+    return _rmsnorm(v, weight, eps, unit_offset).to(out_dtype)
+
+
+def _rmsnorm(x, weight, eps, unit_offset):
+    ms = (x * x).mean(dim=-1, keepdim=True)
+    w = weight.to(torch.float32)
+    if unit_offset:
+        w = w + 1.0
+    return x * torch.rsqrt(ms + eps) * w
+
+
+def linear(x, w, out_dtype):
+    return (x.to(torch.float32) @ w.to(torch.float32).T).to(out_dtype)
+
+
+def rope_append(qkv, n_heads, n_kv, head_dim, positions, cos, sin, rotary_dim, interleaved,
+                k_cache, v_cache, slots, page_size):
+    """Rotates the query heads of ``qkv`` in place; rotates the key heads and stores
+    them, and the value heads transposed, at each token's slot of the pages."""
+    n = qkv.shape[0]
+    x = qkv.view(n, n_heads + 2 * n_kv, head_dim)
+    rot = x[:, : n_heads + n_kv].to(torch.float32)
+    if rotary_dim:
+        c = cos[positions.long()][:, None, :]
+        s = sin[positions.long()][:, None, :]
+        if interleaved:
+            a = rot[..., 0:rotary_dim:2]
+            b = rot[..., 1:rotary_dim:2]
+        else:
+            a = rot[..., : rotary_dim // 2]
+            b = rot[..., rotary_dim // 2 : rotary_dim]
+        ra = a * c - b * s
+        rb = b * c + a * s
+        rot = rot.clone()
+        if interleaved:
+            rot[..., 0:rotary_dim:2] = ra
+            rot[..., 1:rotary_dim:2] = rb
+        else:
+            rot[..., : rotary_dim // 2] = ra
+            rot[..., rotary_dim // 2 : rotary_dim] = rb
+    rot = rot.to(qkv.dtype)
+    x[:, :n_heads] = rot[:, :n_heads]
+    if n_kv:
+        page = (slots // page_size).long()
+        off = (slots % page_size).long()
+        k_cache[page, :, off, :] = rot[:, n_heads:]
+        v_cache[page, :, :, off] = x[:, n_heads + n_kv :]
+
+
+def attention_paged(q, k_cache, v_cache, positions, token_seq, block_table, page_size, scale, window):
+    """q: [N, H, D]; pages as in the framework (keys [pages, G, page, D], values
+    [pages, G, D, page]).  Gathers each token's visible keys through its request's
+    block table and runs a float32 softmax."""
+    n, n_heads, d = q.shape
+    n_kv = k_cache.shape[1]
+    qpk = n_heads // n_kv
+    out = torch.empty((n, n_heads, d), dtype=torch.float32, device=q.device)
+    for t in range(n):
+        pos = int(positions[t])
+        lo = max(0, pos - window + 1) if window else 0
+        keys = torch.arange(lo, pos + 1, device=q.device)
+        pages = block_table[int(token_seq[t])][(keys // page_size).long()].long()
+        offs = (keys % page_size).long()
+        k = k_cache[pages, :, offs, :].to(torch.float32)  # [keys, G, D]
+        v = v_cache[pages, :, :, offs].to(torch.float32)  # [keys, G, D]
+        for h in range(n_heads):
+            g = h // qpk
+            s = (k[:, g, :] @ q[t, h].to(torch.float32)) * scale
+            p = torch.softmax(s, dim=0)
+            out[t, h] = p @ v[:, g, :]
+    return out
+
+
+def attention(qkv, n_heads, n_kv_rows, n_kv, head_dim, k_cache, v_cache, page_size, scale,
+              window, ctx, group, tiles):
+    n = qkv.shape[0]
+    q = qkv.view(n, -1, head_dim)[:, :n_heads]
+    out = attention_paged(
+        q, k_cache, v_cache, ctx.arrays["positions"], ctx.arrays["token_seq"],
+        ctx.arrays[f"block_table_g{group}"], page_size, scale, window,
+    )
+    return out.reshape(n, n_heads * head_dim).to(qkv.dtype)
+
+
+def gated_act(gu, activation):
+    inter = gu.shape[1] // 2
+    g = gu[:, :inter].to(torch.float32)
+    u = gu[:, inter:].to(torch.float32)
+    if activation == "silu":
+        a = g * torch.sigmoid(g)
+    elif activation == "gelu_tanh":
+        a = 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g**3)))
+    else:
+        raise ValueError(activation)
+    return (a * u).to(gu.dtype)
+
+
+def argmax(logits):
+    return torch.argmax(logits, dim=-1).to(torch.int32)
+
+
+class RefOps:
+    """The kernel library's interface over the functions above (CPU or GPU tensors)."""
+
+    def check_attention_sizes(self, n_heads, n_kv, head_dim, page_size):
+        assert n_heads % n_kv == 0 and head_dim % 16 == 0 and page_size % 16 == 0
+
+    def attention_tokens_per_tile(self, n_heads, n_kv):
+        return 16 // min(n_heads // n_kv, 16)
+
+    embed = staticmethod(embed)
+    add_rmsnorm = staticmethod(add_rmsnorm)
+    gather_add_rmsnorm = staticmethod(gather_add_rmsnorm)
+    linear = staticmethod(linear)
+    rope_append = staticmethod(rope_append)
+    attention = staticmethod(attention)
+    gated_act = staticmethod(gated_act)
+    argmax = staticmethod(argmax)
+
+    def sample(self, logits, temperature, top_k, top_p, seeds, draws):
+        from plain_llama import sample_token
+
+        out = []
+        for i in range(logits.shape[0]):
+            k = int(top_k[i])
+            out.append(
+                sample_token(logits[i].cpu(), float(temperature[i]), k if k > 0 else None, float(top_p[i]), int(seeds[i]), int(draws[i]))
+            )
+        return torch.tensor(out, dtype=torch.int32, device=logits.device)

@@ -1,0 +1,345 @@
+"""Each HIP kernel alone against its plain PyTorch counterpart (tests/kernel_refs.py),
+at sizes other than the engine's tiny models: widths and vocabularies that are no
+powers of two, several head sizes and group counts, ragged batches, pages out of order.
+"""
+import math
+import types
+
+import numpy as np
+import pytest
+import torch
+
+import kernel_refs as R
+from yalis_amd.engine.batch import SeqSpan, attention_tiles, build_host_batch, named_arrays
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from yalis_amd.ops.hip import HipOps
+
+    return HipOps(DEV)
+
+
+def rnd(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def close(got, want, atol, rtol=0.0):
+    got = got.float().cpu()
+    want = want.float().cpu()
+    err = (got - want).abs()
+    bound = atol + rtol * want.abs()
+    assert torch.isfinite(got).all(), "kernel produced non-finite values"
+    assert (err <= bound).all(), f"max err {err.max().item():.3e} (bound {bound.min().item():.3e})"
+
+
+# ------------------------------------------------------------------------- embedding
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed(ops, dtype):
+    table = rnd((515, 192), dtype, 0)
+    ids = torch.tensor([0, 514, 3, 3, 77, 200], dtype=torch.int32, device=DEV)
+    got = ops.embed(ids, table)
+    assert got.dtype == torch.float32
+    assert torch.equal(got.cpu(), R.embed(ids.cpu(), table.cpu()))
+
+
+# ------------------------------------------------------------------------------ norm
+@pytest.mark.parametrize("width,rows", [(192, 7), (4096, 33), (1000, 3), (6144, 2)])
+@pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
+def test_add_rmsnorm(ops, width, rows, act, wdtype):
+    res = rnd((rows, width), torch.float32, 1)
+    res[0] *= 1e-4  # a near-zero row: eps matters
+    delta = rnd((rows, width), act, 2)
+    w = (1 + 0.1 * rnd((width,), torch.float32, 3)).to(wdtype)
+    for eps, unit in ((1e-5, False), (1e-6, True)):
+        for d in (delta, None):
+            r_gpu = res.clone()
+            r_ref = res.clone().cpu()
+            got = ops.add_rmsnorm(r_gpu, d, w, eps, unit, act)
+            want = R.add_rmsnorm(r_ref, None if d is None else d.cpu(), w.cpu(), eps, unit, torch.float32)
+            close(r_gpu, r_ref, 1e-6)
+            if act == torch.float32:
+                close(got, want, 2e-5, 2e-5)
+            else:
+                close(got, want, 1e-3, 2**-8)
+
+
+def test_gather_add_rmsnorm(ops):
+    res = rnd((20, 320), torch.float32, 1)
+    delta = rnd((20, 320), torch.bfloat16, 2)
+    w = rnd((320,), torch.bfloat16, 3)
+    rows = torch.tensor([19, 0, 7, 7], dtype=torch.int32, device=DEV)
+    keep = res.clone()
+    got = ops.gather_add_rmsnorm(res, delta, rows, w, 1e-5, False, torch.float32)
+    want = R.gather_add_rmsnorm(keep.cpu(), delta.cpu(), rows.cpu(), w.cpu(), 1e-5, False, torch.float32)
+    assert torch.equal(res, keep), "the gathered form must not change the residual"
+    close(got, want, 2e-5, 2e-5)
+
+
+# ------------------------------------------------------------------------------ gemm
+@pytest.mark.parametrize("m,n,k", [(5, 37, 19), (70, 130, 100), (1, 515, 192), (64, 64, 64), (129, 65, 33)])
+@pytest.mark.parametrize("xd,wd,od", [
+    (torch.float32, torch.float32, torch.float32),
+    (torch.bfloat16, torch.float32, torch.bfloat16),
+    (torch.bfloat16, torch.bfloat16, torch.float32),
+    (torch.float32, torch.bfloat16, torch.float32),
+])
+def test_gemm_fma(ops, m, n, k, xd, wd, od):
+    x = rnd((m, k), xd, 4)
+    w = rnd((n, k), wd, 5)
+    got = ops.gemm_fma(x, w, od)
+    want = x.double().cpu() @ w.double().cpu().T
+    if od == torch.float32:
+        close(got, want, 1e-5 * math.sqrt(k), 1e-5)
+    else:
+        close(got, want, 1e-3, 2**-8)
+
+
+def test_gemm_fma_is_true_float32(ops):
+    """Inputs that a reduced-precision matrix mode would truncate: 1 + 2^-20."""
+    k = 64
+    x = torch.full((4, k), 1.0 + 2.0**-20, device=DEV)
+    w = torch.full((8, k), 1.0 + 2.0**-20, device=DEV)
+    got = ops.gemm_fma(x, w, torch.float32)
+    want = k * (1.0 + 2.0**-20) ** 2
+    assert abs(got[0, 0].item() - want) < 1e-5
+
+
+@pytest.mark.parametrize("m,n,k", [
+    (1, 96, 64), (3, 515, 192), (16, 100, 200), (17, 64, 4096), (33, 130, 72), (64, 520, 328),
+    (8, 4096, 4096), (100, 515, 192), (1, 16, 8),
+])
+@pytest.mark.parametrize("od", [torch.float32, torch.bfloat16])
+def test_gemm_mfma_skinny(ops, m, n, k, od):
+    x = rnd((m, k), torch.bfloat16, 6)
+    w = rnd((n, k), torch.bfloat16, 7)
+    got = ops.gemm_mfma_skinny(x, w, od)
+    want = x.double().cpu() @ w.double().cpu().T
+    if od == torch.float32:
+        close(got, want, 2e-5 * math.sqrt(k), 1e-5)
+    else:
+        close(got, want, 1e-2, 2**-8)
+
+
+def test_gemm_mfma_operand_order(ops):
+    """One-hot operands name the element each lane must hold: y[m, n] = x[m, kx] * w[n, kx]
+    for a single k picks out any mismatch between the two operands' k order."""
+    m, n, k = 16, 16, 64
+    for kk in (0, 7, 8, 31, 32, 63):
+        x = torch.zeros((m, k), dtype=torch.bfloat16, device=DEV)
+        w = torch.zeros((n, k), dtype=torch.bfloat16, device=DEV)
+        x[:, kk] = torch.arange(1, m + 1, dtype=torch.bfloat16)
+        w[:, kk] = torch.arange(1, n + 1, dtype=torch.bfloat16) * 0.5
+        got = ops.gemm_mfma_skinny(x, w, torch.float32).cpu()
+        want = torch.outer(torch.arange(1, m + 1).float(), torch.arange(1, n + 1).float() * 0.5)
+        assert torch.equal(got, want), f"k={kk}"
+
+
+def test_linear_dispatch(ops):
+    x = rnd((200, 192), torch.bfloat16, 8)
+    w = rnd((515, 192), torch.bfloat16, 9)
+    want = x.double().cpu() @ w.double().cpu().T
+    close(ops.linear(x, w, torch.bfloat16), want, 1e-2, 2**-7)
+    close(ops.linear(x, w, torch.float32), want, 1e-4, 1e-5)
+    close(ops.linear(x[:5], w, torch.bfloat16), want[:5], 1e-2, 2**-7)
+    wf = w.float()
+    close(ops.linear(x, wf, torch.bfloat16), want, 1e-2, 2**-7)
+
+
+# ---------------------------------------------------------------- rotary + cache append
+def _tables(rotary_dim, positions, theta=10000.0):
+    inv = 1.0 / (theta ** (torch.arange(0, rotary_dim, 2).float() / rotary_dim))
+    ang = torch.outer(torch.arange(positions).float(), inv)
+    return torch.cos(ang).to(DEV), torch.sin(ang).to(DEV)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("h,g,d,rd,inter", [(4, 2, 16, 16, False), (6, 3, 64, 64, False), (8, 1, 128, 64, True), (3, 3, 48, 32, False), (5, 0, 32, 32, False)])
+def test_rope_append(ops, dtype, h, g, d, rd, inter):
+    n, page, n_pages = 37, 16, 9
+    qkv = rnd((n, (h + 2 * g) * d), dtype, 10)
+    cos, sin = _tables(rd, 200)
+    positions = torch.randint(0, 200, (n,), generator=torch.Generator().manual_seed(1), dtype=torch.int32).to(DEV)
+    slots = torch.randperm(page * n_pages, generator=torch.Generator().manual_seed(2))[:n].to(torch.int32).to(DEV)
+    kc = torch.zeros((n_pages, max(g, 1), page, d), dtype=dtype, device=DEV)
+    vc = torch.zeros((n_pages, max(g, 1), d, page), dtype=dtype, device=DEV)
+    kc_r, vc_r, qkv_r = kc.cpu().clone(), vc.cpu().clone(), qkv.cpu().clone()
+    if g == 0:
+        ops.rope_append(qkv, h, 0, d, positions, cos, sin, rd, inter, None, None, None, page)
+        R.rope_append(qkv_r, h, 0, d, positions.cpu(), cos.cpu(), sin.cpu(), rd, inter, None, None, None, page)
+    else:
+        ops.rope_append(qkv, h, g, d, positions, cos, sin, rd, inter, kc, vc, slots, page)
+        R.rope_append(qkv_r, h, g, d, positions.cpu(), cos.cpu(), sin.cpu(), rd, inter, kc_r, vc_r, slots.cpu(), page)
+    tol = 1e-6 if dtype == torch.float32 else 2**-7
+    close(qkv.view(n, -1, d)[:, :h], qkv_r.view(n, -1, d)[:, :h], tol, tol)
+    if g:
+        close(kc, kc_r, tol, tol)
+        assert torch.equal(vc.cpu(), vc_r), "values are copied, not changed"
+
+
+# ------------------------------------------------------------------------- attention
+def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True, n_pages=64):
+    """spans: list of (cached tokens before the step, new tokens).  Builds pages in a
+    shuffled order, fills cache for the earlier tokens, runs rope-free attention."""
+    gen = torch.Generator().manual_seed(seed)
+    order = torch.randperm(n_pages, generator=gen).tolist()
+    kc = torch.zeros((n_pages, g, page, d), dtype=dtype)
+    vc = torch.zeros((n_pages, g, d, page), dtype=dtype)
+    if poison:
+        kc.fill_(float("nan"))
+        vc.fill_(float("nan"))
+    seqs = []
+    used = 0
+    for cached, new in spans:
+        total = cached + new
+        n_p = -(-total // page)
+        table = np.array(order[used : used + n_p], dtype=np.int32)
+        used += n_p
+        assert used <= n_pages
+        k = torch.randn((total, g, d), generator=gen).to(dtype)
+        v = torch.randn((total, g, d), generator=gen).to(dtype)
+        for pos in range(total):
+            kc[table[pos // page], :, pos % page, :] = k[pos]
+            vc[table[pos // page], :, :, pos % page] = v[pos]
+        seqs.append(SeqSpan(tokens=[0] * new, first_position=cached, block_tables=[table], state_slot=0))
+    hb = build_host_batch(seqs, 1, page)
+    tpt = ops.attention_tokens_per_tile(h, g)
+    arrays = named_arrays(hb, {f"tiles": lambda b: attention_tiles(b, tpt)})
+    ctx = types.SimpleNamespace(
+        arrays={k: torch.from_numpy(np.ascontiguousarray(v)).to(DEV) for k, v in arrays.items()},
+        max_ctx=hb.max_ctx,
+    )
+    ctx_cpu = types.SimpleNamespace(arrays={k: torch.from_numpy(np.ascontiguousarray(v)) for k, v in arrays.items()})
+    n = hb.n_tokens
+    q = (torch.randn((n, h * d), generator=gen) * 1.5).to(dtype)
+    scale = 1.0 / math.sqrt(d)
+    got = ops.attention(q.to(DEV), h, 0, g, d, kc.to(DEV), vc.to(DEV), page, scale, window, ctx, 0, ctx.arrays["tiles"])
+    want = R.attention(q.float(), h, 0, g, d, kc.float(), vc.float(), page, scale, window, ctx_cpu, 0, None)
+    return got, want
+
+
+SPANS = [(0, 5), (17, 1), (0, 70), (63, 2), (100, 1), (31, 34), (0, 1)]
+
+
+@pytest.mark.parametrize("h,g,d,page", [(4, 2, 16, 16), (4, 1, 32, 32), (6, 3, 48, 16), (5, 5, 80, 64), (2, 1, 256, 16)])
+@pytest.mark.parametrize("window", [0, 24])
+def test_attention_generic_f32(ops, h, g, d, page, window):
+    got, want = _attention_case(ops, torch.float32, h, g, d, page, SPANS, window, seed=3)
+    close(got, want, 2e-5, 1e-5)
+
+
+@pytest.mark.parametrize("h,g,d,page", [(4, 2, 16, 16), (6, 3, 48, 32)])
+def test_attention_generic_bf16(ops, h, g, d, page):
+    got, want = _attention_case(ops, torch.bfloat16, h, g, d, page, SPANS, 0, seed=4)
+    close(got, want, 1e-2, 2**-7)
+
+
+@pytest.mark.parametrize("h,g,d,page", [
+    (8, 2, 128, 64), (6, 3, 64, 16), (4, 4, 64, 32), (32, 1, 128, 16), (5, 1, 64, 48), (24, 8, 128, 64), (40, 2, 64, 16),
+])
+@pytest.mark.parametrize("window", [0, 40])
+def test_attention_mfma(ops, h, g, d, page, window):
+    got, want = _attention_case(ops, torch.bfloat16, h, g, d, page, SPANS, window, seed=5)
+    close(got, want, 2e-2, 2**-6)
+
+
+def test_attention_mfma_long_context_splits(ops):
+    """Few waves and many keys: the launch splits the keys and merges the parts."""
+    spans = [(1500, 1), (900, 3), (0, 2)]
+    got, want = _attention_case(ops, torch.bfloat16, 8, 2, 128, 64, spans, 0, seed=6, n_pages=48)
+    close(got, want, 2e-2, 2**-6)
+    got, want = _attention_case(ops, torch.bfloat16, 8, 2, 128, 64, spans, 700, seed=6, n_pages=48)
+    close(got, want, 2e-2, 2**-6)
+
+
+def test_attention_far_key_stands_out(ops):
+    """One far key gets a large score: if a kernel skipped or misplaced it, the output
+    would be the average of the others instead of (almost exactly) that key's value."""
+    h, g, d, page = 8, 2, 128, 64
+    n_ctx = 777
+    for dtype in (torch.bfloat16, torch.float32):
+        gen = torch.Generator().manual_seed(11)
+        kc = torch.zeros((16, g, page, d), dtype=dtype)
+        vc = torch.zeros((16, g, d, page), dtype=dtype)
+        table = np.arange(15, 15 - 13, -1).astype(np.int32)  # pages in reverse
+        k = torch.randn((n_ctx, g, d), generator=gen) * 0.1
+        v = torch.randn((n_ctx, g, d), generator=gen)
+        far = 5  # an early key, hundreds of tokens back
+        q = torch.randn((1, h * d), generator=gen) * 0.1
+        k[far] = 0
+        k[far, 0, :] = q.view(h, d)[1] * 200.0  # head 1 (group 0) loves key `far`
+        for pos in range(n_ctx):
+            kc[table[pos // page], :, pos % page, :] = k[pos].to(dtype)
+            vc[table[pos // page], :, :, pos % page] = v[pos].to(dtype)
+        span = SeqSpan(tokens=[0], first_position=n_ctx - 1, block_tables=[table], state_slot=0)
+        hb = build_host_batch([span], 1, page)
+        tpt = ops.attention_tokens_per_tile(h, g)
+        arrays = named_arrays(hb, {"tiles": lambda b: attention_tiles(b, tpt)})
+        ctx = types.SimpleNamespace(
+            arrays={kk: torch.from_numpy(np.ascontiguousarray(vv)).to(DEV) for kk, vv in arrays.items()},
+            max_ctx=hb.max_ctx,
+        )
+        got = ops.attention(q.to(dtype).to(DEV), h, 0, g, d, kc.to(DEV), vc.to(DEV), page, 1.0 / math.sqrt(d), 0, ctx, 0, ctx.arrays["tiles"])
+        head1 = got.view(h, d)[1].float().cpu()
+        close(head1, v[far, 0].to(dtype).float(), 2e-2, 2**-6)
+
+
+# ------------------------------------------------------------------------ activation
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("act", ["silu", "gelu_tanh"])
+def test_gated_act(ops, dtype, act):
+    gu = rnd((9, 2 * 328), dtype, 12, scale=3.0)
+    got = ops.gated_act(gu, act)
+    want = R.gated_act(gu.float().cpu(), act)
+    if dtype == torch.float32:
+        close(got, want, 1e-6, 1e-5)
+    else:
+        close(got, want, 1e-3, 2**-8)
+
+
+# -------------------------------------------------------------------------- sampling
+def test_argmax_lowest_index_on_ties(ops):
+    logits = rnd((5, 1000), torch.float32, 13)
+    logits[0, 17] = 50.0
+    logits[0, 900] = 50.0
+    logits[1, 999] = 60.0
+    got = ops.argmax(logits).cpu()
+    want = torch.argmax(logits.cpu(), dim=-1)
+    assert got[0].item() == 17 and got[1].item() == 999
+    assert torch.equal(got[2:].long(), want[2:])
+
+
+def _sample(ops, logits, temperature, top_k, top_p, seed, draw):
+    rows = logits.shape[0]
+    f = lambda v, dt: torch.full((rows,), v, dtype=dt, device=DEV)
+    return ops.sample(
+        logits, f(temperature, torch.float32), f(top_k, torch.int32), f(top_p, torch.float32),
+        f(seed, torch.int32), torch.arange(draw, draw + rows, dtype=torch.int32, device=DEV),
+    ).cpu()
+
+
+def test_sample_matches_plain(ops):
+    import plain_llama as P
+
+    logits = rnd((1, 515), torch.float32, 14, scale=2.0)
+    for temperature, top_k, top_p in [(0.7, 0, 1.0), (1.0, 5, 1.0), (1.3, 0, 0.8), (0.9, 50, 0.5), (0.0, 0, 1.0), (1.0, 1, 1.0), (1.0, 0, 0.0)]:
+        for draw in range(20):
+            got = _sample(ops, logits, temperature, top_k, top_p, 99, draw)[0].item()
+            want = P.sample_token(logits[0].cpu(), temperature, top_k or None, top_p, 99, draw)
+            assert got == want, (temperature, top_k, top_p, draw)
+
+
+def test_sample_frequencies(ops):
+    """Draws follow softmax(logits / T): chi-square over many draws."""
+    vocab, draws, temperature = 12, 20000, 0.8
+    logits = torch.linspace(-2, 2, vocab, device=DEV).repeat(draws, 1).contiguous()
+    got = _sample(ops, logits, temperature, 0, 1.0, 5, 0)
+    counts = torch.bincount(got.long(), minlength=vocab).double()
+    p = torch.softmax(logits[0].cpu().double() / temperature, dim=0)
+    chi2 = ((counts - draws * p) ** 2 / (draws * p)).sum().item()
+    assert chi2 < 40.0, chi2  # 11 degrees of freedom: 40 is beyond the 99.99th percentile

@@ -1,0 +1,404 @@
+// Causal attention with grouped key/value heads over the paged cache, for any span:
+// the queries of a step's tokens (prompt portions and single decoded tokens alike)
+// against the keys and values that the block tables name.
+//
+// Arithmetic (reference: yalis/attention/backend_impl/sdpa_and_flex.py:59-90, 300-312):
+// score[h, p, j] = q[h, p] . k[h / (H/G), j] * scale; key j is visible to the query at
+// position p iff j <= p (and p - j < window when a window is set); softmax over the
+// visible keys in float32; output = P . V.
+//
+// Page layout: keys [page][kv_head][page_size][head_dim], values transposed
+// [page][kv_head][head_dim][page_size].  Pages are never cleared, so nothing beyond a
+// request's token count is ever read as a number: invisible scores are replaced, and
+// values of tokens that do not exist yet are zeroed before they meet a probability.
+//
+// Two kernels:
+//  * attn_generic: one wave per (token, head), float32 arithmetic throughout, any
+//    head_dim that is a multiple of 16 up to 256, float32 or bfloat16 storage.  This is
+//    the true-32-bit path and the fallback for head sizes the matrix-core kernel lacks.
+//  * attn_mfma: bfloat16 on the gfx950 matrix cores.  One wave owns 16 "columns": a few
+//    consecutive tokens of one request times the query heads that share one key/value
+//    head.  It computes S^T = K . Q^T and O^T = V^T . P^T, so that keys and transposed
+//    values stream from memory straight into the matrix-core A operand and each lane
+//    keeps one column's softmax state.  The visible keys can be split over several
+//    waves; a second kernel merges the partial results in float32.
+#include <algorithm>
+
+#include "common.h"
+
+// ---------------------------------------------------------------------------- generic
+template <typename T>
+__global__ __launch_bounds__(64) void attn_generic_kernel(
+    const T* __restrict__ q, int q_stride, T* __restrict__ out, const T* __restrict__ k_cache,
+    const T* __restrict__ v_cache, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ token_seq, const int32_t* __restrict__ block_table, int table_width,
+    int page_size, int head_dim, int n_heads, int n_kv, float scale, int window) {
+  __shared__ float qs[256];
+  __shared__ float ps[64];
+  __shared__ int pbase[64];  // (page * n_kv + kv_head) per key of the tile
+  __shared__ int poff[64];
+  const int n = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int qpk = n_heads / n_kv, g = h / qpk;
+  const int pos = positions[n], seq = token_seq[n];
+  const int hi = pos + 1;
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const T* qrow = q + static_cast<size_t>(n) * q_stride + static_cast<size_t>(h) * head_dim;
+  for (int d = lane; d < head_dim; d += 64) qs[d] = to_f32<T>(qrow[d]);
+  __syncthreads();
+  const int32_t* bt = block_table + static_cast<size_t>(seq) * table_width;
+  float m = -INFINITY, l = 0.f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int t0 = lo; t0 < hi; t0 += 64) {
+    const int key = t0 + lane;
+    const bool valid = key < hi;
+    float s = -INFINITY;
+    int base = 0, off = 0;
+    if (valid) {
+      const int page = bt[key / page_size];
+      off = key % page_size;
+      base = page * n_kv + g;
+      const T* kp = k_cache + (static_cast<size_t>(base) * page_size + off) * head_dim;
+      float dot = 0.f;
+      for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], to_f32<T>(kp[d]), dot);
+      s = dot * scale;
+    }
+    const float m_new = fmaxf(m, wave_max(s));  // finite: the tile holds at least one key
+    const float p = valid ? expf(s - m_new) : 0.f;
+    const float alpha = expf(m - m_new);  // 0 on the first tile
+    l = l * alpha + wave_sum(p);
+    m = m_new;
+    __syncthreads();  // the previous tile's ps/pbase are no longer read
+    ps[lane] = p;
+    pbase[lane] = base;
+    poff[lane] = off;
+    __syncthreads();
+    const int count = min(64, hi - t0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = lane + 64 * i;
+      if (d < head_dim) {
+        float a = acc[i] * alpha;
+        for (int j = 0; j < count; ++j) {
+          const T* vp = v_cache + (static_cast<size_t>(pbase[j]) * head_dim + d) * page_size + poff[j];
+          a = fmaf(ps[j], to_f32<T>(*vp), a);
+        }
+        acc[i] = a;
+      }
+    }
+  }
+  T* orow = out + (static_cast<size_t>(n) * n_heads + h) * head_dim;
+  const float inv = 1.f / l;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    if (d < head_dim) orow[d] = from_f32<T>(acc[i] * inv);
+  }
+}
+
+extern "C" int yk_attn_generic(const void* q, int q_stride, void* out, const void* k_cache,
+                               const void* v_cache, int dtype, const int32_t* positions,
+                               const int32_t* token_seq, const int32_t* block_table,
+                               int table_width, int n_tokens, int page_size, int head_dim,
+                               int n_heads, int n_kv, float scale, int window,
+                               hipStream_t stream) {
+  YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv > 0, "attention: bad sizes");
+  YK_REQUIRE(n_heads % n_kv == 0, "attention: the head count must be a multiple of the kv head count");
+  YK_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 256,
+             "attention: head_dim must be a multiple of 16 and at most 256");
+  YK_REQUIRE(page_size > 0 && table_width > 0, "attention: bad page table");
+  YK_REQUIRE(n_heads <= 65535, "attention: too many heads for one launch");
+  YK_REQUIRE(window >= 0, "attention: window must not be negative");
+  if (n_tokens == 0) return 0;
+  dim3 grid(n_tokens, n_heads), block(64);
+  if (dtype == YK_F32)
+    attn_generic_kernel<float><<<grid, block, 0, stream>>>(
+        static_cast<const float*>(q), q_stride, static_cast<float*>(out),
+        static_cast<const float*>(k_cache), static_cast<const float*>(v_cache), positions,
+        token_seq, block_table, table_width, page_size, head_dim, n_heads, n_kv, scale, window);
+  else if (dtype == YK_BF16)
+    attn_generic_kernel<bf16_t><<<grid, block, 0, stream>>>(
+        static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out),
+        static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), positions,
+        token_seq, block_table, table_width, page_size, head_dim, n_heads, n_kv, scale, window);
+  else
+    return yk_fail("attention: unsupported dtype");
+  return yk_check_launch("attn_generic");
+}
+
+// ------------------------------------------------------------------------ matrix cores
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+union AFrag8 {
+  u32x4_t u;
+  bf16x8_t v;
+  bf16_t h[8];
+};
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return static_cast<uint32_t>(f32_to_bf16(lo)) | (static_cast<uint32_t>(f32_to_bf16(hi)) << 16);
+}
+
+// Layout of a tile row handed over by the host: (request, first token index in the
+// batch, token count, position of the first token).
+//
+// Columns of a wave: column c in 0..15 is token c / hpt of the tile and query head
+// h_base + c % hpt, hpt = min(H/G, 16) heads per tile; a kv head with more than 16
+// query heads takes several "chunks" of 16.
+template <int D>
+__global__ __launch_bounds__(64) void attn_mfma_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
+    const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int32_t* __restrict__ tiles, const int32_t* __restrict__ block_table, int table_width,
+    int page_size, int n_heads, int n_kv, int hpt, int chunks, float scale_log2, int window,
+    int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml) {
+  constexpr int KS = D / 32;  // matrix-core steps over the head dimension
+  constexpr int DT = D / 16;  // output tiles over the head dimension
+  const int lane = threadIdx.x, r = lane % 16, gq = lane / 16;
+  const int t = blockIdx.x;
+  const int seq = tiles[4 * t], tok0 = tiles[4 * t + 1], ntok = tiles[4 * t + 2], pos0 = tiles[4 * t + 3];
+  const int g = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+  const int qpk = n_heads / n_kv;
+  const int h_base = g * qpk + chunk * hpt;
+  const int heads_here = min(hpt, qpk - chunk * hpt);
+  const int tt = r / hpt, hh = r % hpt;
+  const bool col_ok = tt < ntok && hh < heads_here;
+  const int pos_c = pos0 + tt;
+  const int lo_c = window > 0 ? max(0, pos_c - window + 1) : 0;
+  const int hi = pos0 + ntok;
+  const int lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int kb_lo = lo / 64, kb_hi = (hi + 63) / 64;
+  const int per_split = (kb_hi - kb_lo + n_splits - 1) / n_splits;
+  const int my_lo = kb_lo + blockIdx.z * per_split;
+  const int my_hi = min(kb_hi, my_lo + per_split);
+  const int32_t* bt = block_table + static_cast<size_t>(seq) * table_width;
+
+  const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+  AFrag8 qf[KS];
+  {
+    const bf16_t* qp = q + static_cast<size_t>(tok0 + (col_ok ? tt : 0)) * q_stride +
+                       static_cast<size_t>(h_base + (col_ok ? hh : 0)) * D + 8 * gq;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      qf[ks].u = col_ok ? *reinterpret_cast<const u32x4_t*>(qp + 32 * ks) : zero4;
+  }
+  float m = -INFINITY, l = 0.f;
+  f32x4_t acc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  for (int kb = my_lo; kb < my_hi; ++kb) {
+    f32x4_t s[4];
+    int page_of[4];
+    int koff_of[4];
+    bool live[4];
+#pragma unroll
+    for (int sub = 0; sub < 4; ++sub) {
+      const int key0 = kb * 64 + 16 * sub;
+      s[sub] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      live[sub] = key0 < hi && key0 + 16 > lo;  // same for every lane
+      page_of[sub] = 0;
+      koff_of[sub] = key0 % page_size;
+      if (live[sub]) {
+        page_of[sub] = bt[key0 / page_size];
+        const bf16_t* kp = k_cache +
+                           ((static_cast<size_t>(page_of[sub]) * n_kv + g) * page_size + koff_of[sub] + r) * D +
+                           8 * gq;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          AFrag8 a;
+          a.u = *reinterpret_cast<const u32x4_t*>(kp + 32 * ks);
+          s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[ks].v, s[sub], 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = key0 + 4 * gq + i;
+        const bool ok = live[sub] && col_ok && key <= pos_c && key >= lo_c;
+        s[sub][i] = ok ? s[sub][i] * scale_log2 : -INFINITY;
+      }
+    }
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int sub = 0; sub < 4; ++sub)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, s[sub][i]);
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m, tmax);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = exp2f(m - m_safe);
+    float psum = 0.f;
+#pragma unroll
+    for (int sub = 0; sub < 4; ++sub)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        s[sub][i] = exp2f(s[sub][i] - m_safe);
+        psum += s[sub][i];
+      }
+    l = l * alpha + psum;
+    m = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[dt] *= alpha;
+
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int sa = 2 * u, sb = 2 * u + 1;
+      if (!live[sa] && !live[sb]) continue;
+      AFrag8 b;
+      b.u[0] = pack_bf16x2(s[sa][0], s[sa][1]);
+      b.u[1] = pack_bf16x2(s[sa][2], s[sa][3]);
+      b.u[2] = pack_bf16x2(s[sb][0], s[sb][1]);
+      b.u[3] = pack_bf16x2(s[sb][2], s[sb][3]);
+      const int key_a = kb * 64 + 16 * sa + 4 * gq;  // first of this lane's four keys in tile a
+      const int key_b = key_a + 16;
+      const bool edge = kb * 64 + 16 * sb + 16 > hi;  // some keys of the pair do not exist yet
+      const bf16_t* va = v_cache + (static_cast<size_t>(page_of[sa]) * n_kv + g) * D * page_size +
+                         koff_of[sa] + 4 * gq;
+      const bf16_t* vb = v_cache + (static_cast<size_t>(page_of[sb]) * n_kv + g) * D * page_size +
+                         koff_of[sb] + 4 * gq;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const size_t row = static_cast<size_t>(16 * dt + r) * page_size;
+        AFrag8 a;
+        u32x2_t xa = {0u, 0u}, xb = {0u, 0u};
+        if (live[sa]) xa = *reinterpret_cast<const u32x2_t*>(va + row);
+        if (live[sb]) xb = *reinterpret_cast<const u32x2_t*>(vb + row);
+        a.u[0] = xa[0];
+        a.u[1] = xa[1];
+        a.u[2] = xb[0];
+        a.u[3] = xb[1];
+        if (edge) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            if (key_a + i >= hi) a.h[i] = 0;
+            if (key_b + i >= hi) a.h[4 + i] = 0;
+          }
+        }
+        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[dt], 0, 0, 0);
+      }
+    }
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+
+  if (n_splits == 1) {
+    if (col_ok) {
+      const float inv = 1.f / l;
+      bf16_t* op = out + (static_cast<size_t>(tok0 + tt) * n_heads + h_base + hh) * D + 4 * gq;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        u32x2_t w;
+        w[0] = pack_bf16x2(acc[dt][0] * inv, acc[dt][1] * inv);
+        w[1] = pack_bf16x2(acc[dt][2] * inv, acc[dt][3] * inv);
+        *reinterpret_cast<u32x2_t*>(op + 16 * dt) = w;
+      }
+    }
+  } else {
+    // partial result of this split: unnormalised output, running maximum and sum
+    const size_t widx = (static_cast<size_t>(t) * gridDim.y + blockIdx.y) * n_splits + blockIdx.z;
+    float* wo = ws_o + (widx * 16 + r) * D + 4 * gq;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4_t*>(wo + 16 * dt) = acc[dt];
+    if (gq == 0) {
+      ws_ml[(widx * 16 + r) * 2] = m;
+      ws_ml[(widx * 16 + r) * 2 + 1] = l;
+    }
+  }
+}
+
+// Merge the splits of every column: weights exp2(m_s - max m), in the order of s.
+template <int D>
+__global__ __launch_bounds__(256) void attn_combine_kernel(
+    bf16_t* __restrict__ out, const int32_t* __restrict__ tiles, int n_heads, int n_kv, int hpt,
+    int chunks, int n_splits, const float* __restrict__ ws_o, const float* __restrict__ ws_ml) {
+  const int t = blockIdx.x;
+  const int tok0 = tiles[4 * t + 1], ntok = tiles[4 * t + 2];
+  const int g = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+  const int qpk = n_heads / n_kv;
+  const int h_base = g * qpk + chunk * hpt;
+  const int heads_here = min(hpt, qpk - chunk * hpt);
+  const size_t w0 = (static_cast<size_t>(t) * gridDim.y + blockIdx.y) * n_splits;
+  for (int e = threadIdx.x; e < 16 * D; e += blockDim.x) {
+    const int c = e / D, d = e % D;
+    const int tt = c / hpt, hh = c % hpt;
+    if (tt >= ntok || hh >= heads_here) continue;
+    float m_max = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) m_max = fmaxf(m_max, ws_ml[((w0 + s) * 16 + c) * 2]);
+    float num = 0.f, den = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+      const float w = exp2f(ws_ml[((w0 + s) * 16 + c) * 2] - m_max);
+      num += w * ws_o[((w0 + s) * 16 + c) * D + d];
+      den += w * ws_ml[((w0 + s) * 16 + c) * 2 + 1];
+    }
+    out[(static_cast<size_t>(tok0 + tt) * n_heads + h_base + hh) * D + d] = f32_to_bf16(num / den);
+  }
+}
+
+extern "C" int yk_attn_mfma_supported(int head_dim) { return head_dim == 64 || head_dim == 128; }
+
+// Heads of one kv head that share a wave, and tokens per tile, for a head layout.
+extern "C" int yk_attn_heads_per_tile(int n_heads, int n_kv) {
+  const int qpk = n_heads / n_kv;
+  return qpk < 16 ? qpk : 16;
+}
+extern "C" int yk_attn_tokens_per_tile(int n_heads, int n_kv) {
+  return 16 / yk_attn_heads_per_tile(n_heads, n_kv);
+}
+
+// Floats of workspace for a launch with n_splits > 1: outputs, then (max, sum) pairs.
+extern "C" size_t yk_attn_mfma_workspace(int n_tiles, int n_heads, int n_kv, int head_dim,
+                                         int n_splits) {
+  if (n_splits <= 1) return 0;
+  const int hpt = yk_attn_heads_per_tile(n_heads, n_kv);
+  const int chunks = (n_heads / n_kv + hpt - 1) / hpt;
+  const size_t w = static_cast<size_t>(n_tiles) * n_kv * chunks * n_splits * 16;
+  return w * head_dim + w * 2;
+}
+
+extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* k_cache,
+                            const void* v_cache, const int32_t* tiles, int n_tiles,
+                            const int32_t* block_table, int table_width, int page_size,
+                            int head_dim, int n_heads, int n_kv, float scale, int window,
+                            int n_splits, float* workspace, size_t workspace_floats,
+                            hipStream_t stream) {
+  YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_mfma: bad head counts");
+  YK_REQUIRE(yk_attn_mfma_supported(head_dim), "attn_mfma: head_dim must be 64 or 128");
+  YK_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_mfma: page_size must be a multiple of 16");
+  YK_REQUIRE(q_stride % 8 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0,
+             "attn_mfma: query rows must be 16-byte aligned");
+  YK_REQUIRE(reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0,
+             "attn_mfma: cache must be 16-byte aligned");
+  YK_REQUIRE(n_splits >= 1 && n_splits <= 65535, "attn_mfma: bad split count");
+  YK_REQUIRE(window >= 0 && table_width > 0, "attn_mfma: bad window or table");
+  if (n_tiles == 0) return 0;
+  const int hpt = yk_attn_heads_per_tile(n_heads, n_kv);
+  const int chunks = (n_heads / n_kv + hpt - 1) / hpt;
+  YK_REQUIRE(n_kv * chunks <= 65535, "attn_mfma: too many heads for one launch");
+  const size_t need = yk_attn_mfma_workspace(n_tiles, n_heads, n_kv, head_dim, n_splits);
+  YK_REQUIRE(workspace_floats >= need, "attn_mfma: workspace too small");
+  float* ws_o = workspace;
+  float* ws_ml = workspace ? workspace + (need / (head_dim + 2)) * head_dim : nullptr;
+  const float scale_log2 = scale * 1.4426950408889634f;
+  dim3 grid(n_tiles, n_kv * chunks, n_splits), block(64);
+#define YK_LAUNCH(DD)                                                                              \
+  attn_mfma_kernel<DD><<<grid, block, 0, stream>>>(                                                \
+      static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out),                          \
+      static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), tiles, block_table, \
+      table_width, page_size, n_heads, n_kv, hpt, chunks, scale_log2, window, n_splits, ws_o, ws_ml); \
+  if (yk_check_launch("attn_mfma")) return -1;                                                     \
+  if (n_splits > 1) {                                                                              \
+    attn_combine_kernel<DD><<<dim3(n_tiles, n_kv * chunks), 256, 0, stream>>>(                     \
+        static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml);      \
+    if (yk_check_launch("attn_combine")) return -1;                                                \
+  }
+  if (head_dim == 64) {
+    YK_LAUNCH(64)
+  } else {
+    YK_LAUNCH(128)
+  }
+#undef YK_LAUNCH
+  return 0;
+}

@@ -1,0 +1,109 @@
+// Shared helpers of the HIP kernels: bfloat16 storage, wave and block reductions,
+// error reporting of the C interface.
+//
+// Conventions of the library: every entry point is extern "C", takes raw device
+// pointers and sizes plus the stream to launch on, checks its arguments on the host
+// (a size a kernel cannot take is refused with a message, never computed wrongly),
+// returns 0 on success and a negative number on failure; yk_last_error() returns the
+// message.  dtype codes: 0 = float32, 1 = bfloat16.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+#define YK_F32 0
+#define YK_BF16 1
+
+typedef uint16_t bf16_t;  // bfloat16 storage
+
+std::string& yk_error_slot();
+int yk_fail(const std::string& msg);
+int yk_check_launch(const char* what);
+
+#define YK_REQUIRE(cond, msg)        \
+  do {                               \
+    if (!(cond)) return yk_fail(msg); \
+  } while (0)
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t x) {
+  return __uint_as_float(static_cast<uint32_t>(x) << 16);
+}
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<bf16_t>((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return static_cast<bf16_t>(u >> 16);
+}
+
+template <typename T>
+__device__ __forceinline__ float to_f32(T x);
+template <>
+__device__ __forceinline__ float to_f32<float>(float x) {
+  return x;
+}
+template <>
+__device__ __forceinline__ float to_f32<bf16_t>(bf16_t x) {
+  return bf16_to_f32(x);
+}
+
+template <typename T>
+__device__ __forceinline__ T from_f32(float x);
+template <>
+__device__ __forceinline__ float from_f32<float>(float x) {
+  return x;
+}
+template <>
+__device__ __forceinline__ bf16_t from_f32<bf16_t>(float x) {
+  return f32_to_bf16(x);
+}
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result.
+// `scratch` is shared memory for 17 floats.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int nwaves = (blockDim.x + kWave - 1) / kWave;
+  __syncthreads();  // scratch may still be read from an earlier call
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  if (wave == 0) {
+    float t = lane < nwaves ? scratch[lane] : 0.f;
+    t = wave_sum(t);
+    if (lane == 0) scratch[16] = t;
+  }
+  __syncthreads();
+  return scratch[16];
+}
+
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+  v = wave_max(v);
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int nwaves = (blockDim.x + kWave - 1) / kWave;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  if (wave == 0) {
+    float t = lane < nwaves ? scratch[lane] : -INFINITY;
+    t = wave_max(t);
+    if (lane == 0) scratch[16] = t;
+  }
+  __syncthreads();
+  return scratch[16];
+}

@@ -1,0 +1,97 @@
+"""Trace replay: feed given token ids through the model step by step and collect
+logits.  Nothing is sampled.  It drives the same runner (model, step function, cache
+manager, kernels) that generation uses.
+
+A step is ``{"step": k, "entries": [{"id": "a", "tokens": [...], "want": [...]}],
+"end": ["a"]}``: every entry brings a request's next tokens (all entries of a step
+run as one batch), ``want`` lists the places among these tokens whose logits are
+asked for, ``end`` lists requests that are over after the step (their pages and
+slot are given back).  The reference's nearest hook is ``generate(get_logits=True)``
+(yalis/engine.py:431-432, 519-520).
+"""
+from __future__ import annotations
+
+import json
+import os
+import sys
+from typing import Dict, Iterable, List, Optional
+
+import numpy as np
+import torch
+
+from .step import ModelRunner, StepEntry
+
+
+class ReplayError(RuntimeError):
+    pass
+
+
+class Replayer:
+    def __init__(self, runner: ModelRunner):
+        self.runner = runner
+        self.handles: Dict[str, int] = {}
+        self._next = 0
+        self.page_log: List[Dict[str, List[int]]] = []  # per step: id -> pages held (group 0)
+
+    def run_step(self, step: dict) -> Optional[torch.Tensor]:
+        """Runs one step; returns float32 logits [wanted, vocab] or None when
+        nothing was wanted."""
+        entries = []
+        for e in step.get("entries", []):
+            rid = str(e["id"])
+            tokens = [int(t) for t in e["tokens"]]
+            want = [int(w) for w in e.get("want", [])]
+            if not tokens:
+                raise ReplayError(f"step {step.get('step')}: request {rid!r} brings no tokens")
+            if rid not in self.handles:
+                handle = self._next
+                self._next += 1
+                if not self.runner.admit(handle):
+                    raise ReplayError(
+                        f"step {step.get('step')}: no state slot left for request {rid!r} "
+                        f"({self.runner.config.max_num_seqs} requests may be live)"
+                    )
+                self.handles[rid] = handle
+            handle = self.handles[rid]
+            if not self.runner.reserve(handle, len(tokens)):
+                raise ReplayError(
+                    f"step {step.get('step')}: the cache pool has no pages left for {len(tokens)} more tokens of request {rid!r} "
+                    f"(free pages per group: {self.runner.free_pages()})"
+                )
+            entries.append(StepEntry(handle, tokens, want))
+        logits = None
+        if entries:
+            logits = self.runner.step(entries)
+            if self.runner.pages.groups:
+                self.page_log.append(
+                    {rid: self.runner.pages.block_table(h, 0).tolist() for rid, h in self.handles.items()}
+                )
+        for rid in step.get("end", []):
+            rid = str(rid)
+            if rid not in self.handles:
+                raise ReplayError(f"step {step.get('step')}: cannot end unknown request {rid!r}")
+            self.runner.release(self.handles.pop(rid))
+        if logits is None or logits.shape[0] == 0:
+            return None
+        return logits
+
+
+def replay_stream(runner: ModelRunner, lines: Iterable[str], out_dir: str, out=sys.stdout) -> None:
+    """Read steps (one JSON object a line), write ``out_dir/<step>.f32`` for steps
+    in which something is wanted, print ``done <step>`` after each."""
+    os.makedirs(out_dir, exist_ok=True)
+    rp = Replayer(runner)
+    for line in lines:
+        line = line.strip()
+        if not line:
+            continue
+        step = json.loads(line)
+        logits = rp.run_step(step)
+        if logits is not None:
+            arr = logits.detach().to(torch.float32).cpu().numpy().astype("<f4", copy=False)
+            tmp = os.path.join(out_dir, f".{step['step']}.f32.tmp")
+            arr.tofile(tmp)
+            os.replace(tmp, os.path.join(out_dir, f"{step['step']}.f32"))
+        elif torch.cuda.is_available():
+            torch.cuda.synchronize()
+        print(f"done {step['step']}", file=out, flush=True)

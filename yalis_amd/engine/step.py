@@ -1,0 +1,196 @@
+"""The step function: run a batch of (request, its next tokens) from the cache and
+return the logits at the wanted places.
+
+``ModelRunner`` owns the model, the cache memory and the page manager.  ``step``
+takes any mix of spans (portions of prompts beside single decoded tokens, cut
+anywhere), runs only those tokens as one batch and returns float32 logits
+``[wanted, vocab]``.  The reference has two step functions, one for whole prompts
+and one for single tokens (yalis/engine.py:63-105 and :108-143), and projects every
+position to the vocabulary (yalis/external/model.py:184); here there is one, and
+the head runs on the wanted rows only.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheMemory, GroupShape, PageManager
+from ..config.runtime import EngineConfig
+from .batch import HostBatch, SeqSpan, build_host_batch, named_arrays, pack
+
+
+class Site:
+    """What one run entry sees of the cache memory during a step."""
+
+    def __init__(self, info, memory: CacheMemory):
+        self.info = info
+        self.group = info.group
+        self.owns_cache = info.owns_cache
+        self._memory = memory
+
+    def kv(self):
+        if self.group is None:
+            return None, None
+        return self._memory.kv(self.group, self.info.index_in_group)
+
+    def state(self) -> Optional[torch.Tensor]:
+        """Per-request state of this entry: [num_slots, ...]; rows are chosen by
+        ``StepContext.arrays['state_slots']``."""
+        if self.info.state_index is None:
+            return None
+        return self._memory.states[self.info.state_index]
+
+
+class StepContext:
+    """Everything a part may read during a step."""
+
+    def __init__(self, host: HostBatch, arrays: Dict[str, torch.Tensor], sites: List[Site], rt):
+        self.host = host
+        self.arrays = arrays
+        self.rt = rt
+        self._sites = sites
+        self.n_tokens = host.n_tokens
+        self.n_seqs = host.n_seqs
+        self.max_qlen = host.max_qlen
+        self.max_ctx = host.max_ctx
+
+    def site(self, entry: int) -> Site:
+        return self._sites[entry]
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step, as callers give it."""
+
+    request: int
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+class _Uploader:
+    """One host-to-device copy per step through pinned staging buffers."""
+
+    def __init__(self, device: str):
+        self.device = torch.device(device)
+        self.cuda = self.device.type == "cuda"
+        self.bufs: List[Optional[torch.Tensor]] = [None, None]
+        self.events: List[Optional[torch.cuda.Event]] = [None, None]
+        self.turn = 0
+
+    def upload(self, buf: np.ndarray) -> torch.Tensor:
+        if not self.cuda:
+            return torch.from_numpy(buf.copy())
+        i = self.turn
+        self.turn ^= 1
+        if self.events[i] is not None:
+            self.events[i].synchronize()
+        if self.bufs[i] is None or self.bufs[i].numel() < buf.size:
+            self.bufs[i] = torch.empty(max(4096, 2 * buf.size), dtype=torch.int32, pin_memory=True)
+        stage = self.bufs[i][: buf.size]
+        stage.numpy()[:] = buf
+        dev = torch.empty(buf.size, dtype=torch.int32, device=self.device)
+        dev.copy_(stage, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self.events[i] = ev
+        return dev
+
+
+class ModelRunner:
+    def __init__(self, model, config: EngineConfig):
+        self.model = model
+        self.config = config
+        self.rt = model.rt
+        self.page_size = config.page_size
+        n_pages = config.resolved_num_pages()
+        self.group_shapes = [GroupShape(n_pages, g.need.window) for g in model.cache_groups]
+        self.pages = PageManager(self.page_size, self.group_shapes, config.max_num_seqs)
+        self.memory = CacheMemory(
+            model,
+            self.page_size,
+            [g.num_pages for g in self.group_shapes],
+            config.max_num_seqs,
+            self.rt.act_dtype,
+            config.device,
+        )
+        self.sites = [Site(info, self.memory) for info in model.sites]
+        self.builders = model.step_input_builders()
+        self.cached: Dict[int, int] = {}  # request -> tokens in the cache
+        self._uploader = _Uploader(config.device)
+        self.last_host_batch: Optional[HostBatch] = None
+
+    # ----------------------------------------------------------------- requests
+    def admit(self, request: int) -> bool:
+        """A state slot for the request (cleared); False when none is free."""
+        slot = self.pages.admit(request)
+        if slot is None:
+            return False
+        self.memory.clear_state(slot)
+        self.cached[request] = 0
+        return True
+
+    def is_live(self, request: int) -> bool:
+        return request in self.cached
+
+    def reserve(self, request: int, n_new_tokens: int) -> bool:
+        """Pages for the request's next ``n_new_tokens`` tokens; False (and no
+        change) when the pool cannot give them."""
+        return self.pages.reserve(request, self.cached[request] + n_new_tokens)
+
+    def release(self, request: int) -> None:
+        self.pages.release(request)
+        del self.cached[request]
+
+    def free_pages(self) -> List[int]:
+        return [self.pages.free_pages(g) for g in range(len(self.group_shapes))]
+
+    # --------------------------------------------------------------------- step
+    @torch.inference_mode()
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run the entries as one batch.  Pages for the new tokens must have been
+        reserved.  Returns float32 logits [sum of wanted places, vocab], in the
+        order of the entries and of their ``want``."""
+        spans = []
+        seen = set()
+        for e in entries:
+            if e.request not in self.cached:
+                raise KeyError(f"request {e.request} is not live")
+            if e.request in seen:
+                raise ValueError(f"request {e.request} occurs twice in one step")
+            seen.add(e.request)
+            first = self.cached[e.request]
+            if first + len(e.tokens) > self.rt.max_positions:
+                raise ValueError(
+                    f"request {e.request} would reach {first + len(e.tokens)} tokens, the engine is sized for {self.rt.max_positions}"
+                )
+            vocab = self.model.spec.vocab_size
+            for t in e.tokens:
+                if not 0 <= int(t) < vocab:
+                    raise ValueError(f"token id {t} is outside the vocabulary of {vocab}")
+            spans.append(
+                SeqSpan(
+                    tokens=e.tokens,
+                    first_position=first,
+                    block_tables=self.pages.block_tables(e.request),
+                    state_slot=self.pages.slot(e.request),
+                    want=e.want,
+                )
+            )
+        hb = build_host_batch(spans, len(self.group_shapes), self.page_size)
+        arrays = named_arrays(hb, self.builders)
+        buf, layout = pack(arrays)
+        dev = self._uploader.upload(buf)
+        views = {
+            name: dev[off : off + int(np.prod(shape, dtype=np.int64))].view(*shape)
+            for name, (off, shape) in layout.items()
+        }
+        ctx = StepContext(hb, views, self.sites, self.rt)
+        self.last_host_batch = hb
+        logits = self.model.forward(ctx)
+        for e in entries:
+            self.cached[e.request] += len(e.tokens)
+            self.pages.advance(e.request, self.cached[e.request])
+        return logits

@@ -1,0 +1,149 @@
+"""The generic decoder: parts assembled from a ``ModelSpec``.
+
+It knows no architecture.  It builds every part named by the spec, gathers the
+tensors they ask for, works out which run entries keep a cache and how those
+caches group by need, and runs a step: embedding, the run order, the final norm
+on the wanted rows, the head (the order of yalis/external/model.py:122-197).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, Dict, List, Optional, Tuple
+
+import torch
+
+from ..config.specs import ModelSpec
+from ..parts import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS
+from ..parts.base import KVNeed, Runtime, StateNeed
+from ..weights.loader import TensorSpec
+
+
+@dataclass(frozen=True)
+class CacheGroup:
+    """Run entries whose mixers need the same kind of pages share one pool and one
+    block table per request."""
+
+    need: KVNeed
+    entries: Tuple[int, ...]  # run-order indices that own a cache in this group
+
+
+@dataclass(frozen=True)
+class SiteInfo:
+    """Where one run entry keeps what it remembers."""
+
+    entry: int
+    layer: int
+    group: Optional[int]  # cache group read by this entry (None: the mixer caches nothing)
+    index_in_group: Optional[int]  # which of the group's caches
+    owns_cache: bool  # False: reads another entry's cache and writes none
+    state_index: Optional[int]  # which per-request state tensor (None: no state)
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec, rt: Runtime):
+        spec.validate()
+        self.spec = spec
+        self.rt = rt
+        self.embedding = EMBEDDINGS.get(spec.embedding.kind)(spec.embedding.params, rt)
+        self.final_norm = NORMS.get(spec.final_norm.kind)(spec.final_norm.params, rt)
+        self.head = HEADS.get(spec.head.kind)(spec.head.params, rt)
+
+        # a layer's mixer needs k/v projections iff some run entry of it owns a cache
+        owns = [False] * len(spec.layers)
+        for e in spec.run_order:
+            if e.cache_from is None:
+                owns[e.layer] = True
+        self.blocks = []
+        for i, ls in enumerate(spec.layers):
+            mixer_params = dict(ls.mixer.params)
+            if not owns[i]:
+                mixer_params["projects_kv"] = False
+            mixer = MIXERS.get(ls.mixer.kind)(mixer_params, rt)
+            ffn = FEED_FORWARDS.get(ls.feed_forward.kind)(ls.feed_forward.params, rt)
+            n1 = NORMS.get(ls.mixer_norm.kind)(ls.mixer_norm.params, rt)
+            n2 = NORMS.get(ls.feed_forward_norm.kind)(ls.feed_forward_norm.params, rt)
+            self.blocks.append(BLOCKS.get(ls.block)(n1, mixer, n2, ffn))
+
+        self.cache_groups, self.state_needs, self.sites = self._plan_memory()
+
+    # ------------------------------------------------------------------ memory plan
+    def _plan_memory(self):
+        groups: List[Tuple[KVNeed, List[int]]] = []
+        states: List[StateNeed] = []
+        sites: List[SiteInfo] = []
+        for i, e in enumerate(self.spec.run_order):
+            mixer = self.blocks[e.layer].mixer
+            need = mixer.kv_need()
+            group = index = None
+            owns = False
+            if need is not None:
+                if e.cache_from is None:
+                    for g, (n, members) in enumerate(groups):
+                        if n == need:
+                            group = g
+                            break
+                    else:
+                        groups.append((need, []))
+                        group = len(groups) - 1
+                    index = len(groups[group][1])
+                    groups[group][1].append(i)
+                    owns = True
+                else:
+                    src = sites[e.cache_from]
+                    src_need = self.blocks[src.layer].mixer.kv_need()
+                    if src.group is None or src_need != need:
+                        raise ValueError(
+                            f"run_order[{i}] borrows the cache of entry {e.cache_from}, whose need {src_need} differs from {need}"
+                        )
+                    group, index = src.group, src.index_in_group
+            elif e.cache_from is not None:
+                raise ValueError(f"run_order[{i}] names cache_from but its mixer keeps no cache")
+            sneed = mixer.state_need()
+            sidx = None
+            if sneed is not None:
+                sidx = len(states)
+                states.append(sneed)
+            sites.append(SiteInfo(i, e.layer, group, index, owns, sidx))
+        cache_groups = [CacheGroup(n, tuple(m)) for n, m in groups]
+        return cache_groups, states, sites
+
+    # ---------------------------------------------------------------------- tensors
+    def all_parts(self):
+        yield self.embedding
+        for b in self.blocks:
+            yield from b.parts()
+        yield self.final_norm
+        yield self.head
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        out: Dict[str, TensorSpec] = {}
+        for p in self.all_parts():
+            for name, spec in p.tensor_specs().items():
+                if name in out and out[name].shape != spec.shape:
+                    raise ValueError(f"tensor {name!r} is asked for with shapes {out[name].shape} and {spec.shape}")
+                out.setdefault(name, spec)
+        return out
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for p in self.all_parts():
+            p.load(tensors)
+
+    def step_input_builders(self) -> Dict[str, Callable]:
+        out: Dict[str, Callable] = {}
+        for p in self.all_parts():
+            for name, fn in p.step_inputs().items():
+                out.setdefault(name, fn)
+        return out
+
+    # -------------------------------------------------------------------------- run
+    def forward(self, ctx) -> torch.Tensor:
+        """Run the step's tokens; returns float32 logits [wanted rows, vocab]."""
+        residual = self.embedding.forward(ctx.arrays["token_ids"])
+        delta = None
+        for i, e in enumerate(self.spec.run_order):
+            delta = self.blocks[e.layer].forward(residual, delta, ctx, ctx.site(i))
+        rows = ctx.arrays["logit_rows"]
+        if rows.numel() == 0:
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=residual.device)
+        h = self.final_norm.gather_add_norm(residual, delta, rows)
+        return self.head.forward(h)

@@ -1,0 +1,332 @@
+"""The kernel library: ctypes bindings of the HIP kernels in ``yalis_amd/csrc``.
+
+Every method takes torch tensors on the GPU, checks what the kernels assume, and
+launches on torch's current stream.  There is no other implementation behind these
+methods: when the library cannot be built or loaded, constructing ``HipOps``
+raises.  Plain matrix products of many rows in bfloat16 go to the vendor library
+through ``torch.matmul`` (the reference uses cuBLAS in the same places,
+yalis/external/model.py:449,462-466,717-722); few-row products, every float32
+product and everything else are the hand-written kernels.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from .build import load_kernels
+
+_F32, _BF16 = 0, 1
+_c_int = ctypes.c_int
+_c_float = ctypes.c_float
+_c_size_t = ctypes.c_size_t
+_vp = ctypes.c_void_p
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return _F32
+    if dtype == torch.bfloat16:
+        return _BF16
+    raise KernelError(f"kernels take float32 and bfloat16 only, got {dtype}")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+_SIGNATURES = {
+    "yk_abi_version": ([], _c_int),
+    "yk_embed": ([_vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
+    "yk_add_rmsnorm": (
+        [_vp, _vp, _c_int, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_float, _c_int, _vp],
+        _c_int,
+    ),
+    "yk_rope_append": (
+        [_vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _c_int, _c_int, _c_int, _vp, _vp, _vp, _c_int, _vp],
+        _c_int,
+    ),
+    "yk_gated_act": ([_vp, _vp, _c_int, _c_int, _c_int, _c_int, _vp], _c_int),
+    "yk_gemm_fma": (
+        [_vp, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
+        _c_int,
+    ),
+    "yk_gemm_skinny_splits": ([_c_int, _c_int, _c_int], _c_int),
+    "yk_gemm_mfma_skinny": (
+        [_vp, _vp, _vp, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
+        _c_int,
+    ),
+    "yk_attn_generic": (
+        [_vp, _c_int, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp],
+        _c_int,
+    ),
+    "yk_attn_mfma_supported": ([_c_int], _c_int),
+    "yk_attn_heads_per_tile": ([_c_int, _c_int], _c_int),
+    "yk_attn_tokens_per_tile": ([_c_int, _c_int], _c_int),
+    "yk_attn_mfma_workspace": ([_c_int, _c_int, _c_int, _c_int, _c_int], _c_size_t),
+    "yk_attn_mfma": (
+        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _vp, _c_size_t, _vp],
+        _c_int,
+    ),
+    "yk_argmax": ([_vp, _vp, _c_int, _c_int, _vp], _c_int),
+    "yk_sample": ([_vp, _vp, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _vp], _c_int),
+}
+
+# Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
+# above it the vendor library does.
+SKINNY_MAX_ROWS = 64
+# Waves the attention launch aims at when it decides how far to split the keys.
+ATTN_TARGET_WAVES = 1024
+
+
+class HipOps:
+    def __init__(self, device: str = "cuda:0"):
+        if not torch.cuda.is_available():
+            raise KernelError("HipOps needs a GPU: torch.cuda.is_available() is False")
+        self.device = torch.device(device)
+        self.lib = load_kernels()
+        self.lib.yk_last_error.restype = ctypes.c_char_p
+        for name, (args, res) in _SIGNATURES.items():
+            fn = getattr(self.lib, name)
+            fn.argtypes = args
+            fn.restype = res
+        if self.lib.yk_abi_version() != 1:
+            raise KernelError("kernel library and bindings disagree; rebuild (python -c 'import __graft_entry__ as g; g.build()')")
+        self._workspace: Optional[torch.Tensor] = None
+
+    # ------------------------------------------------------------------ helpers
+    def _stream(self) -> int:
+        return torch.cuda.current_stream(self.device).cuda_stream
+
+    def _check(self, rc: int) -> None:
+        if rc != 0:
+            raise KernelError(self.lib.yk_last_error().decode())
+
+    def _ws(self, floats: int) -> torch.Tensor:
+        """Float32 scratch that grows and is reused (stream order keeps uses apart)."""
+        if self._workspace is None or self._workspace.numel() < floats:
+            self._workspace = torch.empty(max(floats, 1 << 20), dtype=torch.float32, device=self.device)
+        return self._workspace
+
+    @staticmethod
+    def _rows(t: torch.Tensor, what: str) -> None:
+        if t.dim() != 2 or t.stride(1) != 1:
+            raise KernelError(f"{what}: expected a 2-D tensor with contiguous rows, got shape {tuple(t.shape)} strides {t.stride()}")
+
+    # ---------------------------------------------------------- sizes a part may ask
+    def check_attention_sizes(self, n_heads: int, n_kv: int, head_dim: int, page_size: int) -> None:
+        if n_heads % n_kv:
+            raise KernelError(f"attention: {n_heads} heads are not a multiple of {n_kv} kv heads")
+        if head_dim % 16 or not 16 <= head_dim <= 256:
+            raise KernelError(f"attention: head_dim must be a multiple of 16 between 16 and 256, got {head_dim}")
+        if page_size % 16:
+            raise KernelError(f"attention: page_size must be a multiple of 16, got {page_size}")
+
+    def attention_tokens_per_tile(self, n_heads: int, n_kv: int) -> int:
+        return self.lib.yk_attn_tokens_per_tile(n_heads, n_kv)
+
+    # ------------------------------------------------------------------ embedding
+    def embed(self, token_ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+        self._rows(table, "embed table")
+        n = token_ids.numel()
+        out = torch.empty((n, table.shape[1]), dtype=torch.float32, device=table.device)
+        self._check(
+            self.lib.yk_embed(
+                token_ids.data_ptr(), table.data_ptr(), _code(table.dtype), out.data_ptr(), n,
+                table.shape[1], table.shape[0], self._stream(),
+            )
+        )
+        return out
+
+    # ----------------------------------------------------------------------- norm
+    def _norm(self, residual, delta, rows, weight, eps, unit_offset, out_dtype, n_out):
+        self._rows(residual, "residual")
+        if residual.dtype != torch.float32 or not residual.is_contiguous():
+            raise KernelError("the residual stream must be contiguous float32")
+        width = residual.shape[1]
+        if weight.numel() != width:
+            raise KernelError(f"norm weight has {weight.numel()} elements, rows have {width}")
+        if delta is not None and (tuple(delta.shape) != tuple(residual.shape) or not delta.is_contiguous()):
+            raise KernelError(f"delta {tuple(delta.shape)} does not match the residual {tuple(residual.shape)}")
+        out = torch.empty((n_out, width), dtype=out_dtype, device=residual.device)
+        self._check(
+            self.lib.yk_add_rmsnorm(
+                residual.data_ptr(), _ptr(delta), 0 if delta is None else _code(delta.dtype),
+                _ptr(rows), weight.data_ptr(), _code(weight.dtype), out.data_ptr(), _code(out_dtype),
+                n_out, width, float(eps), int(bool(unit_offset)), self._stream(),
+            )
+        )
+        return out
+
+    def add_rmsnorm(self, residual, delta, weight, eps, unit_offset, out_dtype):
+        return self._norm(residual, delta, None, weight, eps, unit_offset, out_dtype, residual.shape[0])
+
+    def gather_add_rmsnorm(self, residual, delta, rows, weight, eps, unit_offset, out_dtype):
+        return self._norm(residual, delta, rows, weight, eps, unit_offset, out_dtype, rows.numel())
+
+    # --------------------------------------------------------------------- linear
+    def linear(self, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        """x [M, K] . w [N, K]^T -> [M, N]."""
+        self._rows(x, "linear input")
+        self._rows(w, "linear weight")
+        m, k = x.shape
+        n = w.shape[0]
+        if w.shape[1] != k:
+            raise KernelError(f"linear: input has {k} columns, weight has {w.shape[1]}")
+        if m == 0:
+            return torch.empty((0, n), dtype=out_dtype, device=x.device)
+        bf = torch.bfloat16
+        aligned = k % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+        if x.dtype == bf and w.dtype == bf and aligned:
+            if m <= SKINNY_MAX_ROWS or out_dtype != bf:
+                return self.gemm_mfma_skinny(x, w, out_dtype)
+            return torch.matmul(x, w.t())  # vendor library, bfloat16 in and out
+        return self.gemm_fma(x, w, out_dtype)
+
+    def gemm_fma(self, x, w, out_dtype):
+        m, k = x.shape
+        n = w.shape[0]
+        y = torch.empty((m, n), dtype=out_dtype, device=x.device)
+        self._check(
+            self.lib.yk_gemm_fma(
+                x.data_ptr(), _code(x.dtype), w.data_ptr(), _code(w.dtype), y.data_ptr(), _code(out_dtype),
+                m, n, k, x.stride(0), w.stride(0), n, self._stream(),
+            )
+        )
+        return y
+
+    def gemm_mfma_skinny(self, x, w, out_dtype):
+        m, k = x.shape
+        n = w.shape[0]
+        y = torch.empty((m, n), dtype=out_dtype, device=x.device)
+        splits = self.lib.yk_gemm_skinny_splits(m, n, k)
+        ws = self._ws(splits * m * n)
+        self._check(
+            self.lib.yk_gemm_mfma_skinny(
+                x.data_ptr(), w.data_ptr(), y.data_ptr(), _code(out_dtype), ws.data_ptr(), ws.numel(),
+                m, n, k, x.stride(0), w.stride(0), n, self._stream(),
+            )
+        )
+        return y
+
+    # ------------------------------------------------- rotary + append to the cache
+    def rope_append(self, qkv, n_heads, n_kv, head_dim, positions, cos, sin, rotary_dim,
+                    interleaved, k_cache, v_cache, slots, page_size):
+        self._rows(qkv, "qkv")
+        n = qkv.shape[0]
+        if qkv.shape[1] != (n_heads + 2 * n_kv) * head_dim:
+            raise KernelError(f"qkv rows have {qkv.shape[1]} elements, expected {(n_heads + 2 * n_kv) * head_dim}")
+        if positions.numel() != n or (n_kv > 0 and slots.numel() != n):
+            raise KernelError("positions/slots do not match the number of tokens")
+        max_pos = 0
+        if rotary_dim:
+            if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.shape != sin.shape or cos.shape[1] != rotary_dim // 2:
+                raise KernelError("rotary tables must be float32 [positions, rotary_dim/2]")
+            max_pos = cos.shape[0]
+        if n_kv > 0:
+            if k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype:
+                raise KernelError("cache and activations differ in dtype")
+            if tuple(k_cache.shape[1:]) != (n_kv, page_size, head_dim) or tuple(v_cache.shape[1:]) != (n_kv, head_dim, page_size):
+                raise KernelError(f"cache pages have shapes {tuple(k_cache.shape)}, {tuple(v_cache.shape)}")
+        self._check(
+            self.lib.yk_rope_append(
+                qkv.data_ptr(), _code(qkv.dtype), n, qkv.stride(0), n_heads, n_kv, head_dim,
+                positions.data_ptr(), _ptr(cos) if rotary_dim else None, _ptr(sin) if rotary_dim else None,
+                rotary_dim, int(bool(interleaved)), max_pos,
+                _ptr(k_cache) if n_kv else None, _ptr(v_cache) if n_kv else None,
+                _ptr(slots) if n_kv else None, page_size, self._stream(),
+            )
+        )
+
+    # ------------------------------------------------------------------ attention
+    def attention(self, qkv, n_heads, n_kv_rows, n_kv, head_dim, k_cache, v_cache, page_size,
+                  scale, window, ctx, group, tiles) -> torch.Tensor:
+        """Queries are the first n_heads heads of each row of ``qkv``; keys and values
+        come from the cache through the block table of ``group``."""
+        self._rows(qkv, "qkv")
+        n = qkv.shape[0]
+        bt = ctx.arrays[f"block_table_g{group}"]
+        if tuple(k_cache.shape[1:]) != (n_kv, page_size, head_dim) or tuple(v_cache.shape[1:]) != (n_kv, head_dim, page_size):
+            raise KernelError(f"cache pages have shapes {tuple(k_cache.shape)}, {tuple(v_cache.shape)}")
+        if k_cache.dtype != qkv.dtype:
+            raise KernelError("cache and activations differ in dtype")
+        out = torch.empty((n, n_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+        use_mfma = (
+            qkv.dtype == torch.bfloat16
+            and self.lib.yk_attn_mfma_supported(head_dim)
+            and qkv.stride(0) % 8 == 0
+            and qkv.data_ptr() % 16 == 0
+        )
+        if use_mfma:
+            n_tiles = tiles.shape[0]
+            hpt = self.lib.yk_attn_heads_per_tile(n_heads, n_kv)
+            chunks = -(-(n_heads // n_kv) // hpt)
+            waves = n_tiles * n_kv * chunks
+            key_blocks = max(1, -(-ctx.max_ctx // 64))
+            splits = max(1, min(-(-ATTN_TARGET_WAVES // waves), key_blocks, 256))
+            ws_floats = self.lib.yk_attn_mfma_workspace(n_tiles, n_heads, n_kv, head_dim, splits)
+            ws = self._ws(ws_floats) if ws_floats else None
+            self._check(
+                self.lib.yk_attn_mfma(
+                    qkv.data_ptr(), qkv.stride(0), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                    tiles.data_ptr(), n_tiles, bt.data_ptr(), bt.shape[1], page_size, head_dim, n_heads, n_kv,
+                    float(scale), int(window), splits, _ptr(ws), 0 if ws is None else ws.numel(), self._stream(),
+                )
+            )
+        else:
+            self._check(
+                self.lib.yk_attn_generic(
+                    qkv.data_ptr(), qkv.stride(0), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                    _code(qkv.dtype), ctx.arrays["positions"].data_ptr(), ctx.arrays["token_seq"].data_ptr(),
+                    bt.data_ptr(), bt.shape[1], n, page_size, head_dim, n_heads, n_kv, float(scale), int(window),
+                    self._stream(),
+                )
+            )
+        return out
+
+    # ----------------------------------------------------------------- activation
+    def gated_act(self, gu: torch.Tensor, activation: str) -> torch.Tensor:
+        self._rows(gu, "gate/up")
+        if not gu.is_contiguous() or gu.shape[1] % 2:
+            raise KernelError("gate/up must be contiguous with an even number of columns")
+        act = {"silu": 0, "gelu_tanh": 1}.get(activation)
+        if act is None:
+            raise KernelError(f"unknown activation {activation!r}")
+        inter = gu.shape[1] // 2
+        out = torch.empty((gu.shape[0], inter), dtype=gu.dtype, device=gu.device)
+        self._check(
+            self.lib.yk_gated_act(gu.data_ptr(), out.data_ptr(), _code(gu.dtype), gu.shape[0], inter, act, self._stream())
+        )
+        return out
+
+    # ------------------------------------------------------------------- sampling
+    def argmax(self, logits: torch.Tensor) -> torch.Tensor:
+        if logits.dtype != torch.float32 or not logits.is_contiguous() or logits.dim() != 2:
+            raise KernelError("argmax takes contiguous float32 logits [rows, vocab]")
+        out = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device)
+        self._check(self.lib.yk_argmax(logits.data_ptr(), out.data_ptr(), logits.shape[0], logits.shape[1], self._stream()))
+        return out
+
+    def sample(self, logits, temperature, top_k, top_p, seeds, draws) -> torch.Tensor:
+        """Per row: temperature (float32; 0 = greedy), top_k (int32; 0 = off), top_p
+        (float32), seed and draw number (int32).  Returns int32 token ids."""
+        if logits.dtype != torch.float32 or not logits.is_contiguous() or logits.dim() != 2:
+            raise KernelError("sample takes contiguous float32 logits [rows, vocab]")
+        rows = logits.shape[0]
+        for name, t, dt in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
+                            ("top_p", top_p, torch.float32), ("seeds", seeds, torch.int32), ("draws", draws, torch.int32)):
+            if t.dtype != dt or t.numel() != rows or not t.is_contiguous():
+                raise KernelError(f"sample: {name} must be {dt} with one entry per row")
+        out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+        self._check(
+            self.lib.yk_sample(
+                logits.data_ptr(), out.data_ptr(), rows, logits.shape[1], temperature.data_ptr(), top_k.data_ptr(),
+                top_p.data_ptr(), seeds.data_ptr(), draws.data_ptr(), self._stream(),
+            )
+        )
+        return out

@@ -1,0 +1,126 @@
+"""Causal self-attention with grouped key/value heads over a paged cache.
+
+Reference: yalis/external/model.py:525-608 (projection, split into heads, rotary,
+attention, output projection); the mask and softmax rules are those of
+yalis/attention/backend_impl/sdpa_and_flex.py:15-19, 85-90, 300-312: query head h
+reads key/value head h // (H/G), key j is visible to the query at position p iff
+j <= p, softmax in float32.  The reference stores q, k and v rows interleaved per
+group in one matrix (yalis/external/model.py:445-456); here the three checkpoint
+matrices are stacked [q; k; v], which is the same arithmetic.
+
+params: prefix, hidden_size, num_heads, num_kv_heads, head_dim, scale, window
+(None: every earlier key), position (a PartSpec or None), names (optional
+overrides of the four tensor names below the prefix).
+"""
+from __future__ import annotations
+
+from typing import Dict, Mapping
+
+import torch
+
+from ..config.specs import PartSpec
+from ..engine.batch import attention_tiles
+from ..weights.loader import TensorSpec
+from .base import POSITIONS, KVNeed, Mixer, Runtime, register_mixer
+
+
+@register_mixer("attention")
+class Attention(Mixer):
+    def __init__(self, params, rt: Runtime):
+        super().__init__(params, rt)
+        self.prefix = params["prefix"]
+        self.hidden = int(params["hidden_size"])
+        self.n_heads = int(params["num_heads"])
+        self.n_kv = int(params["num_kv_heads"])
+        self.head_dim = int(params["head_dim"])
+        self.scale = float(params["scale"])
+        self.window = params.get("window")
+        if self.n_heads % self.n_kv:
+            raise ValueError(f"num_heads={self.n_heads} is not a multiple of num_kv_heads={self.n_kv}")
+        names = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight"}
+        names.update(params.get("names", {}))
+        self.names = {k: f"{self.prefix}.{v}" for k, v in names.items()}
+        # False when every run entry of this layer borrows another entry's cache
+        self.projects_kv = bool(params.get("projects_kv", True))
+        pos: PartSpec = params.get("position")
+        self.position = None if pos is None else POSITIONS.get(pos.kind)(pos.params, rt)
+        if self.position is not None and self.position.rotary_dim > self.head_dim:
+            raise ValueError("rotary_dim exceeds head_dim")
+        rt.ops.check_attention_sizes(self.n_heads, self.n_kv, self.head_dim, rt.page_size)
+        self.tokens_per_tile = rt.ops.attention_tokens_per_tile(self.n_heads, self.n_kv)
+        self.group = None
+        self.w_qkv = self.w_q = self.w_o = None
+
+    # ---- what it needs
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        hd = self.n_heads * self.head_dim
+        kd = self.n_kv * self.head_dim
+        specs = {
+            self.names["q"]: TensorSpec((hd, self.hidden)),
+            self.names["o"]: TensorSpec((self.hidden, hd)),
+        }
+        if self.projects_kv:
+            specs[self.names["k"]] = TensorSpec((kd, self.hidden))
+            specs[self.names["v"]] = TensorSpec((kd, self.hidden))
+        return specs
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        q = tensors[self.names["q"]]
+        if self.projects_kv:
+            self.w_qkv = torch.cat([q, tensors[self.names["k"]], tensors[self.names["v"]]], dim=0).contiguous()
+            self.w_q = self.w_qkv[: q.shape[0]]
+        else:
+            self.w_q = q
+        self.w_o = tensors[self.names["o"]]
+
+    def kv_need(self) -> KVNeed:
+        return KVNeed(self.n_kv, self.head_dim, self.window)
+
+    def step_inputs(self):
+        tpt = self.tokens_per_tile
+        return {f"attention_tiles_{tpt}": lambda hb: attention_tiles(hb, tpt)}
+
+    # ---- what it computes
+    def forward(self, h: torch.Tensor, ctx, site) -> torch.Tensor:
+        ops = self.rt.ops
+        if site.owns_cache:
+            if not self.projects_kv:
+                raise RuntimeError(f"{self.prefix}: run entry owns a cache but the layer has no k/v projections")
+            qkv = ops.linear(h, self.w_qkv, self.rt.act_dtype)
+            n_kv_rows = self.n_kv
+        else:
+            qkv = ops.linear(h, self.w_q, self.rt.act_dtype)
+            n_kv_rows = 0
+        k_cache, v_cache = site.kv()
+        pos = self.position
+        ops.rope_append(
+            qkv,
+            self.n_heads,
+            n_kv_rows,
+            self.head_dim,
+            ctx.arrays["positions"],
+            None if pos is None else pos.cos,
+            None if pos is None else pos.sin,
+            0 if pos is None else pos.rotary_dim,
+            False if pos is None else pos.interleaved,
+            k_cache,
+            v_cache,
+            ctx.arrays[f"slots_g{site.group}"],
+            self.rt.page_size,
+        )
+        out = ops.attention(
+            qkv,
+            self.n_heads,
+            n_kv_rows,
+            self.n_kv,
+            self.head_dim,
+            k_cache,
+            v_cache,
+            self.rt.page_size,
+            self.scale,
+            0 if self.window is None else int(self.window),
+            ctx,
+            site.group,
+            ctx.arrays[f"attention_tiles_{self.tokens_per_tile}"],
+        )
+        return ops.linear(out, self.w_o, self.rt.act_dtype)

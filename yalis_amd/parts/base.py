@@ -1,0 +1,163 @@
+"""Interfaces of the parts a layer is assembled from, and their registries.
+
+A part is built from ``PartSpec.params`` (its sizes and constants) and a
+``Runtime`` (device, precision, kernel library).  It names the checkpoint tensors
+it needs, receives them once, and computes through ``Runtime.ops`` only.  No part
+knows which model it is in.
+
+Adding a part means: subclass the interface, decorate it with the matching
+``register_*``, and name its ``kind`` in a ``PartSpec``.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Callable, Dict, Mapping, Optional, Tuple
+
+import torch
+
+from ..weights.loader import TensorSpec
+
+
+@dataclass
+class Runtime:
+    """What every part computes with."""
+
+    device: str
+    engine_dtype: str  # "bfloat16" or "float32"
+    ops: Any  # the kernel library (yalis_amd.ops.hip.HipOps)
+    max_positions: int  # longest sequence the engine will run
+    page_size: int = 64
+
+    @property
+    def act_dtype(self) -> torch.dtype:
+        return torch.float32 if self.engine_dtype == "float32" else torch.bfloat16
+
+
+@dataclass(frozen=True)
+class KVNeed:
+    """A mixer's need for cached keys and values: per token ``num_kv_heads`` rows
+    of ``head_dim`` for keys and the same for values.  ``window`` = how many of the
+    latest tokens are ever read again (None: all of them)."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """A mixer's need for per-request state of fixed size (zero at admission)."""
+
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class Part:
+    """Common to all parts."""
+
+    def __init__(self, params: Mapping[str, Any], rt: Runtime):
+        self.params = dict(params)
+        self.rt = rt
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        """Checkpoint name -> what is needed under it."""
+        return {}
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        """Receive the tensors named by ``tensor_specs`` (already on the device)."""
+
+    def step_inputs(self) -> Dict[str, Callable]:
+        """Per-step integer arrays this part wants on the device, by unique name:
+        name -> function(HostBatch) -> numpy int32 array.  They travel in the
+        step's single upload and arrive as ``StepContext.arrays[name]``."""
+        return {}
+
+
+class Mixer(Part):
+    """Mixes information across the tokens of a request (attention here)."""
+
+    def kv_need(self) -> Optional[KVNeed]:
+        return None
+
+    def state_need(self) -> Optional[StateNeed]:
+        return None
+
+    def set_cache_group(self, group: int) -> None:
+        """Told once at build time which cache group holds this mixer's pages."""
+
+    def forward(self, h: torch.Tensor, ctx: Any, site: Any) -> torch.Tensor:
+        """h: [N, hidden] normed activations of the step's tokens; returns the
+        mixer's contribution to the residual stream [N, hidden].  ``site`` gives
+        this run entry's cache and state (engine.step.Site)."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, ctx: Any) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Norm(Part):
+    def add_norm(self, residual: torch.Tensor, delta: Optional[torch.Tensor]) -> torch.Tensor:
+        """residual (float32, [N, size]) += delta in place when delta is given;
+        returns norm(residual) in the activation dtype."""
+        raise NotImplementedError
+
+    def gather_add_norm(self, residual, delta, rows) -> torch.Tensor:
+        """The same on the rows ``rows`` only, without changing ``residual``."""
+        raise NotImplementedError
+
+
+class Position(Part):
+    """A position encoding applied to queries and keys inside a mixer."""
+
+
+class Block:
+    """The arrangement of norms, mixer and feed-forward around the residual.
+    Built from four finished parts: (mixer_norm, mixer, feed_forward_norm,
+    feed_forward)."""
+
+    def parts(self):
+        raise NotImplementedError
+
+    def forward(self, residual, delta, ctx, site):
+        """residual: float32 [N, hidden], updated in place; delta: the previous
+        block's contribution not yet added (or None).  Returns this block's last
+        contribution, left for the next norm to add."""
+        raise NotImplementedError
+
+
+class _Registry:
+    def __init__(self, what: str):
+        self.what = what
+        self.table: Dict[str, Callable[..., Any]] = {}
+
+    def register(self, kind: str):
+        def deco(cls):
+            self.table[kind] = cls
+            cls.kind = kind
+            return cls
+
+        return deco
+
+    def get(self, kind: str):
+        if kind not in self.table:
+            raise KeyError(f"unknown {self.what} {kind!r}; registered: {sorted(self.table)}")
+        return self.table[kind]
+
+
+MIXERS = _Registry("mixer")
+FEED_FORWARDS = _Registry("feed-forward")
+NORMS = _Registry("norm")
+POSITIONS = _Registry("position encoding")
+BLOCKS = _Registry("block arrangement")
+EMBEDDINGS = _Registry("embedding")
+HEADS = _Registry("output head")
+
+register_mixer = MIXERS.register
+register_feed_forward = FEED_FORWARDS.register
+register_norm = NORMS.register
+register_position = POSITIONS.register
+register_block = BLOCKS.register
+register_embedding = EMBEDDINGS.register
+register_head = HEADS.register

@@ -1,0 +1,116 @@
+"""Loading a model's tensors by name.
+
+The parts of a model declare what they need (``TensorSpec`` by checkpoint name);
+``load_tensors`` reads exactly those from the folder and fails with ONE error that
+lists every missing tensor, every unexpected tensor and every wrong shape (the
+reference gets the same from ``load_state_dict(strict=True)``,
+yalis/model_loading.py:201-249).
+
+Precision rule: a floating tensor stored in 16 bits is kept in bfloat16, a tensor
+stored in 32 bits stays in 32 bits (such tensors are stored wide because they need
+it), integer tables become int32.  In the 32-bit mode of the engine every floating
+tensor is widened to float32 (exact).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, Dict, Iterable, Optional, Tuple
+
+import torch
+
+from .safetensors_io import TensorEntry, index_folder, read_tensor
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    """What a part needs under one checkpoint name.
+
+    kind: "float" or "int".
+    init: how the random-weights mode fills it: ("normal", std) or
+        ("one_plus_normal", std) or ("zeros",) or ("randint", high).
+    """
+
+    shape: Tuple[int, ...]
+    kind: str = "float"
+    init: Tuple = ("normal", 0.02)
+
+
+class WeightsError(RuntimeError):
+    """The checkpoint does not hold what the model needs."""
+
+    def __init__(self, where: str, missing, unexpected, wrong_shape, wrong_kind=()):
+        self.missing = list(missing)
+        self.unexpected = list(unexpected)
+        self.wrong_shape = list(wrong_shape)
+        self.wrong_kind = list(wrong_kind)
+        lines = [f"checkpoint in {where!r} does not match the model:"]
+        if self.missing:
+            lines.append(f"  missing tensors ({len(self.missing)}): " + ", ".join(self.missing))
+        if self.unexpected:
+            lines.append(f"  unexpected tensors ({len(self.unexpected)}): " + ", ".join(self.unexpected))
+        for name, got, want in self.wrong_shape:
+            lines.append(f"  wrong shape: {name} has {tuple(got)}, the model needs {tuple(want)}")
+        for name, got, want in self.wrong_kind:
+            lines.append(f"  wrong type: {name} is stored as {got}, the model needs {want}")
+        super().__init__("\n".join(lines))
+
+
+_FLOAT_TAGS = {"F64", "F32", "F16", "BF16"}
+_INT_TAGS = {"I64", "I32", "I16", "I8", "U8"}
+
+# Names a checkpoint may hold that no part asks for and that carry no weights
+# (the reference's converter drops them too, yalis/external/convert_hf_checkpoint.py:705-736).
+IGNORED_SUFFIXES = ("rotary_emb.inv_freq",)
+
+
+def target_dtype(storage_tag: str, kind: str, engine_dtype: str) -> torch.dtype:
+    if kind == "int":
+        return torch.int32
+    if engine_dtype == "float32":
+        return torch.float32
+    if storage_tag in ("F32", "F64"):
+        return torch.float32
+    return torch.bfloat16
+
+
+def check_against(entries: Dict[str, TensorEntry], wanted: Dict[str, TensorSpec], where: str) -> None:
+    missing = [n for n in wanted if n not in entries]
+    unexpected = [
+        n for n in entries if n not in wanted and not n.endswith(IGNORED_SUFFIXES)
+    ]
+    wrong_shape = [
+        (n, entries[n].shape, s.shape)
+        for n, s in wanted.items()
+        if n in entries and tuple(entries[n].shape) != tuple(s.shape)
+    ]
+    wrong_kind = []
+    for n, s in wanted.items():
+        if n in entries:
+            tag = entries[n].dtype
+            ok = tag in (_FLOAT_TAGS if s.kind == "float" else _INT_TAGS)
+            if not ok:
+                wrong_kind.append((n, tag, s.kind))
+    if missing or unexpected or wrong_shape or wrong_kind:
+        raise WeightsError(where, sorted(missing), sorted(unexpected), wrong_shape, wrong_kind)
+
+
+def load_tensors(
+    model_dir: str,
+    wanted: Dict[str, TensorSpec],
+    engine_dtype: str,
+    device: str,
+    progress: Optional[Callable[[str], None]] = None,
+) -> Dict[str, torch.Tensor]:
+    """Read ``wanted`` from the folder onto ``device``; see the module text for
+    the precision rule and the error."""
+    entries = index_folder(model_dir)
+    check_against(entries, wanted, model_dir)
+    out: Dict[str, torch.Tensor] = {}
+    for i, (name, spec) in enumerate(wanted.items()):
+        e = entries[name]
+        t = read_tensor(e)
+        dt = target_dtype(e.dtype, spec.kind, engine_dtype)
+        out[name] = t.to(device=device, dtype=dt).contiguous()
+        if progress is not None and i % 32 == 0:
+            progress(f"loaded {i + 1}/{len(wanted)} tensors")
+    return out
