@@ -1,0 +1,138 @@
+"""The engine against the plain implementation under every way of cutting the work.
+
+The same test bodies run twice: with the plain PyTorch kernels on the CPU (this checks
+the host side: batching, paging, the order of parts) and, marked ``gpu``, with the HIP
+kernels in true float32 and in bfloat16.
+"""
+import pytest
+import torch
+
+import plain_llama as P
+import replay_cases as C
+from kernel_refs import RefOps
+from tiny_configs import ALL
+
+BACKENDS = [
+    pytest.param(("cpu", "float32"), id="cpu-ref-f32"),
+    pytest.param(("cuda:0", "float32"), id="hip-f32", marks=pytest.mark.gpu),
+    pytest.param(("cuda:0", "bfloat16"), id="hip-bf16", marks=pytest.mark.gpu),
+]
+
+# prompt lengths of the brief's two tiny configurations, and own ones for C and D
+LENGTHS = {"A": [5, 17, 32, 61, 77, 40], "B": [1, 40, 130, 66, 25, 90], "C": [50, 3, 97, 140, 64, 31], "D": [33, 129, 70, 2, 65]}
+PAGE = {"A": 16, "B": 32, "C": 16, "D": 64}
+
+_ops_cache = {}
+
+
+def ops_for(device):
+    if device == "cpu":
+        return RefOps()
+    if device not in _ops_cache:
+        from yalis_amd.ops.hip import HipOps
+
+        _ops_cache[device] = HipOps(device)
+    return _ops_cache[device]
+
+
+_plain_cache = {}
+
+
+def setup(name, dtype):
+    cfg = ALL[name]
+    weights = P.random_weights(cfg, seed={"A": 0, "B": 1, "C": 2, "D": 3}[name])
+    reqs = C.make_requests(cfg, LENGTHS[name], seed=10)
+    key = (name, dtype == "bfloat16")
+    if key not in _plain_cache:
+        _plain_cache[key] = C.plain_logits(cfg, weights, reqs, dtype == "bfloat16")
+    return cfg, weights, reqs, _plain_cache[key]
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
+def test_replay_modes(backend, name, mode):
+    device, dtype = backend
+    cfg, weights, reqs, want = setup(name, dtype)
+    steps = {"whole": C.trace_whole, "tail": C.trace_tail, "portions": C.trace_portions, "mixed": C.trace_mixed}[mode](reqs)
+    page = PAGE[name]
+    n_pages = C.pages_needed(steps, reqs, page)
+    runner = C.make_runner(cfg, weights, dtype, device, ops_for(device), page, n_pages)
+    got, rp = C.run_trace(runner, steps)
+    C.assert_matches(got, want, dtype == "bfloat16", f"{name}/{mode}")
+    runner.pages.audit()
+    assert runner.pages.live_requests() == 0
+    assert runner.pages.free_pages(0) == n_pages
+    if mode == "mixed":
+        # the pool is so small that a later request got pages an earlier one gave back
+        first_owner = {}
+        reused = False
+        for held in rp.page_log:
+            for rid, pages in held.items():
+                for p in pages:
+                    if p in first_owner and first_owner[p] != rid:
+                        reused = True
+                    first_owner.setdefault(p, rid)
+        assert reused, "the trace was meant to reuse pages"
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_readmission_reproduces(backend):
+    """Release a request half way (as a preemption does) and replay it from the start:
+    the same logits, from other pages."""
+    device, dtype = backend
+    cfg, weights, reqs, want = setup("A", dtype)
+    toks = reqs["r3"]
+    runner = C.make_runner(cfg, weights, dtype, device, ops_for(device), 16, 6)
+    steps = [
+        {"step": 0, "entries": [{"id": "x", "tokens": toks[:20], "want": []}], "end": ["x"]},
+        {"step": 1, "entries": [{"id": "y", "tokens": reqs["r1"], "want": []}], "end": []},
+        {"step": 2, "entries": [{"id": "x", "tokens": toks[:33], "want": list(range(33))}], "end": []},
+        {"step": 3, "entries": [{"id": "x", "tokens": toks[33:], "want": list(range(len(toks) - 33))}], "end": ["x", "y"]},
+    ]
+    got, _ = C.run_trace(runner, steps)
+    C.assert_matches({"r3": got["x"]}, {"r3": want["r3"]}, dtype == "bfloat16", "readmission")
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_long_decode(backend):
+    """A short prompt, then a long run of single tokens across several pages."""
+    device, dtype = backend
+    cfg = ALL["B"]
+    weights = P.random_weights(cfg, seed=1)
+    toks = C.make_requests(cfg, [200], seed=5)["r0"]
+    want = C.plain_logits(cfg, weights, {"r0": toks}, dtype == "bfloat16")
+    steps = C.trace_tail({"r0": toks}, tail=190)
+    runner = C.make_runner(cfg, weights, dtype, device, ops_for(device), 32, 7)
+    got, _ = C.run_trace(runner, steps)
+    C.assert_matches(got, want, dtype == "bfloat16", "long decode")
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_first_tokens(backend):
+    """The first positions of a sequence, one token at a time from position 0."""
+    device, dtype = backend
+    cfg, weights, reqs, want = setup("C", dtype)
+    toks = reqs["r0"][:6]
+    steps = [{"step": i, "entries": [{"id": "a", "tokens": [t], "want": [0]}], "end": []} for i, t in enumerate(toks)]
+    runner = C.make_runner(cfg, weights, dtype, device, ops_for(device), 16, 2)
+    got, _ = C.run_trace(runner, steps)
+    C.assert_matches({"r0": got["a"]}, {"r0": want["r0"][:6]}, dtype == "bfloat16", "first tokens")
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_far_key_across_pages(backend):
+    """Random weights give flat attention, which would hide a lost far key.  Here the
+    last token equals an early one and the query/key projections of one head are scaled
+    up, so that head looks hundreds of tokens back."""
+    device, dtype = backend
+    cfg = ALL["C"]
+    weights = P.random_weights(cfg, seed=2)
+    for n in ("q_proj", "k_proj"):
+        weights[f"model.layers.0.self_attn.{n}.weight"][:64] *= 30.0
+    toks = C.make_requests(cfg, [300], seed=6)["r0"]
+    toks[-1] = toks[3]
+    want = C.plain_logits(cfg, weights, {"r0": toks}, dtype == "bfloat16")
+    runner = C.make_runner(cfg, weights, dtype, device, ops_for(device), 16, 19)
+    got, _ = C.run_trace(runner, C.trace_tail({"r0": toks}, tail=8))
+    C.assert_matches(got, want, dtype == "bfloat16", "far key")
