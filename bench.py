@@ -1,0 +1,199 @@
+"""The headline measurement: decode tokens per second of a Llama-3-8B-shaped model with
+random bfloat16 weights on one MI355X, batch 8 after 1,024-token prompts, beside the
+prefill rate at 2,048 tokens, decode at batch 1 and 64, and how far the decode step is
+from the memory roofline.  The metric follows the reference's definitions (throughput =
+batch x tokens / time, TBT = mean time of a decode step: yalis/engine.py:531-557).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L]
+
+A step is one decode step through the engine's own path: page reservation, the step
+function over the paged cache, greedy sampling, the token back on the host.
+"""
+import argparse
+import json
+import sys
+import time
+
+HBM_GBPS = 8000.0  # MI355X published peaks
+BF16_FLOPS = 2.5e15
+
+LLAMA3_8B = {
+    "architectures": ["LlamaForCausalLM"],
+    "hidden_size": 4096,
+    "num_hidden_layers": 32,
+    "num_attention_heads": 32,
+    "num_key_value_heads": 8,
+    "head_dim": 128,
+    "intermediate_size": 14336,
+    "vocab_size": 128256,
+    "rms_norm_eps": 1e-5,
+    "rope_theta": 500000.0,
+    "rope_scaling": None,
+    "max_position_embeddings": 8192,
+    "tie_word_embeddings": False,
+}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=32)
+    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (both numbers are reported)")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=1024)
+    ap.add_argument("--prefill-len", type=int, default=2048)
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
+        return 2
+
+    import torch
+
+    from yalis_amd.config.runtime import EngineConfig
+    from yalis_amd.engine.factory import random_runner
+    from yalis_amd.engine.step import StepEntry
+
+    cfg = dict(LLAMA3_8B)
+    full_layers = cfg["num_hidden_layers"]
+    if args.layers is not None:
+        cfg["num_hidden_layers"] = args.layers
+    layers = cfg["num_hidden_layers"]
+    page = 64
+    max_batch = max(args.batch, 1 if args.no_points else 64)
+    total_steps = args.steps + args.warmup + 8
+    ctx_cap = max(args.prompt_len + total_steps + 1, args.prefill_len)
+    pages_per_req = -(-ctx_cap // page)
+    engine = EngineConfig(
+        page_size=page,
+        num_pages=pages_per_req * max_batch,
+        max_num_seqs=max_batch,
+        max_model_len=min(cfg["max_position_embeddings"], pages_per_req * page),
+        max_num_batched_tokens=8192,
+        dtype="bfloat16",
+    )
+    runner = random_runner(cfg, engine, seed=0)
+    ops = runner.rt.ops
+    vocab = cfg["vocab_size"]
+    gen = torch.Generator().manual_seed(0)
+
+    def decode_run(batch: int, steps: int, warmup: int):
+        """Prefill ``batch`` prompts, then time ``steps`` decode steps."""
+        for r in range(batch):
+            assert runner.admit(r)
+            prompt = torch.randint(0, vocab, (args.prompt_len,), generator=gen).tolist()
+            assert runner.reserve(r, len(prompt))
+            logits = runner.step([StepEntry(r, prompt, [len(prompt) - 1])])
+            first = ops.argmax(logits).tolist()
+            if r == 0:
+                toks = []
+            toks.append(first[0])
+
+        def one_step(toks):
+            for r in range(batch):
+                assert runner.reserve(r, 1)
+            logits = runner.step([StepEntry(r, [toks[r]], [0]) for r in range(batch)])
+            return ops.argmax(logits).tolist()
+
+        for _ in range(warmup):
+            toks = one_step(toks)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ctx_sum = 0
+        for _ in range(steps):
+            ctx_sum += sum(runner.cached[r] + 1 for r in range(batch))
+            toks = one_step(toks)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        for r in range(batch):
+            runner.release(r)
+        return dt, ctx_sum / steps  # seconds, mean cached tokens read per step
+
+    c, h, g, d, inter = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["intermediate_size"]
+    layer_params = c * (h + 2 * g) * d + h * d * c + 3 * c * inter
+    weight_bytes = 2 * (layers * (layer_params + 2 * c) + c + vocab * c)
+
+    def step_bytes(batch, mean_ctx_tokens):
+        kv = mean_ctx_tokens * layers * 2 * g * d * 2
+        return weight_bytes + batch * c * 2 + kv
+
+    dt, mean_ctx = decode_run(args.batch, args.steps, args.warmup)
+    ms_per_step = 1e3 * dt / args.steps
+    value = args.batch * args.steps / dt
+    achieved = step_bytes(args.batch, mean_ctx) / (dt / args.steps) / 1e9
+
+    result = {
+        "metric": "decode tok/s (Llama-3-8B shape, batch 8, 1,024-token prompts)",
+        "value": round(value, 2),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic: random N(0,0.02) bf16 weights, seeded uniform-random token ids",
+        "config": {
+            "model": "Llama-3-8B shape",
+            "layers": layers,
+            "layers_of_full_model": full_layers,
+            "hidden_size": c,
+            "num_attention_heads": h,
+            "num_key_value_heads": g,
+            "head_dim": d,
+            "intermediate_size": inter,
+            "vocab_size": vocab,
+            "global_batch": args.batch,
+            "seq_len": args.prompt_len,
+            "context": cfg["max_position_embeddings"],
+            "page_size": page,
+            "parallelism": "single GPU",
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": HBM_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_GBPS, 4),
+        },
+    }
+
+    if not args.no_points:
+        # prefill of one request of 2,048 tokens, whole
+        t = args.prefill_len
+        prompt = torch.randint(0, vocab, (t,), generator=gen).tolist()
+        times = []
+        for i in range(3):
+            assert runner.admit(1000 + i)
+            assert runner.reserve(1000 + i, t)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            logits = runner.step([StepEntry(1000 + i, prompt, [t - 1])])
+            ops.argmax(logits).tolist()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            runner.release(1000 + i)
+        pf = min(times[1:])
+        flops = layers * (2 * t * layer_params + 2 * h * d * t * t) + 2 * vocab * c
+        result["prefill"] = {
+            "value": round(t / pf, 1),
+            "tokens": t,
+            "ms": round(1e3 * pf, 3),
+            "frac": round(flops / pf / BF16_FLOPS, 4),
+        }
+        points = {}
+        for b, name in ((1, "decode_b1"), (64, "decode_b64")):
+            steps = max(8, args.steps // 2)
+            dtb, _ = decode_run(b, steps, 2)
+            points[name] = round(b * steps / dtb, 2)
+        result["points"] = points
+
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

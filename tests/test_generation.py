@@ -1,0 +1,149 @@
+"""Generation through the Python entry point and the scheduler, against the plain
+implementation's whole-sequence recomputation: greedy and seeded temperature sampling,
+under token budgets and page counts that force portions and preemption.
+"""
+import json
+import os
+
+import pytest
+import torch
+
+import plain_llama as P
+from kernel_refs import RefOps
+from tiny_configs import ALL
+from yalis_amd import EngineConfig, InferenceConfig, LLMEngine, ModelConfig
+from yalis_amd.weights.safetensors_io import write_dict
+
+BACKENDS = [
+    pytest.param(("cpu", "fp32"), id="cpu-ref-f32"),
+    pytest.param(("cuda:0", "fp32"), id="hip-f32", marks=pytest.mark.gpu),
+    pytest.param(("cuda:0", "bf16"), id="hip-bf16", marks=pytest.mark.gpu),
+]
+
+
+def write_model(folder, cfg, weights, dtype):
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    write_dict(os.path.join(folder, "model.safetensors"), {k: v.to(dtype).contiguous() for k, v in weights.items()})
+    return str(folder)
+
+
+def make_engine(tmp_path, name, backend, max_batch, temperature, top_k=None, top_p=1.0, **engine_kw):
+    device, precision = backend
+    cfg = ALL[name]
+    weights = P.random_weights(cfg, seed=7)
+    dtype = torch.float32 if precision == "fp32" else torch.bfloat16
+    folder = write_model(tmp_path / name, cfg, weights, dtype)
+    if precision == "bf16":
+        weights = {k: v.to(torch.bfloat16).float() for k, v in weights.items()}
+    ec = EngineConfig(max_num_seqs=max_batch, max_model_len=cfg["max_position_embeddings"],
+                      dtype="float32" if precision == "fp32" else "bfloat16", device=device, **engine_kw)
+    eng = LLMEngine(
+        ModelConfig(model_path=folder, precision=precision),
+        InferenceConfig(max_batch_size=max_batch, max_length_of_generated_sequences=cfg["max_position_embeddings"],
+                        temperature=temperature, top_k=top_k, top_p=top_p, seed=5),
+        device=device, engine_config=ec, ops=RefOps() if device == "cpu" else None,
+    )
+    return eng, cfg, weights
+
+
+def prompts_for(cfg, lengths, seed=3):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in lengths]
+
+
+def margin_ok(cfg, weights, prompt, out, rounder=P._identity):
+    """Greedy tokens are only comparable where the plain logits have a clear winner:
+    a gap between the two largest of more than twice the bfloat16 logit tolerance
+    (tests/replay_cases.py: 4 * 2^-8 of the logits' scale)."""
+    toks = list(prompt)
+    for t in out:
+        logits = P.forward(cfg, weights, toks, rounder)[-1]
+        top2 = torch.topk(logits, 2).values
+        if (top2[0] - top2[1]).item() < 2 * 4 * 2.0**-8 * logits.abs().max().item():
+            return False
+        toks.append(t)
+    return True
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("engine_kw", [
+    dict(page_size=16, num_pages=64, max_num_batched_tokens=2048),
+    dict(page_size=16, num_pages=9, max_num_batched_tokens=24),   # portions and preemption
+])
+def test_greedy_matches_plain(tmp_path, backend, engine_kw):
+    """Tiny A, prompts of 5/17/32/61 tokens, 16 greedy tokens each."""
+    eng, cfg, weights = make_engine(tmp_path, "A", backend, 4, temperature=0.0, **engine_kw)
+    prompts = prompts_for(cfg, [5, 17, 32, 61])
+    out, metrics = eng.generate(prompts, tokens_to_generate=16)
+    assert out.shape == (4, 16)
+    bf16 = backend[1] == "bf16"
+    for p, row in zip(prompts, out.tolist()):
+        want = P.greedy_generate(cfg, weights, p, 16, P.bf16_round if bf16 else P._identity)
+        if bf16:
+            # rounding may flip a near-tie; compare up to the first token whose plain
+            # logits have no clear winner
+            k = 0
+            while k < 16 and row[k] == want[k]:
+                k += 1
+            assert k == 16 or not margin_ok(cfg, weights, p, want[: k + 1], P.bf16_round), (row, want)
+        else:
+            assert row == want
+    assert metrics["BatchSize"] == 4 and metrics["DecodeLength"] == 16
+    if engine_kw["num_pages"] == 9:
+        assert metrics["Preemptions"] > 0, "this pool was meant to force a preemption"
+    eng.runner.pages.audit()
+    assert eng.runner.pages.live_requests() == 0
+
+
+@pytest.mark.parametrize("backend", BACKENDS[:2])
+def test_temperature_sampling_matches_plain(tmp_path, backend):
+    """Tiny B, prompts of 1/40/130 tokens, temperature 0.7, 24 tokens, page size 32: the
+    engine's per-request uniforms are a documented function of (seed, draw), so the
+    plain implementation reproduces the draws."""
+    eng, cfg, weights = make_engine(tmp_path, "B", backend, 3, temperature=0.7, page_size=32, num_pages=16, max_num_batched_tokens=64)
+    prompts = prompts_for(cfg, [1, 40, 130])
+    out, _ = eng.generate(prompts, tokens_to_generate=24)
+    for i, (p, row) in enumerate(zip(prompts, out.tolist())):
+        seed = (5 * 1000003 + i) & 0x7FFFFFFF
+        want = P.sampled_generate(cfg, weights, p, 24, 0.7, None, 1.0, seed)
+        assert row == want
+
+
+@pytest.mark.parametrize("backend", BACKENDS[:2])
+def test_top_k_top_p_sampling(tmp_path, backend):
+    eng, cfg, weights = make_engine(tmp_path, "A", backend, 2, temperature=1.2, top_k=20, top_p=0.8, page_size=16, num_pages=16)
+    prompts = prompts_for(cfg, [9, 30])
+    out, _ = eng.generate(prompts, tokens_to_generate=12)
+    for i, (p, row) in enumerate(zip(prompts, out.tolist())):
+        seed = (5 * 1000003 + i) & 0x7FFFFFFF
+        assert row == P.sampled_generate(cfg, weights, p, 12, 1.2, 20, 0.8, seed)
+
+
+@pytest.mark.parametrize("backend", BACKENDS[:2])
+def test_get_logits_and_eos(tmp_path, backend):
+    eng, cfg, weights = make_engine(tmp_path, "A", backend, 2, temperature=0.0, page_size=16, num_pages=16)
+    prompts = prompts_for(cfg, [12, 20])
+    out, metrics, logits = eng.generate(prompts, tokens_to_generate=6, get_logits=True)
+    assert len(logits) == 6 and logits[0].shape == (2, cfg["vocab_size"])
+    want = P.forward(cfg, weights, prompts[0])[-1]
+    assert (logits[0][0].cpu() - want).abs().max() < 2e-5
+    # make the second generated token of request 0 the EOS: it stops there, padded with EOS
+    eng.eos_token_ids = (int(out[0, 1]),)
+    out2, metrics2 = eng.generate(prompts, tokens_to_generate=6, ignore_eos=False)
+    first = out[0].tolist().index(int(out[0, 1]))
+    assert out2[0, : first + 1].tolist() == out[0, : first + 1].tolist()
+    assert all(t == eng.eos_token_ids[0] for t in out2[0, first + 1 :].tolist())
+
+
+def test_engine_refuses_what_it_cannot_run(tmp_path):
+    eng, cfg, _ = make_engine(tmp_path, "A", ("cpu", "fp32"), 2, temperature=0.0, page_size=16, num_pages=4)
+    with pytest.raises(ValueError, match="max_batch_size"):
+        eng.generate(prompts_for(cfg, [3, 3, 3]), tokens_to_generate=2)
+    with pytest.raises(ValueError, match="leaves no room"):
+        eng.generate(prompts_for(cfg, [128]), tokens_to_generate=2)
+    with pytest.raises(ValueError, match="whole pool"):
+        eng.generate(prompts_for(cfg, [60]), tokens_to_generate=30)
+    with pytest.raises(ValueError, match="tokenizer"):
+        eng.generate(["text"], tokens_to_generate=2)

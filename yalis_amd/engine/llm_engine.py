@@ -1,0 +1,198 @@
+"""The Python entry point, in the manner of the reference's ``LLMEngine``
+(yalis/engine.py:168-573): built from a ``ModelConfig`` and an ``InferenceConfig``,
+``generate(prompts, tokens_to_generate, ...)`` returns the generated tokens and the
+reference's metrics dictionary.  Underneath, requests go through the scheduler and the
+paged step function instead of one static batch.
+"""
+from __future__ import annotations
+
+import os
+import time
+from typing import Dict, List, Optional, Sequence, Union
+
+import torch
+
+from ..config.reader import read_config_json
+from ..config.runtime import EngineConfig, InferenceConfig, ModelConfig
+from ..sampling.sampler import Sampler, SamplingParams
+from .factory import load_runner, random_runner
+from .scheduler import Request, Scheduler
+
+
+def print_rank0(*args, **kwargs) -> None:
+    """The reference prints from rank 0 only (yalis/utils.py); one process here."""
+    print(*args, **kwargs)
+
+
+class LLMEngine:
+    def __init__(
+        self,
+        model_config: ModelConfig,
+        inference_config: InferenceConfig,
+        device: str = "cuda",
+        engine_config: Optional[EngineConfig] = None,
+        random_weights_seed: Optional[int] = None,
+        ops=None,
+    ):
+        """``engine_config`` sizes the paged engine; by default it is derived from the
+        inference configuration: ``max_batch_size`` live requests of
+        ``max_length_of_generated_sequences`` tokens each (the reference's meaning of
+        that option: the longest sequence, prompt included, yalis/engine.py:353-368).
+        ``random_weights_seed``: ignore the folder's weights and make random ones
+        (config.json is still read)."""
+        self.model_config = model_config
+        self.inference_config = inference_config
+        dev = "cuda:0" if device == "cuda" else device
+        raw = read_config_json(model_config.model_path)
+        if engine_config is None:
+            max_len = min(inference_config.max_length, int(raw.get("max_position_embeddings", inference_config.max_length)))
+            engine_config = EngineConfig(
+                max_num_seqs=inference_config.max_batch_size,
+                max_model_len=max_len,
+                max_num_batched_tokens=max(2048, inference_config.max_batch_size),
+                dtype=model_config.dtype,
+                device=dev,
+            )
+        self.engine_config = engine_config
+        if random_weights_seed is None:
+            self.runner = load_runner(model_config.model_path, engine_config, ops=ops)
+        else:
+            self.runner = random_runner(raw, engine_config, random_weights_seed, ops=ops)
+        self.model = self.runner.model
+        self.sampler = Sampler(self.runner.rt.ops, engine_config.device)
+        self.eos_token_ids = tuple(self.model.spec.eos_token_ids)
+        self.tokenizer = self._load_tokenizer(model_config.model_path)
+        self.last_scheduler: Optional[Scheduler] = None
+
+    # --------------------------------------------------------------- tokenizer
+    @staticmethod
+    def _load_tokenizer(path: str):
+        """A tokenizer when the folder has one (the reference always loads one,
+        yalis/engine.py:263); token-id prompts work without."""
+        if not any(os.path.exists(os.path.join(path, f)) for f in ("tokenizer.json", "tokenizer.model")):
+            return None
+        try:
+            from transformers import AutoTokenizer
+
+            return AutoTokenizer.from_pretrained(path)
+        except Exception as e:  # noqa: BLE001 - a missing tokenizer only disables text prompts
+            print_rank0(f"[yalis_amd] tokenizer in {path} could not be loaded ({e}); give token ids")
+            return None
+
+    def _tokenize_prompts(self, prompts) -> List[List[int]]:
+        """yalis/engine.py:306-341: strings are tokenized, lists of ids pass through."""
+        if len(prompts) == 0:
+            raise ValueError("no prompts")
+        if isinstance(prompts[0], str):
+            if self.tokenizer is None:
+                raise ValueError("text prompts need a tokenizer in the model folder; give lists of token ids instead")
+            return [self.tokenizer(p)["input_ids"] for p in prompts]
+        return [[int(t) for t in p] for p in prompts]
+
+    # ----------------------------------------------------------------- generate
+    @torch.inference_mode()
+    def generate(
+        self,
+        prompts: Union[Sequence[str], Sequence[Sequence[int]]],
+        tokens_to_generate: int = 50,
+        report_throughput: bool = False,
+        ignore_eos: Optional[bool] = True,
+        enable_nvtx: Optional[bool] = False,
+        get_logits: Optional[bool] = False,
+    ):
+        """Generate ``tokens_to_generate`` tokens for every prompt.
+
+        Returns ``(tokens [batch, n] int64, metrics)`` and, with ``get_logits``, a
+        list of n float32 tensors [batch, vocab] as well (yalis/engine.py:371-409,
+        570-573).  Rows that stop early at EOS are padded with EOS, as the reference
+        keeps finished rows at EOS (:515-516).  ``enable_nvtx`` is accepted and
+        ignored (no range markers here)."""
+        t_tok = time.perf_counter()
+        ids = self._tokenize_prompts(prompts)
+        tokenize_ms = (time.perf_counter() - t_tok) * 1e3
+        ic = self.inference_config
+        if len(ids) > ic.max_batch_size:
+            # yalis/engine.py:347-352
+            raise ValueError(f"Batch size {len(ids)} exceeds max_batch_size {ic.max_batch_size}")
+        sched = Scheduler(self.runner, self.eos_token_ids)
+        self.last_scheduler = sched
+        reqs: List[Request] = []
+        for i, p in enumerate(ids):
+            params = SamplingParams(
+                temperature=ic.temperature,
+                top_k=ic.top_k,
+                top_p=ic.top_p,
+                max_tokens=tokens_to_generate,
+                ignore_eos=bool(ignore_eos),
+                seed=(ic.seed * 1000003 + i) & 0x7FFFFFFF,
+            )
+            reqs.append(sched.add(p, params))
+
+        cuda = torch.cuda.is_available() and self.engine_config.device.startswith("cuda")
+        sync = torch.cuda.synchronize if cuda else (lambda: None)
+        sync()
+        t0 = time.perf_counter()
+        first_token_at: Dict[int, float] = {}
+        decode_steps = 0
+        decode_time = 0.0
+        while sched.has_work():
+            t_step = time.perf_counter()
+            plan = sched.schedule()
+            if not plan:
+                raise RuntimeError("the scheduler made no progress (pool too small for any request?)")
+            logits = self.runner.step(sched.entries(plan))
+            sampling = [s.request for s in plan if s.samples]
+            toks = self.sampler.sample(logits, [r.params for r in sampling], [len(r.output) for r in sampling])
+            if get_logits:
+                for r, row in zip(sampling, logits):
+                    r.logits.append(row.clone())
+            sched.update(plan, toks)
+            now = time.perf_counter()
+            for r in sampling:
+                first_token_at.setdefault(r.rid, now)
+            if all(s.n_tokens == 1 and s.samples for s in plan):
+                decode_steps += 1
+                decode_time += now - t_step
+        sync()
+        total = time.perf_counter() - t0
+
+        n = max(len(r.output) for r in reqs)
+        pad = self.eos_token_ids[0] if self.eos_token_ids else 0
+        out = torch.full((len(reqs), n), pad, dtype=torch.int64)
+        for i, r in enumerate(reqs):
+            out[i, : len(r.output)] = torch.tensor(r.output, dtype=torch.int64)
+        reasons = {r.finish_reason for r in reqs}
+        metrics = {
+            "BatchSize": len(reqs),
+            "PromptLength": max(len(p) for p in ids),
+            "DecodeLength": n,
+            "Throughput": sum(len(r.output) for r in reqs) / total if total > 0 else 0.0,
+            "TTFT": 1e3 * (max(first_token_at.values()) - t0) if first_token_at else 0.0,
+            "TBT": 1e3 * decode_time / decode_steps if decode_steps else 0.0,
+            "E2E": 1e3 * total,
+            "TokenizationTime": tokenize_ms,
+            "FinishedReason": "EOS" if reasons == {"EOS"} else "Max Token Length",
+            "Preemptions": sched.n_preemptions,
+        }
+        if report_throughput:
+            # the line of yalis/engine.py:558-568
+            print_rank0(
+                f"[Metrics] BatchSize = {metrics['BatchSize']}, PromptLength = {metrics['PromptLength']},"
+                f" DecodeLength = {n}, Throughput = {metrics['Throughput']:.2f} tok/s,"
+                f" TTFT = {metrics['TTFT']:.4f} ms, TBT = {metrics['TBT']:.4f} ms,"
+                f" E2E = {metrics['E2E']:.4f} ms, FinishedReason = {metrics['FinishedReason']}"
+            )
+        if get_logits:
+            vocab = self.model.spec.vocab_size
+            steps = []
+            for j in range(n):
+                rows = [r.logits[j] if j < len(r.logits) else torch.zeros(vocab, device=r.logits[0].device) for r in reqs]
+                steps.append(torch.stack(rows))
+            return out, metrics, steps
+        return out, metrics
+
+    def reset_kv_cache(self, max_batch_size: Optional[int] = None) -> None:
+        """yalis/engine.py:280-304 rebuilds the caches; pages here are given back when
+        requests end, so there is nothing to rebuild unless the batch limit changes."""
+        if max_batch_size is not None and max_batch_size != self.inference_config.max_batch_size:
+            raise ValueError("the number of live requests is fixed when the engine is built")

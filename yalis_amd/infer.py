@@ -1,0 +1,110 @@
+"""Command line in the manner of the reference's examples/infer.py (a script with its
+settings at the top: model, prompts, tokens to generate, max batch size, precision,
+top_p, temperature, ten timed ``generate`` calls, then the outputs; :13-124).  The same
+settings are options here, under the reference's names.
+
+    python -m yalis_amd.infer --model DIR --prompt-ids 1,2,3 --prompt-ids 4,5 \\
+        --tokens-to-generate 32 --temperature 0 --precision bf16
+"""
+from __future__ import annotations
+
+import argparse
+import sys
+from typing import List
+
+import torch
+
+DEFAULT_PROMPTS = [
+    "How to bake a cake?",
+    "Explain quantum mechanics in simple terms.",
+    "What are the benefits of a balanced diet?",
+    "How can I learn to play the guitar?",
+]
+
+
+def parse_args(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--model", "--model-path", dest="model_path", required=True, help="folder with config.json, model.safetensors (and a tokenizer for text prompts)")
+    ap.add_argument("--model-name", default=None)
+    ap.add_argument("--precision", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--prompt", action="append", default=[], help="a text prompt (repeatable; needs a tokenizer)")
+    ap.add_argument("--prompt-ids", action="append", default=[], help="a prompt as comma-separated token ids (repeatable)")
+    ap.add_argument("--random-prompts", default=None, metavar="N,LEN", help="N prompts of LEN seeded random token ids")
+    ap.add_argument("--tokens-to-generate", type=int, default=50)
+    ap.add_argument("--max-batch-size", type=int, default=32)
+    ap.add_argument("--max-length-of-generated-sequences", type=int, default=1024)
+    ap.add_argument("--temperature", type=float, default=1.0)
+    ap.add_argument("--top-k", type=int, default=None)
+    ap.add_argument("--top-p", type=float, default=0.80)
+    ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--iters", type=int, default=1, help="timed generate calls (the reference script runs 10)")
+    ap.add_argument("--no-ignore-eos", action="store_true", help="stop a request at its EOS token")
+    ap.add_argument("--report-throughput", action="store_true")
+    ap.add_argument("--random-weights-seed", type=int, default=None, help="ignore the folder's weights; random ones from this seed")
+    ap.add_argument("--page-size", type=int, default=64)
+    ap.add_argument("--num-pages", type=int, default=None)
+    ap.add_argument("--max-num-batched-tokens", type=int, default=2048)
+    return ap.parse_args(argv)
+
+
+def main(argv=None) -> int:
+    args = parse_args(argv)
+    from yalis_amd import InferenceConfig, LLMEngine, ModelConfig, print_rank0
+    from yalis_amd.config.reader import read_config_json
+    from yalis_amd.config.runtime import EngineConfig
+
+    model_config = ModelConfig(model_name=args.model_name, model_path=args.model_path, precision=args.precision)
+    inference_config = InferenceConfig(
+        max_batch_size=args.max_batch_size,
+        max_length_of_generated_sequences=args.max_length_of_generated_sequences,
+        top_k=args.top_k,
+        top_p=args.top_p,
+        temperature=args.temperature,
+        seed=args.seed,
+    )
+    raw = read_config_json(args.model_path)
+    engine_config = EngineConfig(
+        page_size=args.page_size,
+        num_pages=args.num_pages,
+        max_num_seqs=args.max_batch_size,
+        max_model_len=min(args.max_length_of_generated_sequences, int(raw.get("max_position_embeddings", 1 << 30))),
+        max_num_batched_tokens=args.max_num_batched_tokens,
+        dtype=model_config.dtype,
+    )
+    engine = LLMEngine(model_config, inference_config, engine_config=engine_config, random_weights_seed=args.random_weights_seed)
+
+    prompts: List = []
+    if args.prompt_ids:
+        prompts = [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids]
+    elif args.random_prompts:
+        n, length = (int(x) for x in args.random_prompts.split(","))
+        g = torch.Generator().manual_seed(args.seed)
+        vocab = engine.model.spec.vocab_size
+        prompts = [torch.randint(0, vocab, (length,), generator=g).tolist() for _ in range(n)]
+    elif args.prompt:
+        prompts = list(args.prompt)
+    else:
+        prompts = DEFAULT_PROMPTS[: args.max_batch_size]
+    print_rank0(f"Number of prompts = {len(prompts)}")
+
+    for _ in range(args.iters):
+        output_tokens, metrics = engine.generate(
+            prompts,
+            tokens_to_generate=args.tokens_to_generate,
+            report_throughput=True if args.iters > 1 else args.report_throughput,
+            ignore_eos=not args.no_ignore_eos,
+        )
+    texts = None
+    if engine.tokenizer is not None:
+        texts = engine.tokenizer.batch_decode(output_tokens, skip_special_tokens=True)
+    for i, prompt in enumerate(prompts):
+        print_rank0("==========================\n")
+        print_rank0(f"prompt = {prompt}")
+        print_rank0(f"output = {texts[i] if texts is not None else output_tokens[i].tolist()}")
+    print_rank0("==========================\n")
+    print_rank0(f"metrics = {metrics}")
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
