@@ -1,0 +1,193 @@
+"""Configuration, registry, weights: reading, errors, the random-weights folder."""
+import json
+import os
+import warnings
+
+import pytest
+import torch
+
+from tiny_configs import ALL, TINY_A, TINY_B
+from yalis_amd.config.reader import ConfigError
+from yalis_amd.config.registry import get_architecture, known_architectures, load_model_config
+from yalis_amd.config.runtime import EngineConfig, InferenceConfig, ModelConfig
+from yalis_amd.engine.factory import spec_from_config, tensor_specs_for
+from yalis_amd.models.llama import LlamaConfig
+from yalis_amd.weights.loader import TensorSpec, WeightsError, load_tensors, target_dtype
+from yalis_amd.weights.random_init import write_random_model
+from yalis_amd.weights.safetensors_io import SafetensorsError, index_folder, read_tensor, write_dict
+
+
+def test_llama_config_reads_its_own_keys():
+    c = LlamaConfig.from_dict(TINY_B)
+    assert (c.hidden_size, c.num_hidden_layers, c.num_attention_heads, c.num_key_value_heads) == (128, 3, 4, 1)
+    assert (c.head_dim, c.intermediate_size, c.vocab_size) == (32, 352, 384)
+    assert c.rms_norm_eps == 1e-6 and c.rope_theta == 500000.0 and c.tie_word_embeddings
+    assert c.rope_scaling.factor == 8.0 and c.rope_scaling.original_max_position_embeddings == 64
+    # defaults: groups = heads, head_dim = hidden / heads (yalis/external/config.py:108-125)
+    d = dict(TINY_A)
+    del d["num_key_value_heads"], d["head_dim"]
+    c2 = LlamaConfig.from_dict(d)
+    assert c2.num_key_value_heads == 4 and c2.head_dim == 16
+    # round trip through its own config.json
+    assert LlamaConfig.from_dict(c.to_dict()) == c
+
+
+@pytest.mark.parametrize("change,match", [
+    ({"hidden_act": "gelu"}, "hidden_act"),
+    ({"attention_bias": True}, "attention_bias"),
+    ({"mlp_bias": True}, "mlp_bias"),
+    ({"num_key_value_heads": 3}, "multiple"),
+    ({"rope_scaling": {"rope_type": "yarn", "factor": 2.0}}, "yarn"),
+    ({"rope_scaling": {"rope_type": "llama3", "factor": 8.0}}, "low_freq_factor"),
+    ({"hidden_size": "64"}, "integer"),
+    ({"rms_norm_eps": 0}, "rms_norm_eps"),
+    ({"sliding_window": 128}, "sliding_window"),
+    ({"head_dim": 15}, "even"),
+])
+def test_llama_config_refuses(change, match):
+    with pytest.raises(ConfigError, match=match):
+        LlamaConfig.from_dict({**TINY_A, **change})
+
+
+def test_llama_config_missing_and_unknown_keys():
+    d = dict(TINY_A)
+    del d["intermediate_size"]
+    with pytest.raises(ConfigError, match="intermediate_size"):
+        LlamaConfig.from_dict(d)
+    with pytest.warns(UserWarning, match="mystery_key"):
+        LlamaConfig.from_dict({**TINY_A, "mystery_key": 1})
+    with pytest.raises(ConfigError, match="mystery_key"):
+        LlamaConfig.from_dict({**TINY_A, "mystery_key": 1}, strict=True)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        LlamaConfig.from_dict({**TINY_A, "transformers_version": "4.40", "bos_token_id": 1, "eos_token_id": [2, 3]})
+
+
+def test_registry(tmp_path):
+    assert "LlamaForCausalLM" in known_architectures()
+    with pytest.raises(ConfigError, match="unknown architecture 'NoSuchModel'.*LlamaForCausalLM"):
+        get_architecture("NoSuchModel")
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(TINY_A, f)
+    arch, cfg = load_model_config(str(tmp_path))
+    assert arch.name == "LlamaForCausalLM" and isinstance(cfg, LlamaConfig)
+    with pytest.raises(FileNotFoundError):
+        load_model_config(str(tmp_path / "nothing"))
+
+
+def test_spec_has_every_constant_as_data():
+    _, _, spec = spec_from_config(TINY_B)
+    assert len(spec.layers) == 3 and [e.layer for e in spec.run_order] == [0, 1, 2]
+    m = spec.layers[1].mixer.params
+    assert (m["num_heads"], m["num_kv_heads"], m["head_dim"], m["window"]) == (4, 1, 32, None)
+    assert abs(m["scale"] - 32**-0.5) < 1e-12
+    assert m["position"].params["theta"] == 500000.0 and m["position"].params["scaling"]["factor"] == 8.0
+    assert spec.layers[1].mixer_norm.params["eps"] == 1e-6
+    assert spec.head.params["tied_to"] == "model.embed_tokens.weight"
+
+
+def test_runtime_configs():
+    with pytest.raises(ValueError, match="Invalid precision"):
+        ModelConfig(model_path="/", precision="fp8")
+    with pytest.raises(ValueError, match="does not exist"):
+        ModelConfig(model_name="nope/none")
+    with pytest.raises(ValueError, match="Either"):
+        ModelConfig()
+    assert ModelConfig(model_path="/", precision="bf16").dtype == "bfloat16"
+    for bad in (dict(max_batch_size=0), dict(temperature=-1.0), dict(top_k=0), dict(top_p=1.5), dict(tp_dims=(2, 1, 1)), dict(attention_backend="flash")):
+        with pytest.raises(ValueError):
+            InferenceConfig(**bad)
+    ic = InferenceConfig(max_batch_size=4, top_p=0.8)
+    assert ic.max_length == 1024 and ic.temperature == 1.0 and ic.top_k is None
+    with pytest.raises(ValueError, match="multiple of 16"):
+        EngineConfig(page_size=24)
+    assert EngineConfig(page_size=64, max_num_seqs=4, max_model_len=1000).resolved_num_pages() == 64
+
+
+def test_safetensors_round_trip_and_errors(tmp_path):
+    t = {
+        "a": torch.randn(3, 5),
+        "b": torch.randn(7).to(torch.bfloat16),
+        "c": torch.arange(6, dtype=torch.int64).reshape(2, 3),
+    }
+    os.makedirs(tmp_path / "m")
+    write_dict(str(tmp_path / "m" / "model.safetensors"), t)
+    idx = index_folder(str(tmp_path / "m"))
+    for k, v in t.items():
+        assert torch.equal(read_tensor(idx[k]), v)
+    # the same file read by the safetensors package
+    from safetensors.torch import load_file
+
+    lib = load_file(str(tmp_path / "m" / "model.safetensors"))
+    assert all(torch.equal(lib[k], v) for k, v in t.items())
+    # truncated file
+    data = open(tmp_path / "m" / "model.safetensors", "rb").read()
+    os.makedirs(tmp_path / "t")
+    open(tmp_path / "t" / "model.safetensors", "wb").write(data[:-10])
+    with pytest.raises(SafetensorsError, match="truncated|beyond"):
+        index_folder(str(tmp_path / "t"))
+    with pytest.raises(FileNotFoundError):
+        index_folder(str(tmp_path / "none"))
+    # shards with an index
+    os.makedirs(tmp_path / "s")
+    write_dict(str(tmp_path / "s" / "model-00001-of-00002.safetensors"), {"a": t["a"]})
+    write_dict(str(tmp_path / "s" / "model-00002-of-00002.safetensors"), {"b": t["b"], "c": t["c"]})
+    json.dump({"weight_map": {"a": "model-00001-of-00002.safetensors", "b": "model-00002-of-00002.safetensors", "c": "model-00002-of-00002.safetensors"}},
+              open(tmp_path / "s" / "model.safetensors.index.json", "w"))
+    idx = index_folder(str(tmp_path / "s"))
+    assert torch.equal(read_tensor(idx["c"]), t["c"])
+
+
+def test_precision_rule():
+    assert target_dtype("BF16", "float", "bfloat16") == torch.bfloat16
+    assert target_dtype("F16", "float", "bfloat16") == torch.bfloat16
+    assert target_dtype("F32", "float", "bfloat16") == torch.float32, "a tensor stored in 32 bits stays so"
+    assert target_dtype("BF16", "float", "float32") == torch.float32
+    assert target_dtype("I64", "int", "bfloat16") == torch.int32
+
+
+def test_random_folder_loads_back_bit_exact(tmp_path):
+    folder = write_random_model(str(tmp_path / "b"), TINY_B, seed=1, dtype="bfloat16")
+    specs = tensor_specs_for(TINY_B)
+    assert "lm_head.weight" not in specs, "tied: the head reads the embedding table"
+    loaded = load_tensors(folder, specs, "bfloat16", "cpu")
+    again = write_random_model(str(tmp_path / "b2"), TINY_B, seed=1, dtype="bfloat16")
+    other = write_random_model(str(tmp_path / "b3"), TINY_B, seed=2, dtype="bfloat16")
+    l2 = load_tensors(again, specs, "bfloat16", "cpu")
+    l3 = load_tensors(other, specs, "bfloat16", "cpu")
+    for n, t in loaded.items():
+        assert t.dtype == torch.bfloat16 and tuple(t.shape) == specs[n].shape
+        assert torch.equal(t, l2[n]) and not torch.equal(t, l3[n])
+    w = loaded["model.layers.0.self_attn.q_proj.weight"].float()
+    assert abs(w.std().item() - 0.02) < 0.002 and abs(w.mean().item()) < 0.002
+    n = loaded["model.norm.weight"].float()
+    assert abs(n.mean().item() - 1.0) < 0.05 and 0.05 < n.std().item() < 0.15
+    # the 32-bit engine widens; a 32-bit folder stays 32-bit in a bfloat16 engine
+    assert load_tensors(folder, specs, "float32", "cpu")["model.norm.weight"].dtype == torch.float32
+    f32 = write_random_model(str(tmp_path / "a32"), TINY_A, seed=0, dtype="float32")
+    assert load_tensors(f32, tensor_specs_for(TINY_A), "bfloat16", "cpu")["model.norm.weight"].dtype == torch.float32
+    assert json.load(open(os.path.join(folder, "config.json")))["architectures"] == ["LlamaForCausalLM"]
+
+
+def test_one_error_lists_everything_wrong(tmp_path):
+    folder = write_random_model(str(tmp_path / "a"), TINY_A, seed=0, dtype="bfloat16")
+    specs = tensor_specs_for(TINY_A)
+    path = os.path.join(folder, "model.safetensors")
+    tensors = {n: read_tensor(e) for n, e in index_folder(folder).items()}
+    del tensors["model.layers.1.mlp.up_proj.weight"]
+    del tensors["lm_head.weight"]
+    tensors["model.layers.0.extra.weight"] = torch.zeros(3)
+    tensors["model.norm.weight"] = torch.zeros(65, dtype=torch.bfloat16)
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)  # harmless, ignored
+    tensors["model.layers.0.input_layernorm.weight"] = torch.zeros(64, dtype=torch.int32)
+    write_dict(path, tensors)
+    with pytest.raises(WeightsError) as e:
+        load_tensors(folder, specs, "bfloat16", "cpu")
+    err = e.value
+    assert err.missing == ["lm_head.weight", "model.layers.1.mlp.up_proj.weight"]
+    assert err.unexpected == ["model.layers.0.extra.weight"]
+    assert err.wrong_shape == [("model.norm.weight", (65,), (64,))]
+    assert err.wrong_kind[0][0] == "model.layers.0.input_layernorm.weight"
+    msg = str(err)
+    for piece in ("missing tensors (2)", "unexpected tensors (1)", "model.norm.weight has (65,), the model needs (64,)", "wrong type"):
+        assert piece in msg

@@ -1,0 +1,192 @@
+"""Pins of the plain implementation beside the reference's text: special cases that
+reduce to a library routine, and invariants, each chosen so that a plausible mistake
+(a wrong sign or pairing, a norm in the wrong place, a mask off by one) fails it.
+The reference holds no stored vectors (its tests compare with another library at run
+time, tests/basic_correctness/test_yalis_vs_hf.py:127-185), so parity with it beyond
+these pins is unpinned.
+"""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_llama as P
+from tiny_configs import ALL, TINY_A, TINY_B
+
+
+def test_rms_norm_is_the_library_routine():
+    x = torch.randn(5, 48)
+    w = 1 + 0.1 * torch.randn(48)
+    for eps in (1e-5, 1e-6):
+        assert torch.allclose(P.rms_norm(x, w, eps), F.rms_norm(x, (48,), w, eps), atol=1e-6)
+    # unit weight, no eps: rows of unit root-mean-square
+    y = P.rms_norm(x, torch.ones(48), 0.0)
+    assert torch.allclose((y * y).mean(-1), torch.ones(5), atol=1e-5)
+    # no mean subtraction: a constant row stays constant (a LayerNorm would give 0)
+    c = torch.full((1, 48), 3.0)
+    assert torch.allclose(P.rms_norm(c, torch.ones(48), 0.0), torch.ones(1, 48), atol=1e-6)
+    # eps matters for a tiny row, and is added to the mean square, not to the root
+    tiny = torch.full((1, 48), 1e-4)
+    assert abs(P.rms_norm(tiny, torch.ones(48), 1e-6)[0, 0].item() - 1e-4 / math.sqrt(1e-8 + 1e-6)) < 1e-6
+
+
+def test_rope_is_a_complex_rotation():
+    d = 32
+    x = torch.randn(7, 3, d)
+    pos = torch.tensor([0, 1, 2, 5, 11, 40, 100])
+    inv = P.rope_inv_freq(d, 10000.0, None)
+    cos, sin = P.rope_cos_sin(pos, inv)
+    y = P.apply_rope(x, cos, sin)
+    # pairs (i, i + d/2) as real and imaginary part, times e^{i p theta_i}
+    z = torch.complex(x[..., : d // 2], x[..., d // 2 :]) * torch.polar(torch.ones(7, d // 2), torch.outer(pos.float(), inv))[:, None, :]
+    assert torch.allclose(y, torch.cat([z.real, z.imag], -1), atol=1e-5)
+    assert torch.equal(y[0], x[0]), "position 0 is the identity"
+    assert torch.allclose(y.norm(dim=-1), x.norm(dim=-1), atol=1e-5), "a rotation keeps norms"
+    # first frequency is 1 (theta^0): the first pair at position 1 turns by one radian
+    e = torch.zeros(1, 1, d)
+    e[0, 0, 0] = 1.0
+    c1, s1 = P.rope_cos_sin(torch.tensor([1]), inv)
+    r = P.apply_rope(e, c1, s1)
+    assert abs(r[0, 0, 0].item() - math.cos(1.0)) < 1e-6 and abs(r[0, 0, d // 2].item() - math.sin(1.0)) < 1e-6
+
+
+def test_rope_scores_depend_on_distance_only():
+    d = 16
+    q, k = torch.randn(1, 1, d), torch.randn(1, 1, d)
+    inv = P.rope_inv_freq(d, 500000.0, TINY_B["rope_scaling"])
+
+    def score(m, n):
+        cq, sq = P.rope_cos_sin(torch.tensor([m]), inv)
+        ck, sk = P.rope_cos_sin(torch.tensor([n]), inv)
+        return (P.apply_rope(q, cq, sq) * P.apply_rope(k, ck, sk)).sum().item()
+
+    assert abs(score(9, 4) - score(25, 20)) < 1e-4
+    assert abs(score(9, 4) - score(4, 9)) > 1e-3, "direction matters"
+
+
+def test_llama3_scaling_regimes():
+    s = {"factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0, "original_max_position_embeddings": 64}
+    d, theta = 32, 500000.0
+    plain = P.rope_inv_freq(d, theta, None)
+    scaled = P.rope_inv_freq(d, theta, s)
+    wavelen = 2 * math.pi / plain
+    high = wavelen < 64 / 4.0  # short waves: unchanged
+    low = wavelen > 64 / 1.0  # long waves: divided by the factor
+    mid = ~high & ~low
+    assert high.any() and low.any() and mid.any(), "the tiny configuration is meant to reach all three regimes"
+    assert torch.allclose(scaled[high], plain[high])
+    assert torch.allclose(scaled[low], plain[low] / 8.0)
+    assert ((scaled[mid] < plain[mid]) & (scaled[mid] > plain[mid] / 8.0)).all()
+    one = dict(s, factor=1.0)
+    assert torch.allclose(P.rope_inv_freq(d, theta, one), plain), "factor 1 changes nothing"
+
+
+def test_attention_is_the_library_routine():
+    t, h, g, d = 9, 4, 2, 16
+    q, k, v = torch.randn(t, h, d), torch.randn(t, g, d), torch.randn(t, g, d)
+    got = P.causal_attention(q, k, v, 1 / math.sqrt(d))
+    want = F.scaled_dot_product_attention(
+        q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None], is_causal=True, enable_gqa=True
+    )[0].transpose(0, 1)
+    assert torch.allclose(got, want, atol=1e-5)
+    assert torch.allclose(got[0], v[0].repeat_interleave(h // g, dim=0), atol=1e-6), "the first token sees itself only"
+    # one head, no mask effect on the last row: plain softmax(q k^T / sqrt(d)) v
+    last = torch.softmax((q[-1, 0] @ k[:, 0].T) / math.sqrt(d), -1) @ v[:, 0]
+    assert torch.allclose(got[-1, 0], last, atol=1e-5)
+    # heads 0,1 read group 0 and heads 2,3 group 1 (not interleaved)
+    v2 = v.clone()
+    v2[:, 1] += 1.0
+    got2 = P.causal_attention(q, k, v2, 1 / math.sqrt(d))
+    assert torch.allclose(got2[:, :2], got[:, :2]) and torch.allclose(got2[:, 2:], got[:, 2:] + 1.0, atol=1e-5)
+
+
+def test_window_limits_what_is_seen():
+    t, d = 12, 16
+    q, k, v = torch.randn(t, 1, d), torch.randn(t, 1, d), torch.randn(t, 1, d)
+    full = P.causal_attention(q, k, v, 0.25)
+    w = P.causal_attention(q, k, v, 0.25, window=4)
+    assert torch.allclose(full[:4], w[:4], atol=1e-6)  # the first 4 positions see everything anyway
+    want = torch.softmax((q[9, 0] @ k[6:10, 0].T) * 0.25, -1) @ v[6:10, 0]
+    assert torch.allclose(w[9, 0], want, atol=1e-5)
+
+
+def test_swiglu_and_the_reference_layouts():
+    x = torch.randn(3, 24)
+    wg, wu, wd = torch.randn(40, 24), torch.randn(40, 24), torch.randn(24, 40)
+    want = (F.silu(x @ wg.T) * (x @ wu.T)) @ wd.T
+    assert torch.allclose(P.swiglu_mlp(x, wg, wu, wd), want, atol=1e-4)
+    # the reference's fused matrix interleaves gate and up rows and splits even/odd columns
+    # (yalis/external/convert_hf_checkpoint.py:833-835, yalis/external/model.py:741-743)
+    fused = torch.stack((wg, wu), dim=1).reshape(80, 24)
+    gu = x @ fused.T
+    assert torch.allclose((F.silu(gu[..., ::2]) * gu[..., 1::2]) @ wd.T, want, atol=1e-4)
+    assert torch.equal(P.swiglu_mlp(x, torch.zeros_like(wg), wu, wd), torch.zeros(3, 24)), "zero gate, zero output"
+
+
+def test_fused_qkv_layout_of_the_reference():
+    """yalis/external/model.py:544-557 views the fused projection as [G, qpk + 2, D];
+    with rows arranged as the converter does (convert_hf_checkpoint.py:1285-1302) that
+    equals three separate projections."""
+    c, h, g, d = 24, 4, 2, 8
+    qpk = h // g
+    wq, wk, wv = torch.randn(h * d, c), torch.randn(g * d, c), torch.randn(g * d, c)
+    rows = []
+    for gi in range(g):
+        rows += [wq[gi * qpk * d : (gi + 1) * qpk * d], wk[gi * d : (gi + 1) * d], wv[gi * d : (gi + 1) * d]]
+    fused = torch.cat(rows)
+    x = torch.randn(5, c)
+    qkv = (x @ fused.T).view(5, g, qpk + 2, d)
+    q, k, v = qkv.split((qpk, 1, 1), dim=2)
+    assert torch.allclose(q.reshape(5, h * d), x @ wq.T, atol=1e-5)
+    assert torch.allclose(k.reshape(5, g * d), x @ wk.T, atol=1e-5)
+    assert torch.allclose(v.reshape(5, g * d), x @ wv.T, atol=1e-5)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_model_invariants(name):
+    cfg = ALL[name]
+    w = P.random_weights(cfg, seed=0)
+    toks = torch.randint(0, cfg["vocab_size"], (20,), generator=torch.Generator().manual_seed(1)).tolist()
+    base = P.forward(cfg, w, toks)
+    assert base.shape == (20, cfg["vocab_size"])
+    # only distances count: shifting all positions changes nothing
+    assert torch.allclose(P.forward(cfg, w, toks, first_position=37), base, atol=2e-5)
+    # causality: a later token does not change earlier logits
+    other = list(toks)
+    other[12] = (other[12] + 1) % cfg["vocab_size"]
+    changed = P.forward(cfg, w, other)
+    assert torch.equal(changed[:12], base[:12]) and not torch.allclose(changed[12:], base[12:])
+    # zero layers: logits are the head applied to the normed embedding
+    emb = w["model.embed_tokens.weight"][torch.tensor(toks)]
+    head = w["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else w["lm_head.weight"]
+    want0 = P.rms_norm(emb, w["model.norm.weight"], cfg["rms_norm_eps"]) @ head.T
+    assert torch.allclose(P.forward(cfg, w, toks, n_layers=0), want0, atol=1e-6)
+    # float64 agrees: the float32 result is not an artefact of rounding
+    w64 = {k: v.double() for k, v in w.items()}
+    assert (P.forward(cfg, w64, toks, dtype=torch.float64).float() - base).abs().max() < 1e-5
+
+
+def test_sampling_rules():
+    logits = torch.tensor([2.0, 1.0, 0.5, -1.0])
+    # top_k = 1 is argmax; top-k is applied before the temperature
+    assert P.top_k_filter(logits, 1).tolist() == [2.0, float("-inf"), float("-inf"), float("-inf")]
+    assert torch.isfinite(P.top_k_filter(logits, 2)).sum() == 2
+    # top-p: the token that crosses the threshold is removed, rank 0 is always kept
+    p = torch.softmax(logits, 0)  # 0.609, 0.224, 0.136, 0.030
+    assert torch.isfinite(P.top_p_filter(logits, 0.7)).tolist() == [True, False, False, False]
+    assert torch.isfinite(P.top_p_filter(logits, 0.84)).tolist() == [True, True, False, False]
+    assert torch.isfinite(P.top_p_filter(logits, 0.0)).tolist() == [True, False, False, False]
+    assert abs(p[0] + p[1] - 0.833) < 1e-2
+    # temperature 0 is greedy; a tiny temperature makes the race pick the largest too
+    assert P.sample_token(logits, 0.0, None, 1.0, 1, 0) == 0
+    assert all(P.sample_token(logits, 1e-3, None, 1.0, 1, d) == 0 for d in range(20))
+    # the race follows softmax(logits / T)
+    counts = torch.zeros(4)
+    for d in range(4000):
+        counts[P.sample_token(logits, 1.5, None, 1.0, 3, d)] += 1
+    want = torch.softmax(logits / 1.5, 0) * 4000
+    assert (((counts - want) ** 2) / want).sum() < 25  # 3 degrees of freedom
+    u = P.race_uniforms(3, 0, 1000)
+    assert 0 < u.min() and u.max() < 1 and abs(u.mean() - 0.5) < 0.05
+    assert not (P.race_uniforms(3, 1, 1000) == u).all() and not (P.race_uniforms(4, 0, 1000) == u).all()

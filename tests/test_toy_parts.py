@@ -1,0 +1,258 @@
+"""Generality of the framework, shown with toy parts defined here, without a change to
+the framework's files: a mixer with per-request state of its own, an architecture
+registered from outside, a run order that names a layer twice and lets an entry read
+another entry's cache, and layers with a window beside layers without (two cache groups,
+pages given back while the request is live).  The toy model is nobody's architecture.
+"""
+import math
+
+import pytest
+import torch
+
+import plain_llama as P
+import replay_cases as C
+from kernel_refs import RefOps
+from yalis_amd.config.reader import KeyReader
+from yalis_amd.config.registry import register_architecture
+from yalis_amd.config.runtime import EngineConfig
+from yalis_amd.config.specs import LayerSpec, ModelSpec, PartSpec, RunEntry
+from yalis_amd.engine.factory import build_model, tensor_specs_for
+from yalis_amd.engine.step import ModelRunner
+from yalis_amd.parts import Mixer, StateNeed, register_mixer
+from yalis_amd.weights.loader import TensorSpec
+from yalis_amd.weights.random_init import random_tensors
+
+BACKENDS = [
+    pytest.param(("cpu", "float32"), id="cpu-ref-f32"),
+    pytest.param(("cuda:0", "float32"), id="hip-f32", marks=pytest.mark.gpu),
+    pytest.param(("cuda:0", "bfloat16"), id="hip-bf16", marks=pytest.mark.gpu),
+]
+
+
+# ------------------------------------------------------------------ a mixer with state
+@register_mixer("toy_running_mean")
+class RunningMean(Mixer):
+    """out[t] = W . mean(h[0..t]): needs no cache pages, only a running sum and a count
+    per request, kept in the request's state slot."""
+
+    def __init__(self, params, rt):
+        super().__init__(params, rt)
+        self.hidden = params["hidden_size"]
+        self.name = params["prefix"] + ".mix.weight"
+        self.w = None
+
+    def tensor_specs(self):
+        return {self.name: TensorSpec((self.hidden, self.hidden), "float", ("normal", 0.05))}
+
+    def load(self, tensors):
+        self.w = tensors[self.name]
+
+    def state_need(self):
+        return StateNeed((self.hidden + 1,), torch.float32)
+
+    def forward(self, h, ctx, site):
+        state = site.state()
+        out = torch.empty(h.shape, dtype=torch.float32, device=h.device)
+        for i in range(ctx.n_seqs):
+            slot = int(ctx.host.state_slots[i])
+            a = int(ctx.host.seq_qstart[i])
+            b = a + int(ctx.host.seq_qlen[i])
+            total = torch.cumsum(h[a:b].float(), 0) + state[slot, : self.hidden]
+            count = state[slot, self.hidden] + torch.arange(1, b - a + 1, device=h.device)
+            out[a:b] = total / count[:, None]
+            state[slot, : self.hidden] = total[-1]
+            state[slot, self.hidden] = count[-1]
+        return self.rt.ops.linear(out.to(self.rt.act_dtype), self.w, self.rt.act_dtype)
+
+
+# ----------------------------------------------------------------- a toy architecture
+class ToyConfig:
+    def __init__(self, raw):
+        r = KeyReader(raw)
+        self.hidden = r.integer("hidden_size")
+        self.vocab = r.integer("vocab_size")
+        self.heads = r.integer("heads")
+        self.kv_heads = r.integer("kv_heads")
+        self.head_dim = r.integer("head_dim")
+        self.inter = r.integer("inner_size")
+        self.window = r.integer("window")
+        self.eps = r.number("eps")
+        self.theta = r.number("theta")
+        self.max_positions = r.integer("max_positions")
+        r.finish(strict=True)
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(raw)
+
+
+def build_toy_spec(c: ToyConfig) -> ModelSpec:
+    rotary = PartSpec("rotary", {"rotary_dim": c.head_dim // 2, "theta": c.theta, "pairing": "interleaved", "scaling": None})
+
+    def norm(name):
+        return PartSpec("rmsnorm", {"name": name, "size": c.hidden, "eps": c.eps, "unit_offset": True})
+
+    def attn(prefix, window, position):
+        return PartSpec("attention", {"prefix": prefix, "hidden_size": c.hidden, "num_heads": c.heads, "num_kv_heads": c.kv_heads,
+                                      "head_dim": c.head_dim, "scale": 1.0 / math.sqrt(c.head_dim), "window": window, "position": position})
+
+    def ffn(prefix):
+        return PartSpec("gated_mlp", {"prefix": prefix, "hidden_size": c.hidden, "intermediate_size": c.inter, "activation": "gelu_tanh"})
+
+    def layer(i, mixer):
+        p = f"toy.{i}"
+        return LayerSpec(p, "prenorm", mixer, ffn(p + ".ff"), norm(p + ".n1"), norm(p + ".n2"))
+
+    layers = (
+        layer(0, attn("toy.0.att", None, rotary)),  # all keys, partial interleaved rotary
+        layer(1, PartSpec("toy_running_mean", {"prefix": "toy.1", "hidden_size": c.hidden})),
+        layer(2, attn("toy.2.att", c.window, rotary)),  # a window: its own cache group
+        layer(3, attn("toy.3.att", None, None)),  # no position encoding; only ever borrows a cache
+    )
+    run_order = (
+        RunEntry(0),
+        RunEntry(1),
+        RunEntry(2),
+        RunEntry(0),  # layer 0 again: same weights, a cache of its own
+        RunEntry(3, cache_from=0),  # reads the cache of the first entry, writes none
+        RunEntry(1),  # the stateful mixer again: a second state
+    )
+    return ModelSpec(
+        architecture="ToyForCausalLM", hidden_size=c.hidden, vocab_size=c.vocab, max_positions=c.max_positions,
+        embedding=PartSpec("token_embedding", {"name": "toy.embed", "vocab_size": c.vocab, "hidden_size": c.hidden}),
+        layers=layers, run_order=run_order, final_norm=norm("toy.final"),
+        head=PartSpec("lm_head", {"name": "toy.head", "tied_to": None, "vocab_size": c.vocab, "hidden_size": c.hidden}),
+    )
+
+
+register_architecture("ToyForCausalLM", ToyConfig, build_toy_spec)
+
+TOY = {"architectures": ["ToyForCausalLM"], "hidden_size": 96, "vocab_size": 131, "heads": 4, "kv_heads": 2, "head_dim": 32,
+       "inner_size": 136, "window": 24, "eps": 1e-5, "theta": 1000.0, "max_positions": 256}
+
+
+# ------------------------------------------------- the toy model, plainly and whole
+def toy_plain(weights, tokens, rounder=P._identity):
+    c = ToyConfig(TOY)
+    t = len(tokens)
+    w = lambda n: weights[n].float()
+    x = w("toy.embed")[torch.tensor(tokens)]
+    pos = torch.arange(t)
+    inv = P.rope_inv_freq(c.head_dim // 2, c.theta, None)
+    cos, sin = P.rope_cos_sin(pos, inv)
+
+    def norm(x, name):
+        return rounder(P.rms_norm(x, 1.0 + w(name), c.eps))
+
+    def rope_interleaved_partial(v):
+        rd = c.head_dim // 2
+        a, b = v[..., 0:rd:2], v[..., 1:rd:2]
+        out = v.clone()
+        out[..., 0:rd:2] = a * cos[:, None, :] - b * sin[:, None, :]
+        out[..., 1:rd:2] = b * cos[:, None, :] + a * sin[:, None, :]
+        return out
+
+    def ffn(h, p):
+        g = rounder(h @ w(p + ".gate_proj.weight").T)
+        u = rounder(h @ w(p + ".up_proj.weight").T)
+        a = 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g**3)))
+        return rounder(rounder(a * u) @ w(p + ".down_proj.weight").T)
+
+    def attention(h, p, window, rotate, kv=None):
+        q = rounder(h @ w(p + ".q_proj.weight").T).view(t, c.heads, c.head_dim)
+        if kv is None:
+            k = rounder(h @ w(p + ".k_proj.weight").T).view(t, c.kv_heads, c.head_dim)
+            v = rounder(h @ w(p + ".v_proj.weight").T).view(t, c.kv_heads, c.head_dim)
+            if rotate:
+                k = rounder(rope_interleaved_partial(k))
+            kv = (k, v)
+        if rotate:
+            q = rounder(rope_interleaved_partial(q))
+        a = P.causal_attention(q, kv[0], kv[1], 1.0 / math.sqrt(c.head_dim), pos, pos, window, round_p=rounder)
+        return rounder(rounder(a).reshape(t, -1) @ w(p + ".o_proj.weight").T), kv
+
+    def running_mean(h, p):
+        m = torch.cumsum(h, 0) / torch.arange(1, t + 1)[:, None]
+        return rounder(rounder(m) @ w(p + ".mix.weight").T)
+
+    first_cache = None
+    for layer, borrow in ((0, False), (1, False), (2, False), (0, False), (3, True), (1, False)):
+        p = f"toy.{layer}"
+        h = norm(x, p + ".n1")
+        if layer == 1:
+            a = running_mean(h, p)
+        elif layer == 3:
+            a, _ = attention(h, p + ".att", None, False, kv=first_cache)
+        else:
+            a, kv = attention(h, p + ".att", c.window if layer == 2 else None, True)
+            if first_cache is None:
+                first_cache = kv
+        x = x + a
+        x = x + ffn(norm(x, p + ".n2"), p + ".ff")
+    return norm(x, "toy.final") @ w("toy.head").T
+
+
+def make_toy_runner(device, dtype, num_pages):
+    eng = EngineConfig(page_size=16, num_pages=num_pages, max_num_seqs=4, max_model_len=256, dtype=dtype, device=device)
+    ops = RefOps() if device == "cpu" else None
+    model = build_model(TOY, eng, ops=ops)
+    wd = torch.float32 if dtype == "float32" else torch.bfloat16
+    weights = dict(random_tensors(model.tensor_specs(), 3, wd))
+    model.load({k: v.to(device) for k, v in weights.items()})
+    return ModelRunner(model, eng), {k: v.float() for k, v in weights.items()}
+
+
+def test_toy_model_plan():
+    specs = tensor_specs_for(TOY)
+    assert "toy.3.att.k_proj.weight" not in specs, "a layer that only borrows a cache has no k/v projections"
+    assert "toy.0.att.k_proj.weight" in specs and "toy.1.mix.weight" in specs
+    runner, _ = make_toy_runner("cpu", "float32", 8)
+    m = runner.model
+    assert [(g.need.window, len(g.entries)) for g in m.cache_groups] == [(None, 2), (24, 1)]
+    assert [s.owns_cache for s in m.sites] == [True, False, True, True, False, False]
+    assert (m.sites[4].group, m.sites[4].index_in_group) == (m.sites[0].group, m.sites[0].index_in_group)
+    assert [s.state_index for s in m.sites] == [None, 0, None, None, None, 1]
+    assert len(runner.memory.states) == 2 and runner.memory.states[0].shape == (4, 97)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("mode", ["whole", "portions", "mixed"])
+def test_toy_model_replays(backend, mode):
+    device, dtype = backend
+    bf16 = dtype == "bfloat16"
+    reqs = C.make_requests({"vocab_size": TOY["vocab_size"]}, [70, 33, 90, 12, 55], seed=4)
+    steps = {"whole": C.trace_whole, "portions": C.trace_portions, "mixed": C.trace_mixed}[mode](reqs)
+    n_pages = C.pages_needed(steps, reqs, 16)
+    runner, weights = make_toy_runner(device, dtype, n_pages)
+    rounder = P.bf16_round if bf16 else P._identity
+    want = {rid: toy_plain(weights, toks, rounder) for rid, toks in reqs.items()}
+    got, rp = C.run_trace(runner, steps)
+    C.assert_matches(got, want, bf16, f"toy/{mode}")
+    runner.pages.audit()
+    assert runner.pages.live_requests() == 0 and runner.pages.free_slots() == 4
+    if mode != "whole":
+        # the windowed group gave pages back while requests were still live
+        assert any(-1 in runner_table for runner_table in _window_tables(rp)), "no page left the window"
+
+
+def _window_tables(rp):
+    return rp.window_tables
+
+
+@pytest.fixture(autouse=True)
+def _log_window_tables(monkeypatch):
+    """Record the windowed group's block tables after every step of a replay."""
+    from yalis_amd.engine.replay import Replayer
+
+    orig = Replayer.run_step
+
+    def run_step(self, step):
+        out = orig(self, step)
+        if not hasattr(self, "window_tables"):
+            self.window_tables = []
+        if len(self.runner.pages.groups) > 1:
+            for h in self.handles.values():
+                self.window_tables.append(self.runner.pages.block_table(h, 1).tolist())
+        return out
+
+    monkeypatch.setattr(Replayer, "run_step", run_step)
