@@ -44,6 +44,7 @@ def main() -> int:
     ap.add_argument("--prompt-len", type=int, default=1024)
     ap.add_argument("--prefill-len", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    ap.add_argument("--only-prefill", action="store_true", help="measure the prefill only (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
@@ -117,6 +118,19 @@ def main() -> int:
     def step_bytes(batch, mean_ctx_tokens):
         kv = mean_ctx_tokens * layers * 2 * g * d * 2
         return weight_bytes + batch * c * 2 + kv
+
+    if args.only_prefill:
+        t = args.prefill_len
+        prompt = torch.randint(0, vocab, (t,), generator=gen).tolist()
+        for i in range(3):
+            assert runner.admit(1000 + i) and runner.reserve(1000 + i, t)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            ops.argmax(runner.step([StepEntry(1000 + i, prompt, [t - 1])])).tolist()
+            torch.cuda.synchronize()
+            print(f"prefill {t} tokens: {1e3 * (time.perf_counter() - t0):.3f} ms")
+            runner.release(1000 + i)
+        return 0
 
     dt, mean_ctx = decode_run(args.batch, args.steps, args.warmup)
     ms_per_step = 1e3 * dt / args.steps

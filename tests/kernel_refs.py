@@ -39,14 +39,15 @@ def _rmsnorm(x, weight, eps, unit_offset):
     return x * torch.rsqrt(ms + eps) * w
 
 
-def linear(x, w, out_dtype):
+def linear(x, w, out_dtype, partial_ok=False):
     return (x.to(torch.float32) @ w.to(torch.float32).T).to(out_dtype)
 
 
 def rope_append(qkv, n_heads, n_kv, head_dim, positions, cos, sin, rotary_dim, interleaved,
                 k_cache, v_cache, slots, page_size):
     """Rotates the query heads of ``qkv`` in place; rotates the key heads and stores
-    them, and the value heads transposed, at each token's slot of the pages."""
+    them, and the value heads transposed, at each token's slot of the pages.  Returns the
+    tensor whose rows start with the rotated queries."""
     n = qkv.shape[0]
     x = qkv.view(n, n_heads + 2 * n_kv, head_dim)
     rot = x[:, : n_heads + n_kv].to(torch.float32)
@@ -75,6 +76,7 @@ def rope_append(qkv, n_heads, n_kv, head_dim, positions, cos, sin, rotary_dim, i
         off = (slots % page_size).long()
         k_cache[page, :, off, :] = rot[:, n_heads:]
         v_cache[page, :, :, off] = x[:, n_heads + n_kv :]
+    return qkv
 
 
 def attention_paged(q, k_cache, v_cache, positions, token_seq, block_table, page_size, scale, window):
@@ -101,7 +103,7 @@ def attention_paged(q, k_cache, v_cache, positions, token_seq, block_table, page
     return out
 
 
-def attention(qkv, n_heads, n_kv_rows, n_kv, head_dim, k_cache, v_cache, page_size, scale,
+def attention(qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size, scale,
               window, ctx, group, tiles):
     n = qkv.shape[0]
     q = qkv.view(n, -1, head_dim)[:, :n_heads]
@@ -112,7 +114,7 @@ def attention(qkv, n_heads, n_kv_rows, n_kv, head_dim, k_cache, v_cache, page_si
     return out.reshape(n, n_heads * head_dim).to(qkv.dtype)
 
 
-def gated_act(gu, activation):
+def gated_act(gu, activation, out_dtype=None):
     inter = gu.shape[1] // 2
     g = gu[:, :inter].to(torch.float32)
     u = gu[:, inter:].to(torch.float32)
@@ -122,7 +124,7 @@ def gated_act(gu, activation):
         a = 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g**3)))
     else:
         raise ValueError(activation)
-    return (a * u).to(gu.dtype)
+    return (a * u).to(out_dtype or gu.dtype)
 
 
 def argmax(logits):

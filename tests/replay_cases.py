@@ -133,7 +133,7 @@ def run_trace(runner: ModelRunner, steps: List[dict]):
         assert logits is None or r == logits.shape[0]
         for rid in s["end"]:
             cached.pop(rid, None)
-    out = {rid: torch.stack([d[i] for i in range(len(d))]) for rid, d in rows.items()}
+    out = {rid: torch.stack([d[i] for i in sorted(d)]) for rid, d in rows.items()}
     return out, rp
 
 

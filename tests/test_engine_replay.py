@@ -136,3 +136,31 @@ def test_far_key_across_pages(backend):
     runner = C.make_runner(cfg, weights, dtype, device, ops_for(device), 16, 19)
     got, _ = C.run_trace(runner, C.trace_tail({"r0": toks}, tail=8))
     C.assert_matches(got, want, dtype == "bfloat16", "far key")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_match_eager_steps(dtype):
+    """Decode steps replayed from a captured graph, with eager steps (a prompt portion of
+    another request) between the replays, give what eager decode steps give."""
+    cfg, weights, reqs, want = setup("C", dtype)
+    toks, other = reqs["r3"], reqs["r2"]
+    outs = {}
+    for graphs in (False, True):
+        runner = C.make_runner(cfg, weights, dtype, "cuda:0", ops_for("cuda:0"), 16, 24)
+        runner.use_graphs = graphs
+        steps = [{"step": 0, "entries": [{"id": "a", "tokens": toks[:100], "want": []}], "end": []}]
+        k = 1
+        for j in range(100, len(toks)):
+            if j % 7 == 0:  # an eager step in between: a portion of another request
+                i0 = (j - 100) // 7 * 5
+                steps.append({"step": k, "entries": [{"id": "b", "tokens": other[i0 : i0 + 5], "want": [4]}], "end": []})
+                k += 1
+            steps.append({"step": k, "entries": [{"id": "a", "tokens": [toks[j]], "want": [0]}], "end": []})
+            k += 1
+        got, _ = C.run_trace(runner, steps)
+        outs[graphs] = got
+        assert (runner.graph_replays > 0) == graphs
+    assert torch.equal(outs[True]["a"], outs[False]["a"]), "a replayed step differs from the eager step"
+    assert torch.equal(outs[True]["b"], outs[False]["b"])
+    C.assert_matches({"r3": torch.cat([want["r3"][:0], outs[True]["a"]])}, {"r3": want["r3"][100:]}, dtype == "bfloat16", "graph decode")

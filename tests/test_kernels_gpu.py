@@ -142,6 +142,49 @@ def test_gemm_mfma_operand_order(ops):
         assert torch.equal(got, want), f"k={kk}"
 
 
+def test_split_sums_feed_their_consumers(ops):
+    """A few-row product may stay as unreduced K slices; norm, rotary + append and the
+    gated activation add them up themselves and must agree with the reduced path."""
+    from yalis_amd.ops.hip import SplitSum
+
+    m, k = 5, 4096
+    x = rnd((m, k), torch.bfloat16, 20, 0.5)
+    # norm
+    w = rnd((256, k), torch.bfloat16, 21, 0.05)
+    part = ops.linear(x, w, torch.bfloat16, partial_ok=True)
+    assert isinstance(part, SplitSum) and part.n_splits > 1, "this shape was meant to split K"
+    full = part.tensor.sum(0)
+    assert (full.cpu() - (x.double().cpu() @ w.double().cpu().T).float()).abs().max() < 1e-3
+    res = rnd((m, 256), torch.float32, 22)
+    nw = (1 + 0.1 * rnd((256,), torch.float32, 23)).to(torch.bfloat16)
+    r1, r2 = res.clone(), res.clone()
+    got = ops.add_rmsnorm(r1, part, nw, 1e-5, False, torch.bfloat16)
+    want = ops.add_rmsnorm(r2, full, nw, 1e-5, False, torch.bfloat16)
+    close(r1, r2, 2e-6, 2e-6)
+    close(got, want, 1e-2, 2**-7)
+    rows = torch.tensor([4, 0], dtype=torch.int32, device=DEV)
+    # two float32 summation orders: a few units in the last place
+    close(ops.gather_add_rmsnorm(res, part, rows, nw, 1e-5, False, torch.float32),
+          ops.gather_add_rmsnorm(res, full, rows, nw, 1e-5, False, torch.float32), 2e-6, 2e-6)
+    # gated activation
+    close(ops.gated_act(part, "silu", torch.bfloat16), ops.gated_act(full.to(torch.bfloat16), "silu"), 1e-2, 2**-7)
+    close(ops.gated_act(part, "silu", torch.float32), R.gated_act(full.cpu(), "silu"), 1e-5, 1e-5)
+    # rotary + append: 2 query heads, 1 kv head of 64 -> 256 columns
+    cos, sin = _tables(64, 100)
+    positions = torch.tensor([3, 4, 50, 0, 99], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([5, 6, 40, 0, 63], dtype=torch.int32, device=DEV)
+    kc = torch.zeros((4, 1, 16, 64), dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros((4, 1, 64, 16), dtype=torch.bfloat16, device=DEV)
+    q = ops.rope_append(part, 2, 1, 64, positions, cos, sin, 64, False, kc, vc, slots, 16)
+    assert q.shape == (m, 128) and q.dtype == torch.bfloat16
+    kr, vr = torch.zeros((4, 1, 16, 64)), torch.zeros((4, 1, 64, 16))
+    ref2 = full.clone().cpu()
+    R.rope_append(ref2, 2, 1, 64, positions.cpu(), cos.cpu(), sin.cpu(), 64, False, kr, vr, slots.cpu(), 16)
+    close(q, ref2[:, :128], 1e-2, 2**-7)
+    close(kc, kr, 1e-2, 2**-7)
+    close(vc, vr, 1e-2, 2**-7)
+
+
 def test_linear_dispatch(ops):
     x = rnd((200, 192), torch.bfloat16, 8)
     w = rnd((515, 192), torch.bfloat16, 9)
@@ -220,8 +263,8 @@ def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True,
     n = hb.n_tokens
     q = (torch.randn((n, h * d), generator=gen) * 1.5).to(dtype)
     scale = 1.0 / math.sqrt(d)
-    got = ops.attention(q.to(DEV), h, 0, g, d, kc.to(DEV), vc.to(DEV), page, scale, window, ctx, 0, ctx.arrays["tiles"])
-    want = R.attention(q.float(), h, 0, g, d, kc.float(), vc.float(), page, scale, window, ctx_cpu, 0, None)
+    got = ops.attention(q.to(DEV), h, g, d, kc.to(DEV), vc.to(DEV), page, scale, window, ctx, 0, ctx.arrays["tiles"])
+    want = R.attention(q.float(), h, g, d, kc.float(), vc.float(), page, scale, window, ctx_cpu, 0, None)
     return got, want
 
 
@@ -286,7 +329,7 @@ def test_attention_far_key_stands_out(ops):
             arrays={kk: torch.from_numpy(np.ascontiguousarray(vv)).to(DEV) for kk, vv in arrays.items()},
             max_ctx=hb.max_ctx,
         )
-        got = ops.attention(q.to(dtype).to(DEV), h, 0, g, d, kc.to(DEV), vc.to(DEV), page, 1.0 / math.sqrt(d), 0, ctx, 0, ctx.arrays["tiles"])
+        got = ops.attention(q.to(dtype).to(DEV), h, g, d, kc.to(DEV), vc.to(DEV), page, 1.0 / math.sqrt(d), 0, ctx, 0, ctx.arrays["tiles"])
         head1 = got.view(h, d)[1].float().cpu()
         close(head1, v[far, 0].to(dtype).float(), 2e-2, 2**-6)
 

@@ -132,6 +132,9 @@ class EngineConfig:
     max_model_len: longest sequence (prompt plus generated) a request may reach.
     max_num_batched_tokens: token budget of one step (decode tokens plus prompt portions).
     dtype: "bfloat16" or "float32" (the latter is the true 32-bit path).
+    decode_graphs: replay steps that hold single tokens only from captured HIP graphs
+        (the reference's YALIS_DISABLE_DECODE_CUDAGRAPHS switches the same off,
+        yalis/engine.py:44-48).
     """
 
     page_size: int = 64
@@ -141,6 +144,7 @@ class EngineConfig:
     max_num_batched_tokens: int = 2048
     dtype: str = "bfloat16"
     device: str = "cuda:0"
+    decode_graphs: bool = True  # capture steps of single tokens as HIP graphs
 
     def __post_init__(self) -> None:
         self.dtype = canonical_dtype(self.dtype)

@@ -147,6 +147,15 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 // Columns of a wave: column c in 0..15 is token c / hpt of the tile and query head
 // h_base + c % hpt, hpt = min(H/G, 16) heads per tile; a kv head with more than 16
 // query heads takes several "chunks" of 16.
+//
+// Keys are walked in blocks of 64 = two groups of 32.  Within a group the 16 rows of the
+// two score products are assigned to keys so that afterwards lane group g holds the
+// probabilities of keys 8g .. 8g+7 of the group in order: row i of the first product is key
+// 8*(i/4) + i%4, row i of the second is key 8*(i/4) + 4 + i%4.  Then the transposed values
+// feed the second product as one 16-byte load per lane (8 consecutive keys of one value
+// row).  Every load is unconditional (addresses are clamped into allocated pages, what they
+// bring for keys that do not count is masked or zeroed), so that the values of a block and
+// the keys of the next are in flight while the block's scores are worked on.
 template <int D>
 __global__ __launch_bounds__(64) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
@@ -174,6 +183,7 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
   const int my_lo = kb_lo + blockIdx.z * per_split;
   const int my_hi = min(kb_hi, my_lo + per_split);
   const int32_t* bt = block_table + static_cast<size_t>(seq) * table_width;
+  const int last_page_col = min(table_width - 1, (hi - 1) / page_size);
 
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
   AFrag8 qf[KS];
@@ -181,106 +191,109 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
     const bf16_t* qp = q + static_cast<size_t>(tok0 + (col_ok ? tt : 0)) * q_stride +
                        static_cast<size_t>(h_base + (col_ok ? hh : 0)) * D + 8 * gq;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      qf[ks].u = col_ok ? *reinterpret_cast<const u32x4_t*>(qp + 32 * ks) : zero4;
+    for (int ks = 0; ks < KS; ++ks) {
+      qf[ks].u = *reinterpret_cast<const u32x4_t*>(qp + 32 * ks);
+      if (!col_ok) qf[ks].u = zero4;
+    }
   }
   float m = -INFINITY, l = 0.f;
   f32x4_t acc[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
+  // the key this lane's score rows stand for, relative to the block: [group][product]
+  const int krow = 8 * (r / 4) + r % 4;
+  // a page that exists for any key: keys beyond the request read the last allocated page
+  auto page_of = [&](int key) { return max(0, bt[min(key / page_size, last_page_col)]); };
+
+  AFrag8 kf[2][2][KS];
+#define ATT_LOAD_K(KB)                                                                            \
+  _Pragma("unroll") for (int u = 0; u < 2; ++u) _Pragma("unroll") for (int sb = 0; sb < 2; ++sb) { \
+    const int key = (KB) * 64 + 32 * u + krow + 4 * sb;                                           \
+    const bf16_t* kp = k_cache + ((static_cast<size_t>(page_of(key)) * n_kv + g) * page_size + key % page_size) * D + 8 * gq; \
+    _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                             \
+        kf[u][sb][ks].u = *reinterpret_cast<const u32x4_t*>(kp + 32 * ks);                        \
+  }
+
+  if (my_lo < my_hi) ATT_LOAD_K(my_lo)
   for (int kb = my_lo; kb < my_hi; ++kb) {
-    f32x4_t s[4];
-    int page_of[4];
-    int koff_of[4];
-    bool live[4];
+    // values of this block: lane (r, gq) holds 8 consecutive keys of value row 16*dt + r
+    AFrag8 vf[2][DT];
 #pragma unroll
-    for (int sub = 0; sub < 4; ++sub) {
-      const int key0 = kb * 64 + 16 * sub;
-      s[sub] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      live[sub] = key0 < hi && key0 + 16 > lo;  // same for every lane
-      page_of[sub] = 0;
-      koff_of[sub] = key0 % page_size;
-      if (live[sub]) {
-        page_of[sub] = bt[key0 / page_size];
-        const bf16_t* kp = k_cache +
-                           ((static_cast<size_t>(page_of[sub]) * n_kv + g) * page_size + koff_of[sub] + r) * D +
-                           8 * gq;
+    for (int u = 0; u < 2; ++u) {
+      const int key = kb * 64 + 32 * u + 8 * gq;
+      const bf16_t* vp = v_cache + (static_cast<size_t>(page_of(key)) * n_kv + g) * D * page_size + key % page_size;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          AFrag8 a;
-          a.u = *reinterpret_cast<const u32x4_t*>(kp + 32 * ks);
-          s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[ks].v, s[sub], 0, 0, 0);
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = key0 + 4 * gq + i;
-        const bool ok = live[sub] && col_ok && key <= pos_c && key >= lo_c;
-        s[sub][i] = ok ? s[sub][i] * scale_log2 : -INFINITY;
-      }
+      for (int dt = 0; dt < DT; ++dt)
+        vf[u][dt].u = *reinterpret_cast<const u32x4_t*>(vp + static_cast<size_t>(16 * dt + r) * page_size);
     }
+    // scores
+    f32x4_t s[2][2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int sb = 0; sb < 2; ++sb) {
+        s[u][sb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          s[u][sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][sb][ks].v, qf[ks].v, s[u][sb], 0, 0, 0);
+      }
+    if (kb + 1 < my_hi) ATT_LOAD_K(kb + 1)
     float tmax = -INFINITY;
 #pragma unroll
-    for (int sub = 0; sub < 4; ++sub)
+    for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, s[sub][i]);
+      for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = kb * 64 + 32 * u + 8 * gq + 4 * sb + i;
+          const bool ok = col_ok && key <= pos_c && key >= lo_c;
+          s[u][sb][i] = ok ? s[u][sb][i] * scale_log2 : -INFINITY;
+          tmax = fmaxf(tmax, s[u][sb][i]);
+        }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
     const float m_new = fmaxf(m, tmax);
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
     const float alpha = exp2f(m - m_safe);
     float psum = 0.f;
+    AFrag8 pf[2];
 #pragma unroll
-    for (int sub = 0; sub < 4; ++sub)
+    for (int u = 0; u < 2; ++u) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        s[sub][i] = exp2f(s[sub][i] - m_safe);
-        psum += s[sub][i];
+      for (int sb = 0; sb < 2; ++sb) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          s[u][sb][i] = exp2f(s[u][sb][i] - m_safe);
+          psum += s[u][sb][i];
+        }
+        pf[u].u[2 * sb] = pack_bf16x2(s[u][sb][0], s[u][sb][1]);
+        pf[u].u[2 * sb + 1] = pack_bf16x2(s[u][sb][2], s[u][sb][3]);
       }
+    }
     l = l * alpha + psum;
     m = m_new;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[dt] *= alpha;
-
+    // values of keys that do not exist yet may be anything: zero them (last block only)
+    if (kb * 64 + 64 > hi) {
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int sa = 2 * u, sb = 2 * u + 1;
-      if (!live[sa] && !live[sb]) continue;
-      AFrag8 b;
-      b.u[0] = pack_bf16x2(s[sa][0], s[sa][1]);
-      b.u[1] = pack_bf16x2(s[sa][2], s[sa][3]);
-      b.u[2] = pack_bf16x2(s[sb][0], s[sb][1]);
-      b.u[3] = pack_bf16x2(s[sb][2], s[sb][3]);
-      const int key_a = kb * 64 + 16 * sa + 4 * gq;  // first of this lane's four keys in tile a
-      const int key_b = key_a + 16;
-      const bool edge = kb * 64 + 16 * sb + 16 > hi;  // some keys of the pair do not exist yet
-      const bf16_t* va = v_cache + (static_cast<size_t>(page_of[sa]) * n_kv + g) * D * page_size +
-                         koff_of[sa] + 4 * gq;
-      const bf16_t* vb = v_cache + (static_cast<size_t>(page_of[sb]) * n_kv + g) * D * page_size +
-                         koff_of[sb] + 4 * gq;
+      for (int u = 0; u < 2; ++u) {
+        const int key = kb * 64 + 32 * u + 8 * gq;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const size_t row = static_cast<size_t>(16 * dt + r) * page_size;
-        AFrag8 a;
-        u32x2_t xa = {0u, 0u}, xb = {0u, 0u};
-        if (live[sa]) xa = *reinterpret_cast<const u32x2_t*>(va + row);
-        if (live[sb]) xb = *reinterpret_cast<const u32x2_t*>(vb + row);
-        a.u[0] = xa[0];
-        a.u[1] = xa[1];
-        a.u[2] = xb[0];
-        a.u[3] = xb[1];
-        if (edge) {
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            if (key_a + i >= hi) a.h[i] = 0;
-            if (key_b + i >= hi) a.h[4 + i] = 0;
-          }
-        }
-        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[dt], 0, 0, 0);
+          for (int e = 0; e < 8; ++e)
+            if (key + e >= hi) vf[u][dt].h[e] = 0;
       }
     }
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[u][dt].v, pf[u].v, acc[dt], 0, 0, 0);
   }
+#undef ATT_LOAD_K
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
 
@@ -310,6 +323,7 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
 }
 
 // Merge the splits of every column: weights exp2(m_s - max m), in the order of s.
+// A thread owns four consecutive output elements of one column.
 template <int D>
 __global__ __launch_bounds__(256) void attn_combine_kernel(
     bf16_t* __restrict__ out, const int32_t* __restrict__ tiles, int n_heads, int n_kv, int hpt,
@@ -321,19 +335,27 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(
   const int h_base = g * qpk + chunk * hpt;
   const int heads_here = min(hpt, qpk - chunk * hpt);
   const size_t w0 = (static_cast<size_t>(t) * gridDim.y + blockIdx.y) * n_splits;
-  for (int e = threadIdx.x; e < 16 * D; e += blockDim.x) {
-    const int c = e / D, d = e % D;
+  for (int e = threadIdx.x; e < 16 * (D / 4); e += blockDim.x) {
+    const int c = e / (D / 4), d = (e % (D / 4)) * 4;
     const int tt = c / hpt, hh = c % hpt;
     if (tt >= ntok || hh >= heads_here) continue;
+    const float* ml = ws_ml + (w0 * 16 + c) * 2;
     float m_max = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) m_max = fmaxf(m_max, ws_ml[((w0 + s) * 16 + c) * 2]);
-    float num = 0.f, den = 0.f;
+#pragma unroll 4
+    for (int s = 0; s < n_splits; ++s) m_max = fmaxf(m_max, ml[static_cast<size_t>(s) * 32]);
+    f32x4_t num = {0.f, 0.f, 0.f, 0.f};
+    float den = 0.f;
+#pragma unroll 4
     for (int s = 0; s < n_splits; ++s) {
-      const float w = exp2f(ws_ml[((w0 + s) * 16 + c) * 2] - m_max);
-      num += w * ws_o[((w0 + s) * 16 + c) * D + d];
-      den += w * ws_ml[((w0 + s) * 16 + c) * 2 + 1];
+      const float w = exp2f(ml[static_cast<size_t>(s) * 32] - m_max);
+      num += w * *reinterpret_cast<const f32x4_t*>(ws_o + ((w0 + s) * 16 + c) * D + d);
+      den += w * ml[static_cast<size_t>(s) * 32 + 1];
     }
-    out[(static_cast<size_t>(tok0 + tt) * n_heads + h_base + hh) * D + d] = f32_to_bf16(num / den);
+    const float inv = 1.f / den;
+    u32x2_t o;
+    o[0] = pack_bf16x2(num[0] * inv, num[1] * inv);
+    o[1] = pack_bf16x2(num[2] * inv, num[3] * inv);
+    *reinterpret_cast<u32x2_t*>(out + (static_cast<size_t>(tok0 + tt) * n_heads + h_base + hh) * D + d) = o;
   }
 }
 

@@ -6,6 +6,8 @@
 // yalis/external/model.py:894-909 with the table of :786-820; cache append
 // yalis/attention/utils/flash_utils.py:34-43,64-89; silu(gate) * up
 // yalis/external/model.py:741-743.  Everything is computed in float32 and rounded once.
+#include <algorithm>
+
 #include "common.h"
 
 // ------------------------------------------------------------------ error reporting
@@ -23,7 +25,7 @@ int yk_check_launch(const char* what) {
   return 0;
 }
 extern "C" const char* yk_last_error() { return yk_error_slot().c_str(); }
-extern "C" int yk_abi_version() { return 1; }
+extern "C" int yk_abi_version() { return 2; }
 
 // ------------------------------------------------------------------------- embedding
 // out[n, :] = float(table[ids[n], :])
@@ -39,10 +41,43 @@ __global__ void embed_kernel(const int32_t* __restrict__ ids, const T* __restric
   for (int c = threadIdx.x; c < width; c += blockDim.x) dst[c] = to_f32<T>(src[c]);
 }
 
+// eight elements per thread, no loop (bfloat16 tables whose width is a multiple of 8)
+__global__ void embed_bf16x8_kernel(const int32_t* __restrict__ ids, const bf16_t* __restrict__ table,
+                                    float* __restrict__ out, int width, int vocab, size_t total_vec) {
+  const size_t v = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
+  if (v >= total_vec) return;
+  const int per_row = width / 8;
+  const size_t n = v / per_row;
+  const int c = static_cast<int>(v % per_row) * 8;
+  int id = ids[n];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const uint4 raw = *reinterpret_cast<const uint4*>(table + static_cast<size_t>(id) * width + c);
+  const uint32_t wds[4] = {raw.x, raw.y, raw.z, raw.w};
+  float4 lo, hi;
+  lo.x = __uint_as_float(wds[0] << 16);
+  lo.y = __uint_as_float(wds[0] & 0xffff0000u);
+  lo.z = __uint_as_float(wds[1] << 16);
+  lo.w = __uint_as_float(wds[1] & 0xffff0000u);
+  hi.x = __uint_as_float(wds[2] << 16);
+  hi.y = __uint_as_float(wds[2] & 0xffff0000u);
+  hi.z = __uint_as_float(wds[3] << 16);
+  hi.w = __uint_as_float(wds[3] & 0xffff0000u);
+  float* dst = out + n * width + c;
+  *reinterpret_cast<float4*>(dst) = lo;
+  *reinterpret_cast<float4*>(dst + 4) = hi;
+}
+
 extern "C" int yk_embed(const int32_t* ids, const void* table, int table_dtype, float* out,
                         int n_tokens, int width, int vocab, hipStream_t stream) {
   YK_REQUIRE(n_tokens >= 0 && width > 0 && vocab > 0, "embed: bad sizes");
   if (n_tokens == 0) return 0;
+  if (table_dtype == YK_BF16 && width % 8 == 0 && reinterpret_cast<uintptr_t>(table) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(out) % 16 == 0) {
+    const size_t total_vec = static_cast<size_t>(n_tokens) * (width / 8);
+    embed_bf16x8_kernel<<<static_cast<unsigned>((total_vec + 255) / 256), 256, 0, stream>>>(
+        ids, static_cast<const bf16_t*>(table), out, width, vocab, total_vec);
+    return yk_check_launch("embed");
+  }
   dim3 grid(n_tokens), block(256);
   if (table_dtype == YK_F32)
     embed_kernel<float><<<grid, block, 0, stream>>>(ids, static_cast<const float*>(table), out, width, vocab);
@@ -53,13 +88,47 @@ extern "C" int yk_embed(const int32_t* ids, const void* table, int table_dtype, 
   return yk_check_launch("embed");
 }
 
+// ---------------------------------------------------------------- four-wide accessors
+template <typename T>
+__device__ __forceinline__ float4 load4(const T* p);
+template <>
+__device__ __forceinline__ float4 load4<float>(const float* p) {
+  return *reinterpret_cast<const float4*>(p);
+}
+template <>
+__device__ __forceinline__ float4 load4<bf16_t>(const bf16_t* p) {
+  const uint2 raw = *reinterpret_cast<const uint2*>(p);
+  float4 v;
+  v.x = __uint_as_float(raw.x << 16);
+  v.y = __uint_as_float(raw.x & 0xffff0000u);
+  v.z = __uint_as_float(raw.y << 16);
+  v.w = __uint_as_float(raw.y & 0xffff0000u);
+  return v;
+}
+template <typename T>
+__device__ __forceinline__ void store4(T* p, float4 v);
+template <>
+__device__ __forceinline__ void store4<float>(float* p, float4 v) {
+  *reinterpret_cast<float4*>(p) = v;
+}
+template <>
+__device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float4 v) {
+  uint2 raw;
+  raw.x = static_cast<uint32_t>(f32_to_bf16(v.x)) | (static_cast<uint32_t>(f32_to_bf16(v.y)) << 16);
+  raw.y = static_cast<uint32_t>(f32_to_bf16(v.z)) | (static_cast<uint32_t>(f32_to_bf16(v.w)) << 16);
+  *reinterpret_cast<uint2*>(p) = raw;
+}
+
 // ------------------------------------------------------------- residual add + RMS norm
 // For row r (source row rows[r] when rows is given):
-//   v = residual[src] + delta[src]           (float32; delta may be absent)
-//   residual[src] = v                        (only when rows is null)
+//   v = residual[src] + sum over s of delta[s][src]   (float32; delta may be absent;
+//       n_splits > 1: delta holds the unreduced K slices of a product, float32)
+//   residual[src] = v                                  (only when rows is null)
 //   out[r] = v * rsqrt(mean(v^2) + eps) * (weight [+ 1])
+// General form: any width, two passes over the row.
 template <typename TD, typename TW, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
+                                   int n_splits, size_t split_stride,
                                    const int32_t* __restrict__ rows, const TW* __restrict__ weight,
                                    TO* __restrict__ out, int width, float eps, int unit_offset) {
   __shared__ float scratch[17];
@@ -71,7 +140,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
     float v = res[c];
     if (del) {
-      v += to_f32<TD>(del[c]);
+      for (int s = 0; s < n_splits; ++s) v += to_f32<TD>(del[s * split_stride + c]);
       if (!rows) res[c] = v;
     }
     ss += v * v;
@@ -81,120 +150,209 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
   TO* o = out + static_cast<size_t>(r) * width;
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
     float v = res[c];
-    if (del && rows) v += to_f32<TD>(del[c]);  // not written back in the gathered form
+    if (del && rows)  // not written back in the gathered form
+      for (int s = 0; s < n_splits; ++s) v += to_f32<TD>(del[s * split_stride + c]);
     float w = to_f32<TW>(weight[c]);
     if (unit_offset) w += 1.f;
     o[c] = from_f32<TO>(v * inv * w);
   }
 }
 
-template <typename TD, typename TW>
-static int launch_add_rmsnorm_o(float* residual, const void* delta, const int32_t* rows,
-                                const void* weight, void* out, int out_dtype, int n_rows, int width,
-                                float eps, int unit_offset, hipStream_t stream) {
-  dim3 grid(n_rows), block(width >= 2048 ? 512 : 256);
-  if (out_dtype == YK_F32)
-    add_rmsnorm_kernel<TD, TW, float><<<grid, block, 0, stream>>>(
-        residual, static_cast<const TD*>(delta), rows, static_cast<const TW*>(weight),
-        static_cast<float*>(out), width, eps, unit_offset);
-  else if (out_dtype == YK_BF16)
-    add_rmsnorm_kernel<TD, TW, bf16_t><<<grid, block, 0, stream>>>(
-        residual, static_cast<const TD*>(delta), rows, static_cast<const TW*>(weight),
-        static_cast<bf16_t*>(out), width, eps, unit_offset);
-  else
-    return yk_fail("add_rmsnorm: unsupported output dtype");
+// Fast form: width a multiple of 4 and at most 4 * NORM_IT * blockDim; the row stays in
+// registers, every load of a thread is issued before the first use.
+constexpr int NORM_IT = 8;
+template <typename TD, typename TW, typename TO>
+__global__ __launch_bounds__(512) void add_rmsnorm_vec_kernel(
+    float* __restrict__ residual, const TD* __restrict__ delta, int n_splits, size_t split_stride,
+    const int32_t* __restrict__ rows, const TW* __restrict__ weight, TO* __restrict__ out,
+    int width, float eps, int unit_offset) {
+  __shared__ float scratch[17];
+  const int r = blockIdx.x;
+  const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
+  float* res = residual + src * width;
+  const TD* del = delta ? delta + src * width : nullptr;
+  float4 v[NORM_IT], w[NORM_IT];
+  float ss = 0.f;
+#pragma unroll
+  for (int it = 0; it < NORM_IT; ++it) {
+    const int c = (threadIdx.x + it * blockDim.x) * 4;
+    if (c < width) {
+      v[it] = load4<float>(res + c);
+      w[it] = load4<TW>(weight + c);
+    }
+  }
+  if (del) {
+    // four slices at a time, all loads issued before the first sum; a slice index beyond
+    // the last is clamped and its value dropped, so that the loads carry no condition
+    for (int s0 = 0; s0 < n_splits; s0 += 4) {
+#pragma unroll
+      for (int it = 0; it < NORM_IT; ++it) {
+        const int c = (threadIdx.x + it * blockDim.x) * 4;
+        if (c < width) {
+          float4 d[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) d[j] = load4<TD>(del + static_cast<size_t>(min(s0 + j, n_splits - 1)) * split_stride + c);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            if (s0 + j < n_splits) {
+              v[it].x += d[j].x;
+              v[it].y += d[j].y;
+              v[it].z += d[j].z;
+              v[it].w += d[j].w;
+            }
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < NORM_IT; ++it) {
+    const int c = (threadIdx.x + it * blockDim.x) * 4;
+    if (c < width) {
+      if (del && !rows) store4<float>(res + c, v[it]);
+      ss += v[it].x * v[it].x + v[it].y * v[it].y + v[it].z * v[it].z + v[it].w * v[it].w;
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = rsqrtf(ss / static_cast<float>(width) + eps);
+  const float off = unit_offset ? 1.f : 0.f;
+  TO* o = out + static_cast<size_t>(r) * width;
+#pragma unroll
+  for (int it = 0; it < NORM_IT; ++it) {
+    const int c = (threadIdx.x + it * blockDim.x) * 4;
+    if (c < width) {
+      float4 y;
+      y.x = v[it].x * inv * (w[it].x + off);
+      y.y = v[it].y * inv * (w[it].y + off);
+      y.z = v[it].z * inv * (w[it].z + off);
+      y.w = v[it].w * inv * (w[it].w + off);
+      store4<TO>(o + c, y);
+    }
+  }
+}
+
+template <typename TD, typename TW, typename TO>
+static int launch_add_rmsnorm(float* residual, const void* delta, int n_splits, size_t split_stride,
+                              const int32_t* rows, const void* weight, void* out, int n_rows,
+                              int width, float eps, int unit_offset, hipStream_t stream) {
+  const bool aligned = width % 4 == 0 && reinterpret_cast<uintptr_t>(residual) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(delta) % 16 == 0 && reinterpret_cast<uintptr_t>(weight) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(out) % 16 == 0 && split_stride % 4 == 0;
+  if (aligned && width <= 4 * NORM_IT * 512) {
+    // two four-wide chunks per thread where the row allows, at most 512 threads
+    int threads = ((width / 4 + 1) / 2 + 63) / 64 * 64;
+    threads = std::max(64, std::min(threads, 512));
+    add_rmsnorm_vec_kernel<TD, TW, TO><<<n_rows, threads, 0, stream>>>(
+        residual, static_cast<const TD*>(delta), n_splits, split_stride, rows,
+        static_cast<const TW*>(weight), static_cast<TO*>(out), width, eps, unit_offset);
+  } else {
+    add_rmsnorm_kernel<TD, TW, TO><<<n_rows, width >= 2048 ? 512 : 256, 0, stream>>>(
+        residual, static_cast<const TD*>(delta), n_splits, split_stride, rows,
+        static_cast<const TW*>(weight), static_cast<TO*>(out), width, eps, unit_offset);
+  }
   return yk_check_launch("add_rmsnorm");
 }
 
-// delta may be null (then delta_dtype is ignored); rows may be null.
-extern "C" int yk_add_rmsnorm(float* residual, const void* delta, int delta_dtype,
+// delta may be null (then delta_dtype is ignored); rows may be null.  n_splits > 1 needs
+// float32 delta laid out [n_splits][rows of the residual][width].
+extern "C" int yk_add_rmsnorm(float* residual, const void* delta, int delta_dtype, int n_splits,
                               const int32_t* rows, const void* weight, int weight_dtype, void* out,
-                              int out_dtype, int n_rows, int width, float eps, int unit_offset,
-                              hipStream_t stream) {
-  YK_REQUIRE(n_rows >= 0 && width > 0, "add_rmsnorm: bad sizes");
+                              int out_dtype, int n_rows, int n_residual_rows, int width, float eps,
+                              int unit_offset, hipStream_t stream) {
+  YK_REQUIRE(n_rows >= 0 && width > 0 && n_residual_rows >= 0, "add_rmsnorm: bad sizes");
   YK_REQUIRE(eps >= 0.f, "add_rmsnorm: eps must not be negative");
+  YK_REQUIRE(n_splits >= 1, "add_rmsnorm: bad split count");
+  YK_REQUIRE(n_splits == 1 || delta_dtype == YK_F32, "add_rmsnorm: unreduced slices must be float32");
   if (n_rows == 0) return 0;
-  if (!delta) delta_dtype = YK_F32;
-#define YK_CASE(DD, TD, WD, TW)                        \
-  if (delta_dtype == DD && weight_dtype == WD)         \
-    return launch_add_rmsnorm_o<TD, TW>(residual, delta, rows, weight, out, out_dtype, n_rows, width, eps, unit_offset, stream);
-  YK_CASE(YK_F32, float, YK_F32, float)
-  YK_CASE(YK_F32, float, YK_BF16, bf16_t)
-  YK_CASE(YK_BF16, bf16_t, YK_F32, float)
-  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t)
+  if (!delta) {
+    delta_dtype = YK_F32;
+    n_splits = 1;
+  }
+  const size_t stride = static_cast<size_t>(n_residual_rows) * width;
+#define YK_CASE(DD, TD, WD, TW, OD, TO)                                  \
+  if (delta_dtype == DD && weight_dtype == WD && out_dtype == OD)        \
+    return launch_add_rmsnorm<TD, TW, TO>(residual, delta, n_splits, stride, rows, weight, out, n_rows, width, eps, unit_offset, stream);
+  YK_CASE(YK_F32, float, YK_F32, float, YK_F32, float)
+  YK_CASE(YK_F32, float, YK_F32, float, YK_BF16, bf16_t)
+  YK_CASE(YK_F32, float, YK_BF16, bf16_t, YK_F32, float)
+  YK_CASE(YK_F32, float, YK_BF16, bf16_t, YK_BF16, bf16_t)
+  YK_CASE(YK_BF16, bf16_t, YK_F32, float, YK_F32, float)
+  YK_CASE(YK_BF16, bf16_t, YK_F32, float, YK_BF16, bf16_t)
+  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t, YK_F32, float)
+  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t, YK_BF16, bf16_t)
 #undef YK_CASE
   return yk_fail("add_rmsnorm: unsupported dtype combination");
 }
 
 // -------------------------------------------------- rotary + append to the paged cache
-// One block per token.  The token's row of `qkv` holds n_heads query heads, then
-// n_kv key heads, then n_kv value heads, each of head_dim elements.  Query heads are
-// rotated in place; key heads are rotated and stored at the token's slot of the key
-// pages [page][kv_head][page_size][head_dim]; value heads are stored transposed in the
-// value pages [page][kv_head][head_dim][page_size].  n_kv may be 0 (rotate queries only).
-// Rotation of a pair (a, b) by the angle of (position, pair index i):
-//   a' = a cos - b sin, b' = b cos + a sin; pairs are (i, i + rotary_dim/2) ("half")
-//   or (2i, 2i + 1) ("interleaved"); elements beyond rotary_dim pass unchanged.
-template <typename T>
-__global__ void rope_append_kernel(T* __restrict__ qkv, int row_stride, int n_heads, int n_kv,
-                                   int head_dim, const int32_t* __restrict__ positions,
+// One workgroup per (token, head).  The token's row of `src` holds n_heads query heads,
+// then n_kv key heads, then n_kv value heads, each of head_dim elements; with n_splits > 1
+// `src` holds the unreduced float32 K slices of the projection and they are summed here.
+// Query heads are rotated into `q_out` (which may be `src` itself); key heads are rotated
+// and stored at the token's slot of the key pages [page][kv_head][page_size][head_dim];
+// value heads are stored transposed in the value pages [page][kv_head][head_dim][page_size].
+// n_kv may be 0 (rotate queries only).  Rotation of a pair (a, b) by the angle of
+// (position, pair index i): a' = a cos - b sin, b' = b cos + a sin; pairs are
+// (i, i + rotary_dim/2) ("half") or (2i, 2i + 1) ("interleaved"); elements beyond
+// rotary_dim pass unchanged.
+template <typename TS, typename T>
+__global__ void rope_append_kernel(const TS* src, int n_splits, size_t split_stride,
+                                   int src_stride, T* q_out, int q_stride, int n_heads,
+                                   int n_kv, int head_dim, const int32_t* __restrict__ positions,
                                    const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                    int rotary_dim, int interleaved, int max_positions,
                                    T* __restrict__ k_cache, T* __restrict__ v_cache,
                                    const int32_t* __restrict__ slots, int page_size) {
-  const int n = blockIdx.x;
-  T* row = qkv + static_cast<size_t>(n) * row_stride;
+  const int n = blockIdx.x, h = blockIdx.y;
   int pos = positions[n];
   pos = pos < 0 ? 0 : (pos >= max_positions ? max_positions - 1 : pos);
   const int half = rotary_dim / 2;
   const float* cs = cos_t ? cos_t + static_cast<size_t>(pos) * half : nullptr;
   const float* sn = sin_t ? sin_t + static_cast<size_t>(pos) * half : nullptr;
-  size_t page = 0;
-  int off = 0;
-  if (n_kv > 0) {
+  const TS* row = src + static_cast<size_t>(n) * src_stride;
+  auto value = [&](int idx) {
+    float a = 0.f;
+    for (int s0 = 0; s0 < n_splits; s0 += 4) {  // four slices in flight, see add_rmsnorm
+      float d[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) d[j] = to_f32<TS>(row[static_cast<size_t>(min(s0 + j, n_splits - 1)) * split_stride + idx]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (s0 + j < n_splits) a += d[j];
+    }
+    return a;
+  };
+  const bool is_q = h < n_heads;
+  T* dst;
+  if (is_q) {
+    dst = q_out + static_cast<size_t>(n) * q_stride + static_cast<size_t>(h) * head_dim;
+  } else {
     const int slot = slots[n];
-    page = static_cast<size_t>(slot / page_size);
-    off = slot % page_size;
+    const size_t page = static_cast<size_t>(slot / page_size);
+    const int off = slot % page_size;
+    const int g = h - n_heads;
+    dst = k_cache + ((page * n_kv + g) * page_size + off) * head_dim;
+    // the value head of the same group, transposed
+    T* vdst = v_cache + (page * n_kv + g) * head_dim * page_size + off;
+    const int vbase = (n_heads + n_kv + g) * head_dim;
+    for (int d = threadIdx.x; d < head_dim; d += blockDim.x)
+      vdst[static_cast<size_t>(d) * page_size] = from_f32<T>(value(vbase + d));
   }
-  const size_t page_elems = static_cast<size_t>(n_kv) * page_size * head_dim;
-
-  // rotated pairs of the query and key heads
-  const int rot_heads = n_heads + n_kv;
-  for (int w = threadIdx.x; w < rot_heads * half; w += blockDim.x) {
-    const int h = w / half, i = w % half;
+  const int base = h * head_dim;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
     const int ia = interleaved ? 2 * i : i;
     const int ib = interleaved ? 2 * i + 1 : i + half;
-    T* head = row + static_cast<size_t>(h) * head_dim;
-    const float a = to_f32<T>(head[ia]), b = to_f32<T>(head[ib]);
+    const float a = value(base + ia), b = value(base + ib);
     const float c = cs[i], s = sn[i];
-    const T ra = from_f32<T>(a * c - b * s);
-    const T rb = from_f32<T>(b * c + a * s);
-    if (h < n_heads) {
-      head[ia] = ra;
-      head[ib] = rb;
-    } else {
-      const int g = h - n_heads;
-      T* dst = k_cache + page * page_elems + (static_cast<size_t>(g) * page_size + off) * head_dim;
-      dst[ia] = ra;
-      dst[ib] = rb;
-    }
+    dst[ia] = from_f32<T>(a * c - b * s);
+    dst[ib] = from_f32<T>(b * c + a * s);
   }
-  // key elements that do not rotate
-  const int rest = head_dim - rotary_dim;
-  for (int w = threadIdx.x; w < n_kv * rest; w += blockDim.x) {
-    const int g = w / rest, d = rotary_dim + w % rest;
-    const T* head = row + static_cast<size_t>(n_heads + g) * head_dim;
-    k_cache[page * page_elems + (static_cast<size_t>(g) * page_size + off) * head_dim + d] = head[d];
-  }
-  // values, transposed
-  for (int w = threadIdx.x; w < n_kv * head_dim; w += blockDim.x) {
-    const int g = w / head_dim, d = w % head_dim;
-    const T* head = row + static_cast<size_t>(n_heads + n_kv + g) * head_dim;
-    v_cache[page * page_elems + (static_cast<size_t>(g) * head_dim + d) * page_size + off] = head[d];
-  }
+  for (int d = rotary_dim + threadIdx.x; d < head_dim; d += blockDim.x) dst[d] = from_f32<T>(value(base + d));
 }
 
-extern "C" int yk_rope_append(void* qkv, int dtype, int n_tokens, int row_stride, int n_heads,
+// src_dtype/n_splits describe `src`; act_dtype is the dtype of q_out and of the cache.
+extern "C" int yk_rope_append(const void* src, int src_dtype, int n_splits, int src_stride,
+                              void* q_out, int act_dtype, int q_stride, int n_tokens, int n_heads,
                               int n_kv, int head_dim, const int32_t* positions, const float* cos_t,
                               const float* sin_t, int rotary_dim, int interleaved,
                               int max_positions, void* k_cache, void* v_cache,
@@ -202,62 +360,113 @@ extern "C" int yk_rope_append(void* qkv, int dtype, int n_tokens, int row_stride
   YK_REQUIRE(n_tokens >= 0 && n_heads >= 0 && n_kv >= 0 && head_dim > 0, "rope_append: bad sizes");
   YK_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0,
              "rope_append: rotary_dim must be even and at most head_dim");
-  YK_REQUIRE(row_stride >= (n_heads + 2 * n_kv) * head_dim, "rope_append: row stride too small");
+  YK_REQUIRE(src_stride >= (n_heads + 2 * n_kv) * head_dim, "rope_append: row stride too small");
+  YK_REQUIRE(q_stride >= n_heads * head_dim, "rope_append: query row stride too small");
   YK_REQUIRE(rotary_dim == 0 || (cos_t && sin_t && max_positions > 0), "rope_append: missing table");
   YK_REQUIRE(n_kv == 0 || (k_cache && v_cache && slots && page_size > 0), "rope_append: missing cache");
-  if (n_tokens == 0) return 0;
-  dim3 grid(n_tokens), block(256);
-  if (dtype == YK_F32)
-    rope_append_kernel<float><<<grid, block, 0, stream>>>(
-        static_cast<float*>(qkv), row_stride, n_heads, n_kv, head_dim, positions, cos_t, sin_t,
-        rotary_dim, interleaved, max_positions, static_cast<float*>(k_cache),
-        static_cast<float*>(v_cache), slots, page_size);
-  else if (dtype == YK_BF16)
-    rope_append_kernel<bf16_t><<<grid, block, 0, stream>>>(
-        static_cast<bf16_t*>(qkv), row_stride, n_heads, n_kv, head_dim, positions, cos_t, sin_t,
-        rotary_dim, interleaved, max_positions, static_cast<bf16_t*>(k_cache),
-        static_cast<bf16_t*>(v_cache), slots, page_size);
-  else
-    return yk_fail("rope_append: unsupported dtype");
-  return yk_check_launch("rope_append");
+  YK_REQUIRE(n_splits >= 1 && (n_splits == 1 || src_dtype == YK_F32), "rope_append: unreduced slices must be float32");
+  YK_REQUIRE(n_heads + n_kv <= 65535, "rope_append: too many heads for one launch");
+  if (n_tokens == 0 || n_heads + n_kv == 0) return 0;
+  dim3 grid(n_tokens, n_heads + n_kv), block(head_dim <= 128 ? 64 : 128);
+  const size_t stride = static_cast<size_t>(n_tokens) * src_stride;
+#define YK_CASE(SD, TS, AD, T)                                                                          \
+  if (src_dtype == SD && act_dtype == AD) {                                                             \
+    rope_append_kernel<TS, T><<<grid, block, 0, stream>>>(                                              \
+        static_cast<const TS*>(src), n_splits, stride, src_stride, static_cast<T*>(q_out), q_stride,    \
+        n_heads, n_kv, head_dim, positions, cos_t, sin_t, rotary_dim, interleaved, max_positions,       \
+        static_cast<T*>(k_cache), static_cast<T*>(v_cache), slots, page_size);                          \
+    return yk_check_launch("rope_append");                                                              \
+  }
+  YK_CASE(YK_F32, float, YK_F32, float)
+  YK_CASE(YK_F32, float, YK_BF16, bf16_t)
+  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t)
+#undef YK_CASE
+  return yk_fail("rope_append: unsupported dtype combination");
 }
 
 // ------------------------------------------------------------------ gated activation
-// out[n, j] = act(gu[n, j]) * gu[n, inter + j]; act 0 = silu, 1 = gelu (tanh form)
+// out[n, j] = act(gu[n, j]) * gu[n, inter + j]; act 0 = silu, 1 = gelu (tanh form).
+// With n_splits > 1, gu holds unreduced float32 K slices [n_splits][rows][2 * inter].
 __device__ __forceinline__ float act_silu(float z) { return z / (1.f + expf(-z)); }
 __device__ __forceinline__ float act_gelu_tanh(float z) {
   const float k = 0.7978845608028654f;  // sqrt(2/pi)
   return 0.5f * z * (1.f + tanhf(k * (z + 0.044715f * z * z * z)));
 }
+__device__ __forceinline__ float act_apply(float z, int act) { return act == 0 ? act_silu(z) : act_gelu_tanh(z); }
 
-template <typename T>
-__global__ void gated_act_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter,
-                                 size_t total, int act) {
+template <typename TS, typename TO>
+__global__ void gated_act_kernel(const TS* __restrict__ gu, int n_splits, size_t split_stride,
+                                 TO* __restrict__ out, int inter, size_t total, int act) {
   for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total;
        i += static_cast<size_t>(gridDim.x) * blockDim.x) {
     const size_t n = i / inter, j = i % inter;
-    const float g = to_f32<T>(gu[n * 2 * inter + j]);
-    const float u = to_f32<T>(gu[n * 2 * inter + inter + j]);
-    const float a = act == 0 ? act_silu(g) : act_gelu_tanh(g);
-    out[i] = from_f32<T>(a * u);
+    float g = 0.f, u = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+      g += to_f32<TS>(gu[s * split_stride + n * 2 * inter + j]);
+      u += to_f32<TS>(gu[s * split_stride + n * 2 * inter + inter + j]);
+    }
+    out[i] = from_f32<TO>(act_apply(g, act) * u);
   }
 }
 
-extern "C" int yk_gated_act(const void* gu, void* out, int dtype, int n_rows, int inter, int act,
+// four outputs per thread, no loop (inter a multiple of 4)
+template <typename TS, typename TO>
+__global__ void gated_act_vec_kernel(const TS* __restrict__ gu, int n_splits, size_t split_stride,
+                                     TO* __restrict__ out, int inter, size_t total_vec, int act) {
+  const size_t v = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
+  if (v >= total_vec) return;
+  const int per_row = inter / 4;
+  const size_t n = v / per_row;
+  const int j = static_cast<int>(v % per_row) * 4;
+  const TS* p = gu + n * 2 * inter + j;
+  float4 g = load4<TS>(p), u = load4<TS>(p + inter);
+  for (int s0 = 1; s0 < n_splits; s0 += 2) {  // two slices in flight
+    const int s1 = min(s0 + 1, n_splits - 1);
+    const float4 g2 = load4<TS>(p + s0 * split_stride), u2 = load4<TS>(p + s0 * split_stride + inter);
+    const float4 g3 = load4<TS>(p + s1 * split_stride), u3 = load4<TS>(p + s1 * split_stride + inter);
+    g.x += g2.x; g.y += g2.y; g.z += g2.z; g.w += g2.w;
+    u.x += u2.x; u.y += u2.y; u.z += u2.z; u.w += u2.w;
+    if (s0 + 1 < n_splits) {
+      g.x += g3.x; g.y += g3.y; g.z += g3.z; g.w += g3.w;
+      u.x += u3.x; u.y += u3.y; u.z += u3.z; u.w += u3.w;
+    }
+  }
+  float4 y;
+  y.x = act_apply(g.x, act) * u.x;
+  y.y = act_apply(g.y, act) * u.y;
+  y.z = act_apply(g.z, act) * u.z;
+  y.w = act_apply(g.w, act) * u.w;
+  store4<TO>(out + n * inter + j, y);
+}
+
+template <typename TS, typename TO>
+static int launch_gated_act(const void* gu, int n_splits, void* out, int n_rows, int inter, int act,
                             hipStream_t stream) {
+  const size_t stride = static_cast<size_t>(n_rows) * 2 * inter;
+  const bool aligned = inter % 4 == 0 && reinterpret_cast<uintptr_t>(gu) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  if (aligned) {
+    const size_t total_vec = static_cast<size_t>(n_rows) * (inter / 4);
+    YK_REQUIRE((total_vec + 255) / 256 < (1ull << 31), "gated_act: too large for one launch");
+    gated_act_vec_kernel<TS, TO><<<static_cast<unsigned>((total_vec + 255) / 256), 256, 0, stream>>>(
+        static_cast<const TS*>(gu), n_splits, stride, static_cast<TO*>(out), inter, total_vec, act);
+  } else {
+    const size_t total = static_cast<size_t>(n_rows) * inter;
+    const int grid = static_cast<int>(std::min<size_t>((total + 255) / 256, 65535));
+    gated_act_kernel<TS, TO><<<grid, 256, 0, stream>>>(static_cast<const TS*>(gu), n_splits, stride,
+                                                        static_cast<TO*>(out), inter, total, act);
+  }
+  return yk_check_launch("gated_act");
+}
+
+extern "C" int yk_gated_act(const void* gu, int src_dtype, int n_splits, void* out, int out_dtype,
+                            int n_rows, int inter, int act, hipStream_t stream) {
   YK_REQUIRE(n_rows >= 0 && inter > 0, "gated_act: bad sizes");
   YK_REQUIRE(act == 0 || act == 1, "gated_act: unknown activation");
+  YK_REQUIRE(n_splits >= 1 && (n_splits == 1 || src_dtype == YK_F32), "gated_act: unreduced slices must be float32");
   if (n_rows == 0) return 0;
-  const size_t total = static_cast<size_t>(n_rows) * inter;
-  const int block = 256;
-  const int grid = static_cast<int>(std::min<size_t>((total + block - 1) / block, 65535));
-  if (dtype == YK_F32)
-    gated_act_kernel<float><<<grid, block, 0, stream>>>(static_cast<const float*>(gu),
-                                                         static_cast<float*>(out), inter, total, act);
-  else if (dtype == YK_BF16)
-    gated_act_kernel<bf16_t><<<grid, block, 0, stream>>>(static_cast<const bf16_t*>(gu),
-                                                          static_cast<bf16_t*>(out), inter, total, act);
-  else
-    return yk_fail("gated_act: unsupported dtype");
-  return yk_check_launch("gated_act");
+  if (src_dtype == YK_F32 && out_dtype == YK_F32) return launch_gated_act<float, float>(gu, n_splits, out, n_rows, inter, act, stream);
+  if (src_dtype == YK_F32 && out_dtype == YK_BF16) return launch_gated_act<float, bf16_t>(gu, n_splits, out, n_rows, inter, act, stream);
+  if (src_dtype == YK_BF16 && out_dtype == YK_BF16) return launch_gated_act<bf16_t, bf16_t>(gu, n_splits, out, n_rows, inter, act, stream);
+  return yk_fail("gated_act: unsupported dtype combination");
 }

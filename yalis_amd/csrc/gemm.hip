@@ -100,6 +100,7 @@ extern "C" int yk_gemm_fma(const void* x, int x_dtype, const void* w, int w_dtyp
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 union Frag8 {
   u32x4_t u;
@@ -111,56 +112,91 @@ union Frag8 {
 //   C (16 x 16): lane holds C[4g .. 4g+3][r].
 // Here A = 16 rows of the weight (output features), B = 16 rows of x (tokens), so that
 // C[i][r] = y[token r][feature 4g + i].
-constexpr int SK_WAVES = 4;
+//
+// A workgroup of W waves owns 16*W weight rows (16 per wave) and 16*MT rows of x over one
+// slice of K (blockIdx.z); more waves share one staging of x, fewer give more workgroups.  K is walked in chunks of 256: the chunk of x is staged in LDS
+// once for all four waves; every wave streams its 16 weight rows straight from memory
+// into the A operand, 8 steps (512 contiguous bytes of every row) per chunk, with the next
+// chunk's loads issued before the current chunk is multiplied.  Measured on MI355X, a wave
+// that keeps 512 bytes of 16 rows in flight reads close to what contiguous streaming gives;
+// fewer bytes per row, or more rows per wave, read markedly slower.
+constexpr int SK_KC = 256;           // K elements per chunk
+constexpr int SK_STEPS = SK_KC / 32;  // matrix-core steps per chunk
+constexpr int SK_PAD = 8;            // bf16 elements of padding per LDS row (keeps 16-byte reads conflict-free)
 
-template <int MT>
-__global__ __launch_bounds__(SK_WAVES * 64) void gemm_mfma_skinny_kernel(
-    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, float* __restrict__ part, int M,
-    int N, int K, int ldx, int ldw, int k_chunk) {
+template <int MT, int W, typename TO>
+__global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, float* __restrict__ part,
+    TO* __restrict__ y, int M, int N, int K, int ldx, int ldw, int ldy, int k_block) {
+  __shared__ __attribute__((aligned(16))) bf16_t xs[16 * MT][SK_KC + SK_PAD];
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
   const int r = lane % 16, g = lane / 16;
-  const int n0 = (blockIdx.x * SK_WAVES + wave) * 16;
+  const int n0 = blockIdx.x * (16 * W) + 16 * wave;
   const int m0 = blockIdx.y * (16 * MT);
-  const int ks = blockIdx.z * k_chunk;
-  const int ke = min(K, ks + k_chunk);
-  if (n0 >= N) return;
+  const int kb0 = blockIdx.z * k_block;
+  const int kb1 = min(K, kb0 + k_block);
+
   f32x4_t acc[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  const bool row_ok = (n0 + r) < N;
-  const bf16_t* wrow = w + static_cast<size_t>(row_ok ? n0 + r : 0) * ldw;
-  const bf16_t* xrow[MT];
-  bool x_ok[MT];
+
+  // A row beyond N is read from the last row instead and never stored; K beyond the slice
+  // is read from the last 8 elements instead and meets zeros of x.  So the weight loads
+  // carry no conditions.
+  const bf16_t* wrow = w + static_cast<size_t>(min(n0 + r, N - 1)) * ldw;
+  const int k_last = K - 8;
+  Frag8 a_cur[SK_STEPS], a_next[SK_STEPS];
+#define SK_LOAD_A(A, KC0)                                                                    \
+  _Pragma("unroll") for (int u = 0; u < SK_STEPS; ++u)                                        \
+      A[u].u = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wrow + min((KC0) + 32 * u + 8 * g, k_last)));
+
+  SK_LOAD_A(a_next, kb0)
+  for (int kc = kb0; kc < kb1; kc += SK_KC) {
 #pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const int m = m0 + 16 * t + r;
-    x_ok[t] = m < M;
-    xrow[t] = x + static_cast<size_t>(x_ok[t] ? m : 0) * ldx;
-  }
-  const u32x4_t zero = {0u, 0u, 0u, 0u};
-  for (int kb = ks; kb < ke; kb += 32) {
-    // each lane group takes 8 of the step's 32; a chunk beyond ke feeds zeros
-    const int k = kb + 8 * g;
-    const bool k_ok = k < ke;
-    Frag8 a;
-    a.u = (row_ok && k_ok) ? *reinterpret_cast<const u32x4_t*>(wrow + k) : zero;
+    for (int u = 0; u < SK_STEPS; ++u) a_cur[u] = a_next[u];
+    if (kc + SK_KC < kb1) SK_LOAD_A(a_next, kc + SK_KC)
+    __syncthreads();  // the previous chunk of x has been read by every wave
+    // stage x[m0 .. m0+16*MT)[kc .. kc+256) as 16-byte pieces; zeros outside M and the slice
+    for (int e = threadIdx.x; e < 16 * MT * (SK_KC / 8); e += W * 64) {
+      const int row = e / (SK_KC / 8), piece = e % (SK_KC / 8);
+      const int m = m0 + row, k = kc + 8 * piece;
+      u32x4_t v = {0u, 0u, 0u, 0u};
+      if (m < M && k < kb1) v = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(m) * ldx + k);
+      *reinterpret_cast<u32x4_t*>(&xs[row][8 * piece]) = v;
+    }
+    __syncthreads();
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      Frag8 b;
-      b.u = (x_ok[t] && k_ok) ? *reinterpret_cast<const u32x4_t*>(xrow[t] + k) : zero;
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[t], 0, 0, 0);
+    for (int u = 0; u < SK_STEPS; ++u) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        Frag8 b;
+        b.u = *reinterpret_cast<const u32x4_t*>(&xs[16 * t + r][32 * u + 8 * g]);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_cur[u].v, b.v, acc[t], 0, 0, 0);
+      }
     }
   }
-  // part[split][m][n]
-  float* out = part + static_cast<size_t>(blockIdx.z) * M * N;
+#undef SK_LOAD_A
+
+  const bool to_part = part != nullptr;
+  float* pout = to_part ? part + static_cast<size_t>(blockIdx.z) * M * N : nullptr;
+  const int n = n0 + 4 * g;
+  if (n >= N) return;
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = m0 + 16 * t + r;
     if (m >= M) continue;
+    if (to_part && n + 3 < N && N % 4 == 0) {
+      *reinterpret_cast<f32x4_t*>(pout + static_cast<size_t>(m) * N + n) = acc[t];
+    } else {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int n = n0 + 4 * g + i;
-      if (n < N) out[static_cast<size_t>(m) * N + n] = acc[t][i];
+      for (int e = 0; e < 4; ++e) {
+        if (n + e < N) {
+          if (to_part)
+            pout[static_cast<size_t>(m) * N + n + e] = acc[t][e];
+          else
+            y[static_cast<size_t>(m) * ldy + n + e] = from_f32<TO>(acc[t][e]);
+        }
+      }
     }
   }
 }
@@ -178,58 +214,90 @@ __global__ void reduce_splits_kernel(const float* __restrict__ part, TO* __restr
   }
 }
 
-// How the skinny kernel would split K for these sizes (also tells the caller how much
-// workspace it needs: splits * M * N floats).
-extern "C" int yk_gemm_skinny_splits(int M, int N, int K) {
-  const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  const long tiles = static_cast<long>((N + 16 * SK_WAVES - 1) / (16 * SK_WAVES)) * ((M + 16 * mt - 1) / (16 * mt));
-  // aim at about 8 workgroups (32 waves) per compute unit, at least 256 of K per split
-  long want = (256L * 8 + tiles - 1) / tiles;
-  long max_by_k = std::max(1, K / 256);
-  long s = std::max(1L, std::min(want, max_by_k));
-  return static_cast<int>(std::min(s, 64L));
+static int skinny_mt(int M) { return M <= 16 ? 1 : (M <= 32 ? 2 : 4); }
+
+// How the skinny kernel cuts the work for these sizes: waves per workgroup (each wave owns
+// 16 weight rows), the number of K slices and the length of one (a multiple of 256).  The
+// aim is at least two workgroups per compute unit with as many waves sharing one staging
+// of x as that allows, and at least 512 of K per workgroup.  A caller that takes the
+// slices unreduced needs splits * M * N floats.
+static int skinny_plan(int M, int N, int K, int* waves_out, int* k_block_out) {
+  const int mt = skinny_mt(M);
+  const long mtiles = (M + 16 * mt - 1) / (16 * mt);
+  const long max_by_k = std::max(1, K / 512);
+  int waves = 4;
+  long s = 1;
+  for (int w : {16, 8, 4}) {
+    if (w > 4 * mt && w > 8) continue;  // many waves only pay when x is wide
+    const long tiles = static_cast<long>((N + 16 * w - 1) / (16 * w)) * mtiles;
+    const long want = (512 + tiles - 1) / tiles;
+    waves = w;
+    s = std::max(1L, std::min(want, max_by_k));
+    if (tiles * s >= 512 || w == 4) break;
+  }
+  s = std::min(s, 32L);
+  int k_block = static_cast<int>((K + s - 1) / s);
+  k_block = (k_block + SK_KC - 1) / SK_KC * SK_KC;
+  if (waves_out) *waves_out = waves;
+  if (k_block_out) *k_block_out = k_block;
+  return (K + k_block - 1) / k_block;
 }
 
+extern "C" int yk_gemm_skinny_splits(int M, int N, int K) { return skinny_plan(M, N, K, nullptr, nullptr); }
+
+template <typename TO>
+static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, int M, int N, int K,
+                         int ldx, int ldw, int ldy, int waves, int k_block, int splits, hipStream_t stream) {
+  const int mt = skinny_mt(M);
+  dim3 grid((N + 16 * waves - 1) / (16 * waves), (M + 16 * mt - 1) / (16 * mt), splits);
+  YK_REQUIRE(grid.y <= 65535, "gemm_mfma_skinny: too many rows for one launch");
+  dim3 block(waves * 64);
+#define SK_GO(MT_, W_)                                                                                   \
+  if (mt == MT_ && waves == W_) {                                                                       \
+    gemm_mfma_skinny_kernel<MT_, W_, TO><<<grid, block, 0, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block); \
+    return yk_check_launch("gemm_mfma_skinny");                                                         \
+  }
+  SK_GO(1, 4) SK_GO(1, 8) SK_GO(2, 4) SK_GO(2, 8) SK_GO(4, 4) SK_GO(4, 8) SK_GO(4, 16)
+#undef SK_GO
+  return yk_fail("gemm_mfma_skinny: no kernel for this plan");
+}
+
+// keep_splits != 0: leave the K slices unreduced in `workspace` ([splits][M][N] float32) for
+// a consumer that sums them itself (y is not written unless there is a single slice and
+// y is given).  Returns the number of slices written to the workspace (0: y holds the
+// result), or a negative number on error.
 extern "C" int yk_gemm_mfma_skinny(const void* x, const void* w, void* y, int y_dtype,
                                    float* workspace, size_t workspace_floats, int M, int N, int K,
-                                   int ldx, int ldw, int ldy, hipStream_t stream) {
+                                   int ldx, int ldw, int ldy, int keep_splits,
+                                   hipStream_t stream) {
   YK_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_mfma_skinny: bad sizes");
-  YK_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0,
+  YK_REQUIRE(K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0,
              "gemm_mfma_skinny: K and the leading dimensions must be multiples of 8");
   YK_REQUIRE((reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(w) % 16 == 0),
              "gemm_mfma_skinny: operands must be 16-byte aligned");
   YK_REQUIRE(ldx >= K && ldw >= K && ldy >= N, "gemm_mfma_skinny: leading dimensions too small");
+  YK_REQUIRE(y_dtype == YK_F32 || y_dtype == YK_BF16, "gemm_mfma_skinny: unsupported output dtype");
   if (M == 0) return 0;
-  const int splits = yk_gemm_skinny_splits(M, N, K);
-  int k_chunk = (K + splits - 1) / splits;
-  k_chunk = (k_chunk + 31) / 32 * 32;
-  const int real_splits = (K + k_chunk - 1) / k_chunk;
-  const bool direct = real_splits == 1 && y_dtype == YK_F32 && ldy == N;
-  YK_REQUIRE(direct || workspace_floats >= static_cast<size_t>(real_splits) * M * N,
-             "gemm_mfma_skinny: workspace too small");
-  float* part = direct ? static_cast<float*>(y) : workspace;
-  const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  dim3 grid((N + 16 * SK_WAVES - 1) / (16 * SK_WAVES), (M + 16 * mt - 1) / (16 * mt), real_splits);
-  YK_REQUIRE(grid.y <= 65535, "gemm_mfma_skinny: too many rows for one launch");
-  dim3 block(SK_WAVES * 64);
+  int k_block = 0, waves = 4;
+  const int splits = skinny_plan(M, N, K, &waves, &k_block);
   const bf16_t* xp = static_cast<const bf16_t*>(x);
   const bf16_t* wp = static_cast<const bf16_t*>(w);
-  if (mt == 1)
-    gemm_mfma_skinny_kernel<1><<<grid, block, 0, stream>>>(xp, wp, part, M, N, K, ldx, ldw, k_chunk);
-  else if (mt == 2)
-    gemm_mfma_skinny_kernel<2><<<grid, block, 0, stream>>>(xp, wp, part, M, N, K, ldx, ldw, k_chunk);
-  else
-    gemm_mfma_skinny_kernel<4><<<grid, block, 0, stream>>>(xp, wp, part, M, N, K, ldx, ldw, k_chunk);
-  if (yk_check_launch("gemm_mfma_skinny")) return -1;
-  if (direct) return 0;
+  if (splits == 1 && !keep_splits) {
+    int rc = y_dtype == YK_F32
+                 ? launch_skinny<float>(xp, wp, nullptr, static_cast<float*>(y), M, N, K, ldx, ldw, ldy, waves, k_block, 1, stream)
+                 : launch_skinny<bf16_t>(xp, wp, nullptr, static_cast<bf16_t*>(y), M, N, K, ldx, ldw, ldy, waves, k_block, 1, stream);
+    return rc;
+  }
+  YK_REQUIRE(workspace && workspace_floats >= static_cast<size_t>(splits) * M * N,
+             "gemm_mfma_skinny: workspace too small");
+  if (launch_skinny<float>(xp, wp, workspace, nullptr, M, N, K, ldx, ldw, ldy, waves, k_block, splits, stream)) return -1;
+  if (keep_splits) return splits;
   const size_t total = static_cast<size_t>(M) * N;
   const int rb = 256;
   const int rg = static_cast<int>(std::min<size_t>((total + rb - 1) / rb, 65535));
   if (y_dtype == YK_F32)
-    reduce_splits_kernel<float><<<rg, rb, 0, stream>>>(part, static_cast<float*>(y), M, N, ldy, real_splits);
-  else if (y_dtype == YK_BF16)
-    reduce_splits_kernel<bf16_t><<<rg, rb, 0, stream>>>(part, static_cast<bf16_t*>(y), M, N, ldy, real_splits);
+    reduce_splits_kernel<float><<<rg, rb, 0, stream>>>(workspace, static_cast<float*>(y), M, N, ldy, splits);
   else
-    return yk_fail("gemm_mfma_skinny: unsupported output dtype");
+    reduce_splits_kernel<bf16_t><<<rg, rb, 0, stream>>>(workspace, static_cast<bf16_t*>(y), M, N, ldy, splits);
   return yk_check_launch("reduce_splits");
 }

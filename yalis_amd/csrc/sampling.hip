@@ -83,10 +83,56 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ 
   if (threadIdx.x == 0) out[blockIdx.x] = best.i == 0x7fffffff ? 0 : best.i;
 }
 
+// Large vocabularies, few rows: first the best of each of ARGMAX_CHUNKS slices of the
+// row, then the best of those (the lowest index still wins ties: slices are in order).
+constexpr int ARGMAX_CHUNKS = 32;
+
+__global__ __launch_bounds__(256) void argmax_part_kernel(const float* __restrict__ logits,
+                                                          float* __restrict__ part_v,
+                                                          int32_t* __restrict__ part_i, int vocab) {
+  __shared__ ArgMax scratch[17];
+  const float* row = logits + static_cast<size_t>(blockIdx.x) * vocab;
+  const int per = (vocab + ARGMAX_CHUNKS - 1) / ARGMAX_CHUNKS;
+  const int lo = blockIdx.y * per, hi = min(vocab, lo + per);
+  ArgMax best{-INFINITY, 0x7fffffff};
+  for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) best = better(best, ArgMax{row[i], i});
+  best = block_argmax(best, scratch);
+  if (threadIdx.x == 0) {
+    part_v[blockIdx.x * ARGMAX_CHUNKS + blockIdx.y] = best.v;
+    part_i[blockIdx.x * ARGMAX_CHUNKS + blockIdx.y] = best.i;
+  }
+}
+
+__global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restrict__ part_v,
+                                                          const int32_t* __restrict__ part_i,
+                                                          int32_t* __restrict__ out) {
+  const int lane = threadIdx.x;
+  ArgMax x = lane < ARGMAX_CHUNKS ? ArgMax{part_v[blockIdx.x * ARGMAX_CHUNKS + lane], part_i[blockIdx.x * ARGMAX_CHUNKS + lane]}
+                                  : ArgMax{-INFINITY, 0x7fffffff};
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    ArgMax y;
+    y.v = __shfl_xor(x.v, o, 64);
+    y.i = __shfl_xor(x.i, o, 64);
+    x = better(x, y);
+  }
+  if (lane == 0) out[blockIdx.x] = x.i == 0x7fffffff ? 0 : x.i;
+}
+
+// workspace: n_rows * 32 floats and as many ints (may be null for small vocabularies)
 extern "C" int yk_argmax(const float* logits, int32_t* out, int n_rows, int vocab,
-                         hipStream_t stream) {
+                         float* workspace, size_t workspace_floats, hipStream_t stream) {
   YK_REQUIRE(n_rows >= 0 && vocab > 0, "argmax: bad sizes");
   if (n_rows == 0) return 0;
+  const size_t need = static_cast<size_t>(n_rows) * ARGMAX_CHUNKS * 2;
+  if (vocab >= 8192 && workspace && workspace_floats >= need && n_rows <= 65535) {
+    float* pv = workspace;
+    int32_t* pi = reinterpret_cast<int32_t*>(workspace + static_cast<size_t>(n_rows) * ARGMAX_CHUNKS);
+    argmax_part_kernel<<<dim3(n_rows, ARGMAX_CHUNKS), 256, 0, stream>>>(logits, pv, pi, vocab);
+    if (yk_check_launch("argmax_part")) return -1;
+    argmax_final_kernel<<<n_rows, 64, 0, stream>>>(pv, pi, out);
+    return yk_check_launch("argmax_final");
+  }
   argmax_kernel<<<n_rows, 1024, 0, stream>>>(logits, out, vocab);
   return yk_check_launch("argmax");
 }

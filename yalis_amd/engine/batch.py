@@ -45,7 +45,9 @@ class HostBatch:
     extra: Dict[str, np.ndarray] = field(default_factory=dict)
 
 
-def build_host_batch(spans: Sequence[SeqSpan], n_groups: int, page_size: int) -> HostBatch:
+def build_host_batch(spans: Sequence[SeqSpan], n_groups: int, page_size: int, table_widths: Sequence[int] = ()) -> HostBatch:
+    """``table_widths``: block-table width per cache group when it must not depend on the
+    batch (a captured graph); by default the widest table of the batch."""
     if not spans:
         raise ValueError("a step needs at least one request")
     qlen = np.array([len(s.tokens) for s in spans], dtype=np.int32)
@@ -70,6 +72,10 @@ def build_host_batch(spans: Sequence[SeqSpan], n_groups: int, page_size: int) ->
     slots: List[np.ndarray] = []
     for g in range(n_groups):
         width = max(1, max(len(s.block_tables[g]) for s in spans))
+        if table_widths:
+            if table_widths[g] < width:
+                raise ValueError(f"block tables of group {g} need {width} columns, {table_widths[g]} were fixed")
+            width = table_widths[g]
         bt = np.full((n, width), -1, dtype=np.int32)
         for i, s in enumerate(spans):
             t = np.asarray(s.block_tables[g], dtype=np.int32)

@@ -99,6 +99,23 @@ class _Uploader:
         return dev
 
 
+class _DecodeGraph:
+    """One captured decode step: the graph, the integer buffer its kernels read, the
+    logits it writes, and what must stay alive while it may be replayed."""
+
+    def __init__(self, graph, ints, layout, logits, keep):
+        self.graph = graph
+        self.ints = ints
+        self.layout = layout
+        self.logits = logits
+        self.keep = keep
+
+
+# Decode steps of up to this many requests are captured as graphs (larger batches run
+# their products through the vendor library, which is left out of captures).
+GRAPH_MAX_SEQS = 64
+
+
 class ModelRunner:
     def __init__(self, model, config: EngineConfig):
         self.model = model
@@ -121,6 +138,15 @@ class ModelRunner:
         self.cached: Dict[int, int] = {}  # request -> tokens in the cache
         self._uploader = _Uploader(config.device)
         self.last_host_batch: Optional[HostBatch] = None
+        # Steps that hold single tokens only are launch-bound: each shape of such a step
+        # is captured once as a HIP graph and replayed (the reference gets the same from
+        # torch.compile's reduce-overhead mode, yalis/engine.py:44-48,109).
+        self.use_graphs = (
+            torch.device(config.device).type == "cuda" and config.decode_graphs and model.graph_capturable
+        )
+        self._graphs: Dict[Tuple, _DecodeGraph] = {}
+        self._table_widths = [-(-config.max_model_len // self.page_size) for _ in self.group_shapes]
+        self.graph_replays = 0
 
     # ----------------------------------------------------------------- requests
     def admit(self, request: int) -> bool:
@@ -179,18 +205,58 @@ class ModelRunner:
                     want=e.want,
                 )
             )
-        hb = build_host_batch(spans, len(self.group_shapes), self.page_size)
-        arrays = named_arrays(hb, self.builders)
-        buf, layout = pack(arrays)
-        dev = self._uploader.upload(buf)
-        views = {
-            name: dev[off : off + int(np.prod(shape, dtype=np.int64))].view(*shape)
-            for name, (off, shape) in layout.items()
-        }
-        ctx = StepContext(hb, views, self.sites, self.rt)
-        self.last_host_batch = hb
-        logits = self.model.forward(ctx)
+        decode_only = all(len(s.tokens) == 1 and len(s.want) == 1 for s in spans)
+        if self.use_graphs and decode_only and len(spans) <= GRAPH_MAX_SEQS:
+            logits = self._graph_step(spans)
+        else:
+            hb = build_host_batch(spans, len(self.group_shapes), self.page_size)
+            buf, layout = pack(named_arrays(hb, self.builders))
+            dev = self._uploader.upload(buf)
+            ctx = StepContext(hb, self._views(dev, layout), self.sites, self.rt)
+            self.last_host_batch = hb
+            logits = self.model.forward(ctx)
         for e in entries:
             self.cached[e.request] += len(e.tokens)
             self.pages.advance(e.request, self.cached[e.request])
         return logits
+
+    @staticmethod
+    def _views(dev: torch.Tensor, layout) -> Dict[str, torch.Tensor]:
+        return {
+            name: dev[off : off + int(np.prod(shape, dtype=np.int64))].view(*shape)
+            for name, (off, shape) in layout.items()
+        }
+
+    def _graph_step(self, spans) -> torch.Tensor:
+        """A step of single tokens through a captured graph.  The graph is keyed by what
+        fixes its launches: the number of requests and the power-of-two bucket of the
+        longest context (it decides how far attention splits the keys).  Block tables
+        have the engine's full width, so the integer buffer keeps one layout."""
+        hb = build_host_batch(spans, len(self.group_shapes), self.page_size, self._table_widths)
+        bucket = 256
+        while bucket < hb.max_ctx:
+            bucket *= 2
+        hb.max_ctx = bucket
+        buf, layout = pack(named_arrays(hb, self.builders))
+        key = (hb.n_seqs, bucket)
+        entry = self._graphs.get(key)
+        self.last_host_batch = hb
+        if entry is None:
+            ints = torch.empty(buf.size, dtype=torch.int32, device=self.config.device)
+            ints.copy_(self._uploader.upload(buf))
+            ctx = StepContext(hb, self._views(ints, layout), self.sites, self.rt)
+            ops = self.rt.ops
+            ops.reserve_workspaces(hb.n_seqs)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                logits = self.model.forward(ctx)
+            entry = _DecodeGraph(graph, ints, layout, logits, ops.workspaces())
+            self._graphs[key] = entry
+        else:
+            if layout != entry.layout:
+                raise RuntimeError("a decode step's integer arrays changed shape under a captured graph")
+            entry.ints.copy_(self._uploader.upload(buf), non_blocking=True)
+        entry.graph.replay()
+        self.graph_replays += 1
+        return entry.logits

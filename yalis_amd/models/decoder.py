@@ -65,6 +65,8 @@ class DecoderModel:
             self.blocks.append(BLOCKS.get(ls.block)(n1, mixer, n2, ffn))
 
         self.cache_groups, self.state_needs, self.sites = self._plan_memory()
+        # a step may be replayed from a captured graph only if every part allows it
+        self.graph_capturable = all(getattr(p, "graph_capturable", False) for p in self.all_parts())
 
     # ------------------------------------------------------------------ memory plan
     def _plan_memory(self):

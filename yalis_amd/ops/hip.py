@@ -44,21 +44,22 @@ _SIGNATURES = {
     "yk_abi_version": ([], _c_int),
     "yk_embed": ([_vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_add_rmsnorm": (
-        [_vp, _vp, _c_int, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_float, _c_int, _vp],
+        [_vp, _vp, _c_int, _c_int, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp],
         _c_int,
     ),
     "yk_rope_append": (
-        [_vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _c_int, _c_int, _c_int, _vp, _vp, _vp, _c_int, _vp],
+        [_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp,
+         _c_int, _c_int, _c_int, _vp, _vp, _vp, _c_int, _vp],
         _c_int,
     ),
-    "yk_gated_act": ([_vp, _vp, _c_int, _c_int, _c_int, _c_int, _vp], _c_int),
+    "yk_gated_act": ([_vp, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_gemm_fma": (
         [_vp, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
         _c_int,
     ),
     "yk_gemm_skinny_splits": ([_c_int, _c_int, _c_int], _c_int),
     "yk_gemm_mfma_skinny": (
-        [_vp, _vp, _vp, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
+        [_vp, _vp, _vp, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
         _c_int,
     ),
     "yk_attn_generic": (
@@ -73,7 +74,7 @@ _SIGNATURES = {
         [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _vp, _c_size_t, _vp],
         _c_int,
     ),
-    "yk_argmax": ([_vp, _vp, _c_int, _c_int, _vp], _c_int),
+    "yk_argmax": ([_vp, _vp, _c_int, _c_int, _vp, _c_size_t, _vp], _c_int),
     "yk_sample": ([_vp, _vp, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _vp], _c_int),
 }
 
@@ -81,7 +82,29 @@ _SIGNATURES = {
 # above it the vendor library does.
 SKINNY_MAX_ROWS = 64
 # Waves the attention launch aims at when it decides how far to split the keys.
-ATTN_TARGET_WAVES = 1024
+ATTN_TARGET_WAVES = 2048
+
+
+class SplitSum:
+    """The unreduced K slices of a product: float32 [slices, rows, columns] whose sum over
+    the first axis is the result.  The kernels that consume a projection (norm, rotary +
+    append, gated activation) add the slices themselves, which saves a pass over memory
+    and a rounding.  It lives in the library's workspace: consume it before the next
+    product is launched."""
+
+    def __init__(self, tensor: torch.Tensor):
+        self.tensor = tensor
+        self.shape = tuple(tensor.shape[1:])
+        self.n_splits = tensor.shape[0]
+        self.dtype = torch.float32
+        self.device = tensor.device
+
+    def reduce(self) -> torch.Tensor:
+        """The product itself, float32 (for code that does not add the slices itself)."""
+        return self.tensor.sum(0)
+
+    def float(self) -> torch.Tensor:
+        return self.reduce()
 
 
 class HipOps:
@@ -95,9 +118,10 @@ class HipOps:
             fn = getattr(self.lib, name)
             fn.argtypes = args
             fn.restype = res
-        if self.lib.yk_abi_version() != 1:
+        if self.lib.yk_abi_version() != 2:
             raise KernelError("kernel library and bindings disagree; rebuild (python -c 'import __graft_entry__ as g; g.build()')")
-        self._workspace: Optional[torch.Tensor] = None
+        self._workspace: Optional[torch.Tensor] = None  # attention splits, argmax parts
+        self._gemm_workspace: Optional[torch.Tensor] = None  # K slices of products
 
     # ------------------------------------------------------------------ helpers
     def _stream(self) -> int:
@@ -110,8 +134,23 @@ class HipOps:
     def _ws(self, floats: int) -> torch.Tensor:
         """Float32 scratch that grows and is reused (stream order keeps uses apart)."""
         if self._workspace is None or self._workspace.numel() < floats:
-            self._workspace = torch.empty(max(floats, 1 << 20), dtype=torch.float32, device=self.device)
+            self._workspace = torch.empty(max(floats, 1 << 22), dtype=torch.float32, device=self.device)
         return self._workspace
+
+    def _gemm_ws(self, floats: int) -> torch.Tensor:
+        if self._gemm_workspace is None or self._gemm_workspace.numel() < floats:
+            self._gemm_workspace = torch.empty(max(floats, 1 << 22), dtype=torch.float32, device=self.device)
+        return self._gemm_workspace
+
+    def reserve_workspaces(self, rows: int) -> None:
+        """Make the scratch buffers large enough for steps of ``rows`` tokens before a
+        graph is captured (a buffer must not be replaced while a capture is running)."""
+        self._ws(1 << 24)
+        self._gemm_ws(1 << 24)
+
+    def workspaces(self):
+        """The scratch buffers in use, for whoever must keep them alive (a captured graph)."""
+        return (self._workspace, self._gemm_workspace)
 
     @staticmethod
     def _rows(t: torch.Tensor, what: str) -> None:
@@ -151,14 +190,19 @@ class HipOps:
         width = residual.shape[1]
         if weight.numel() != width:
             raise KernelError(f"norm weight has {weight.numel()} elements, rows have {width}")
-        if delta is not None and (tuple(delta.shape) != tuple(residual.shape) or not delta.is_contiguous()):
+        n_splits = 1
+        if isinstance(delta, SplitSum):
+            n_splits, delta = delta.n_splits, delta.tensor
+            if tuple(delta.shape[1:]) != tuple(residual.shape):
+                raise KernelError(f"delta {tuple(delta.shape[1:])} does not match the residual {tuple(residual.shape)}")
+        elif delta is not None and (tuple(delta.shape) != tuple(residual.shape) or not delta.is_contiguous()):
             raise KernelError(f"delta {tuple(delta.shape)} does not match the residual {tuple(residual.shape)}")
         out = torch.empty((n_out, width), dtype=out_dtype, device=residual.device)
         self._check(
             self.lib.yk_add_rmsnorm(
-                residual.data_ptr(), _ptr(delta), 0 if delta is None else _code(delta.dtype),
+                residual.data_ptr(), _ptr(delta), 0 if delta is None else _code(delta.dtype), n_splits,
                 _ptr(rows), weight.data_ptr(), _code(weight.dtype), out.data_ptr(), _code(out_dtype),
-                n_out, width, float(eps), int(bool(unit_offset)), self._stream(),
+                n_out, residual.shape[0], width, float(eps), int(bool(unit_offset)), self._stream(),
             )
         )
         return out
@@ -170,8 +214,9 @@ class HipOps:
         return self._norm(residual, delta, rows, weight, eps, unit_offset, out_dtype, rows.numel())
 
     # --------------------------------------------------------------------- linear
-    def linear(self, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-        """x [M, K] . w [N, K]^T -> [M, N]."""
+    def linear(self, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, partial_ok: bool = False):
+        """x [M, K] . w [N, K]^T -> [M, N].  With ``partial_ok`` the result may come as a
+        ``SplitSum`` for a consumer that adds the slices itself."""
         self._rows(x, "linear input")
         self._rows(w, "linear weight")
         m, k = x.shape
@@ -184,7 +229,7 @@ class HipOps:
         aligned = k % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
         if x.dtype == bf and w.dtype == bf and aligned:
             if m <= SKINNY_MAX_ROWS or out_dtype != bf:
-                return self.gemm_mfma_skinny(x, w, out_dtype)
+                return self.gemm_mfma_skinny(x, w, out_dtype, partial_ok)
             return torch.matmul(x, w.t())  # vendor library, bfloat16 in and out
         return self.gemm_fma(x, w, out_dtype)
 
@@ -200,27 +245,44 @@ class HipOps:
         )
         return y
 
-    def gemm_mfma_skinny(self, x, w, out_dtype):
+    def gemm_mfma_skinny(self, x, w, out_dtype, partial_ok: bool = False):
         m, k = x.shape
         n = w.shape[0]
-        y = torch.empty((m, n), dtype=out_dtype, device=x.device)
         splits = self.lib.yk_gemm_skinny_splits(m, n, k)
-        ws = self._ws(splits * m * n)
-        self._check(
-            self.lib.yk_gemm_mfma_skinny(
-                x.data_ptr(), w.data_ptr(), y.data_ptr(), _code(out_dtype), ws.data_ptr(), ws.numel(),
-                m, n, k, x.stride(0), w.stride(0), n, self._stream(),
-            )
+        keep = bool(partial_ok and splits > 1)
+        ws = self._gemm_ws(splits * m * n) if splits > 1 else None
+        y = None if keep else torch.empty((m, n), dtype=out_dtype, device=x.device)
+        rc = self.lib.yk_gemm_mfma_skinny(
+            x.data_ptr(), w.data_ptr(), _ptr(y), _code(out_dtype), _ptr(ws), 0 if ws is None else ws.numel(),
+            m, n, k, x.stride(0), w.stride(0), n, int(keep), self._stream(),
         )
+        if rc < 0:
+            raise KernelError(self.lib.yk_last_error().decode())
+        if keep:
+            return SplitSum(ws[: splits * m * n].view(splits, m, n))
         return y
 
     # ------------------------------------------------- rotary + append to the cache
     def rope_append(self, qkv, n_heads, n_kv, head_dim, positions, cos, sin, rotary_dim,
-                    interleaved, k_cache, v_cache, slots, page_size):
-        self._rows(qkv, "qkv")
-        n = qkv.shape[0]
-        if qkv.shape[1] != (n_heads + 2 * n_kv) * head_dim:
-            raise KernelError(f"qkv rows have {qkv.shape[1]} elements, expected {(n_heads + 2 * n_kv) * head_dim}")
+                    interleaved, k_cache, v_cache, slots, page_size) -> torch.Tensor:
+        """Rotates the query heads, appends rotated keys and values to the pages; returns
+        the tensor whose rows start with the rotated queries (``qkv`` itself, rotated in
+        place, or a new [N, n_heads * head_dim] tensor when ``qkv`` is a SplitSum)."""
+        n_splits = 1
+        src = qkv
+        if isinstance(qkv, SplitSum):
+            n_splits, src = qkv.n_splits, qkv.tensor
+            n, cols = qkv.shape
+            act = k_cache.dtype if n_kv else torch.bfloat16
+            q_out = torch.empty((n, n_heads * head_dim), dtype=act, device=src.device)
+            src_stride = cols
+        else:
+            self._rows(qkv, "qkv")
+            n, cols = qkv.shape
+            q_out = qkv
+            src_stride = qkv.stride(0)
+        if cols != (n_heads + 2 * n_kv) * head_dim:
+            raise KernelError(f"qkv rows have {cols} elements, expected {(n_heads + 2 * n_kv) * head_dim}")
         if positions.numel() != n or (n_kv > 0 and slots.numel() != n):
             raise KernelError("positions/slots do not match the number of tokens")
         max_pos = 0
@@ -229,25 +291,28 @@ class HipOps:
                 raise KernelError("rotary tables must be float32 [positions, rotary_dim/2]")
             max_pos = cos.shape[0]
         if n_kv > 0:
-            if k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype:
+            if k_cache.dtype != q_out.dtype or v_cache.dtype != q_out.dtype:
                 raise KernelError("cache and activations differ in dtype")
             if tuple(k_cache.shape[1:]) != (n_kv, page_size, head_dim) or tuple(v_cache.shape[1:]) != (n_kv, head_dim, page_size):
                 raise KernelError(f"cache pages have shapes {tuple(k_cache.shape)}, {tuple(v_cache.shape)}")
         self._check(
             self.lib.yk_rope_append(
-                qkv.data_ptr(), _code(qkv.dtype), n, qkv.stride(0), n_heads, n_kv, head_dim,
+                src.data_ptr(), _code(src.dtype), n_splits, src_stride, q_out.data_ptr(), _code(q_out.dtype),
+                q_out.stride(0), n, n_heads, n_kv, head_dim,
                 positions.data_ptr(), _ptr(cos) if rotary_dim else None, _ptr(sin) if rotary_dim else None,
                 rotary_dim, int(bool(interleaved)), max_pos,
                 _ptr(k_cache) if n_kv else None, _ptr(v_cache) if n_kv else None,
                 _ptr(slots) if n_kv else None, page_size, self._stream(),
             )
         )
+        return q_out
 
     # ------------------------------------------------------------------ attention
-    def attention(self, qkv, n_heads, n_kv_rows, n_kv, head_dim, k_cache, v_cache, page_size,
+    def attention(self, qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size,
                   scale, window, ctx, group, tiles) -> torch.Tensor:
-        """Queries are the first n_heads heads of each row of ``qkv``; keys and values
-        come from the cache through the block table of ``group``."""
+        """Queries are the first n_heads heads of each row of ``qkv`` (whatever follows
+        them in the row is skipped); keys and values come from the cache through the
+        block table of ``group``."""
         self._rows(qkv, "qkv")
         n = qkv.shape[0]
         bt = ctx.arrays[f"block_table_g{group}"]
@@ -290,17 +355,29 @@ class HipOps:
         return out
 
     # ----------------------------------------------------------------- activation
-    def gated_act(self, gu: torch.Tensor, activation: str) -> torch.Tensor:
-        self._rows(gu, "gate/up")
-        if not gu.is_contiguous() or gu.shape[1] % 2:
-            raise KernelError("gate/up must be contiguous with an even number of columns")
+    def gated_act(self, gu, activation: str, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        n_splits = 1
+        src = gu
+        if isinstance(gu, SplitSum):
+            n_splits, src = gu.n_splits, gu.tensor
+            rows, cols = gu.shape
+            out_dtype = out_dtype or torch.bfloat16
+        else:
+            self._rows(gu, "gate/up")
+            if not gu.is_contiguous():
+                raise KernelError("gate/up must be contiguous")
+            rows, cols = gu.shape
+            out_dtype = out_dtype or gu.dtype
+        if cols % 2:
+            raise KernelError("gate/up must have an even number of columns")
         act = {"silu": 0, "gelu_tanh": 1}.get(activation)
         if act is None:
             raise KernelError(f"unknown activation {activation!r}")
-        inter = gu.shape[1] // 2
-        out = torch.empty((gu.shape[0], inter), dtype=gu.dtype, device=gu.device)
+        inter = cols // 2
+        out = torch.empty((rows, inter), dtype=out_dtype, device=src.device)
         self._check(
-            self.lib.yk_gated_act(gu.data_ptr(), out.data_ptr(), _code(gu.dtype), gu.shape[0], inter, act, self._stream())
+            self.lib.yk_gated_act(src.data_ptr(), _code(src.dtype), n_splits, out.data_ptr(), _code(out_dtype),
+                                  rows, inter, act, self._stream())
         )
         return out
 
@@ -309,7 +386,9 @@ class HipOps:
         if logits.dtype != torch.float32 or not logits.is_contiguous() or logits.dim() != 2:
             raise KernelError("argmax takes contiguous float32 logits [rows, vocab]")
         out = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device)
-        self._check(self.lib.yk_argmax(logits.data_ptr(), out.data_ptr(), logits.shape[0], logits.shape[1], self._stream()))
+        ws = self._ws(64 * logits.shape[0])
+        self._check(self.lib.yk_argmax(logits.data_ptr(), out.data_ptr(), logits.shape[0], logits.shape[1],
+                                       ws.data_ptr(), ws.numel(), self._stream()))
         return out
 
     def sample(self, logits, temperature, top_k, top_p, seeds, draws) -> torch.Tensor:

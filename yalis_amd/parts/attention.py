@@ -26,6 +26,8 @@ from .base import POSITIONS, KVNeed, Mixer, Runtime, register_mixer
 
 @register_mixer("attention")
 class Attention(Mixer):
+
+    graph_capturable = True
     def __init__(self, params, rt: Runtime):
         super().__init__(params, rt)
         self.prefix = params["prefix"]
@@ -86,14 +88,14 @@ class Attention(Mixer):
         if site.owns_cache:
             if not self.projects_kv:
                 raise RuntimeError(f"{self.prefix}: run entry owns a cache but the layer has no k/v projections")
-            qkv = ops.linear(h, self.w_qkv, self.rt.act_dtype)
+            qkv = ops.linear(h, self.w_qkv, self.rt.act_dtype, partial_ok=True)
             n_kv_rows = self.n_kv
         else:
-            qkv = ops.linear(h, self.w_q, self.rt.act_dtype)
+            qkv = ops.linear(h, self.w_q, self.rt.act_dtype, partial_ok=True)
             n_kv_rows = 0
         k_cache, v_cache = site.kv()
         pos = self.position
-        ops.rope_append(
+        q = ops.rope_append(
             qkv,
             self.n_heads,
             n_kv_rows,
@@ -109,9 +111,8 @@ class Attention(Mixer):
             self.rt.page_size,
         )
         out = ops.attention(
-            qkv,
+            q,
             self.n_heads,
-            n_kv_rows,
             self.n_kv,
             self.head_dim,
             k_cache,
@@ -123,4 +124,4 @@ class Attention(Mixer):
             site.group,
             ctx.arrays[f"attention_tiles_{self.tokens_per_tile}"],
         )
-        return ops.linear(out, self.w_o, self.rt.act_dtype)
+        return ops.linear(out, self.w_o, self.rt.act_dtype, partial_ok=True)

@@ -55,6 +55,11 @@ class StateNeed:
 class Part:
     """Common to all parts."""
 
+    # True when ``forward`` reads the step's data through device arrays only
+    # (``ctx.arrays``, cache and state tensors), never through host values such as
+    # ``ctx.host``: only then may a step be captured once as a graph and replayed.
+    graph_capturable = False
+
     def __init__(self, params: Mapping[str, Any], rt: Runtime):
         self.params = dict(params)
         self.rt = rt
@@ -81,9 +86,6 @@ class Mixer(Part):
 
     def state_need(self) -> Optional[StateNeed]:
         return None
-
-    def set_cache_group(self, group: int) -> None:
-        """Told once at build time which cache group holds this mixer's pages."""
 
     def forward(self, h: torch.Tensor, ctx: Any, site: Any) -> torch.Tensor:
         """h: [N, hidden] normed activations of the step's tokens; returns the

@@ -20,6 +20,8 @@ from .base import Part, Runtime, register_embedding, register_head
 class TokenEmbedding(Part):
     """params: name, vocab_size, hidden_size."""
 
+    graph_capturable = True
+
     def __init__(self, params, rt: Runtime):
         super().__init__(params, rt)
         self.name = params["name"]
@@ -42,6 +44,8 @@ class TokenEmbedding(Part):
 class LMHead(Part):
     """params: name, tied_to (name of the embedding table, or None), vocab_size,
     hidden_size."""
+
+    graph_capturable = True
 
     def __init__(self, params, rt: Runtime):
         super().__init__(params, rt)

@@ -22,6 +22,8 @@ ACTIVATIONS = ("silu", "gelu_tanh")
 
 @register_feed_forward("gated_mlp")
 class GatedMLP(FeedForward):
+
+    graph_capturable = True
     def __init__(self, params, rt: Runtime):
         super().__init__(params, rt)
         self.prefix = params["prefix"]
@@ -48,6 +50,6 @@ class GatedMLP(FeedForward):
 
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
         ops = self.rt.ops
-        gu = ops.linear(h, self.w_gate_up, self.rt.act_dtype)
-        a = ops.gated_act(gu, self.activation)
-        return ops.linear(a, self.w_down, self.rt.act_dtype)
+        gu = ops.linear(h, self.w_gate_up, self.rt.act_dtype, partial_ok=True)
+        a = ops.gated_act(gu, self.activation, self.rt.act_dtype)
+        return ops.linear(a, self.w_down, self.rt.act_dtype, partial_ok=True)

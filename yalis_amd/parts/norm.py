@@ -20,6 +20,8 @@ from .base import Norm, Runtime, register_norm
 class RMSNorm(Norm):
     """params: name (checkpoint tensor), size, eps, unit_offset."""
 
+    graph_capturable = True
+
     def __init__(self, params, rt: Runtime):
         super().__init__(params, rt)
         self.name = params["name"]
