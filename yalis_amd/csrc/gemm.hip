@@ -113,25 +113,36 @@ union Frag8 {
 // Here A = 16 rows of the weight (output features), B = 16 rows of x (tokens), so that
 // C[i][r] = y[token r][feature 4g + i].
 //
-// A workgroup of W waves owns 16*W weight rows (16 per wave) and 16*MT rows of x over one
-// slice of K (blockIdx.z); more waves share one staging of x, fewer give more workgroups.  K is walked in chunks of 256: the chunk of x is staged in LDS
-// once for all four waves; every wave streams its 16 weight rows straight from memory
-// into the A operand, 8 steps (512 contiguous bytes of every row) per chunk, with the next
-// chunk's loads issued before the current chunk is multiplied.  Measured on MI355X, a wave
-// that keeps 512 bytes of 16 rows in flight reads close to what contiguous streaming gives;
-// fewer bytes per row, or more rows per wave, read markedly slower.
-constexpr int SK_KC = 256;           // K elements per chunk
+// A workgroup of W waves (W = blockDim.x / 64, chosen per shape by the host) owns 16*W
+// weight rows (16 per wave) and 16*MT rows of x over one slice of K (blockIdx.z).  K is
+// walked in chunks of 256.  The chunk of x is staged in LDS once for all waves.  Every wave
+// streams its own 16 weight rows with loads that cover two rows x 512 contiguous bytes
+// each (measured on MI355X: that pattern reads about a fifth faster than the 16 rows x 64
+// bytes the matrix-core operand layout would ask of memory directly), parks the chunk in a
+// wave-private piece of LDS and reads it back in operand layout; the next chunk's loads
+// are in flight while the current one is multiplied.  Nothing is conditional in the loop:
+// rows beyond N are read from the last row and never stored, K beyond the slice is read
+// from valid places and meets zeros of x.
+constexpr int SK_KC = 256;            // K elements per chunk
 constexpr int SK_STEPS = SK_KC / 32;  // matrix-core steps per chunk
-constexpr int SK_PAD = 8;            // bf16 elements of padding per LDS row (keeps 16-byte reads conflict-free)
+constexpr int SK_PAD = 8;             // bf16 elements of padding per LDS row (keeps 16-byte reads conflict-free)
+constexpr int SK_ROW = SK_KC + SK_PAD;
+constexpr int SK_MAX_WAVES = 8;
 
-template <int MT, int W, typename TO>
-__global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
+static size_t skinny_lds_bytes(int mt, int waves) {
+  return static_cast<size_t>(16 * mt + 16 * waves) * SK_ROW * sizeof(bf16_t);
+}
+
+template <int MT, typename TO>
+__global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_mfma_skinny_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, float* __restrict__ part,
     TO* __restrict__ y, int M, int N, int K, int ldx, int ldw, int ldy, int k_block) {
-  __shared__ __attribute__((aligned(16))) bf16_t xs[16 * MT][SK_KC + SK_PAD];
+  extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
+  bf16_t(*xs)[SK_ROW] = reinterpret_cast<bf16_t(*)[SK_ROW]>(lds);  // [16 * MT][SK_ROW]
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  bf16_t(*wl)[SK_ROW] = reinterpret_cast<bf16_t(*)[SK_ROW]>(lds + static_cast<size_t>(16 * MT + 16 * wave) * SK_ROW);  // this wave's [16][SK_ROW]
   const int r = lane % 16, g = lane / 16;
-  const int n0 = blockIdx.x * (16 * W) + 16 * wave;
+  const int n0 = (blockIdx.x * (blockDim.x / 64) + wave) * 16;
   const int m0 = blockIdx.y * (16 * MT);
   const int kb0 = blockIdx.z * k_block;
   const int kb1 = min(K, kb0 + k_block);
@@ -140,24 +151,30 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  // A row beyond N is read from the last row instead and never stored; K beyond the slice
-  // is read from the last 8 elements instead and meets zeros of x.  So the weight loads
-  // carry no conditions.
-  const bf16_t* wrow = w + static_cast<size_t>(min(n0 + r, N - 1)) * ldw;
-  const int k_last = K - 8;
-  Frag8 a_cur[SK_STEPS], a_next[SK_STEPS];
-#define SK_LOAD_A(A, KC0)                                                                    \
-  _Pragma("unroll") for (int u = 0; u < SK_STEPS; ++u)                                        \
-      A[u].u = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wrow + min((KC0) + 32 * u + 8 * g, k_last)));
-
-  SK_LOAD_A(a_next, kb0)
-  for (int kc = kb0; kc < kb1; kc += SK_KC) {
+  // load j of a chunk: lanes 0..31 take row 2j, lanes 32..63 row 2j+1, 16 bytes each
+  const int half = lane / 32, l32 = lane % 32;
+  const bf16_t* wrow[SK_STEPS];
 #pragma unroll
-    for (int u = 0; u < SK_STEPS; ++u) a_cur[u] = a_next[u];
-    if (kc + SK_KC < kb1) SK_LOAD_A(a_next, kc + SK_KC)
+  for (int j = 0; j < SK_STEPS; ++j) wrow[j] = w + static_cast<size_t>(min(n0 + 2 * j + half, N - 1)) * ldw;
+  const int k_last = K - 8;
+  u32x4_t regs[SK_STEPS];
+#define SK_LOAD_W(KC0)                                                                      \
+  {                                                                                          \
+    const int kk_ = min((KC0) + 8 * l32, k_last);                                            \
+    _Pragma("unroll") for (int j = 0; j < SK_STEPS; ++j)                                     \
+        regs[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wrow[j] + kk_)); \
+  }
+
+  SK_LOAD_W(kb0)
+  for (int kc = kb0; kc < kb1; kc += SK_KC) {
+    // park the chunk that has arrived (this wave's earlier reads of the piece are done:
+    // LDS operations of a wave complete in order), then start the next chunk's loads
+#pragma unroll
+    for (int j = 0; j < SK_STEPS; ++j) *reinterpret_cast<u32x4_t*>(&wl[2 * j + half][8 * l32]) = regs[j];
+    if (kc + SK_KC < kb1) SK_LOAD_W(kc + SK_KC)
     __syncthreads();  // the previous chunk of x has been read by every wave
     // stage x[m0 .. m0+16*MT)[kc .. kc+256) as 16-byte pieces; zeros outside M and the slice
-    for (int e = threadIdx.x; e < 16 * MT * (SK_KC / 8); e += W * 64) {
+    for (int e = threadIdx.x; e < 16 * MT * (SK_KC / 8); e += blockDim.x) {
       const int row = e / (SK_KC / 8), piece = e % (SK_KC / 8);
       const int m = m0 + row, k = kc + 8 * piece;
       u32x4_t v = {0u, 0u, 0u, 0u};
@@ -167,15 +184,17 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
     __syncthreads();
 #pragma unroll
     for (int u = 0; u < SK_STEPS; ++u) {
+      Frag8 a;
+      a.u = *reinterpret_cast<const u32x4_t*>(&wl[r][32 * u + 8 * g]);
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
         Frag8 b;
         b.u = *reinterpret_cast<const u32x4_t*>(&xs[16 * t + r][32 * u + 8 * g]);
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_cur[u].v, b.v, acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[t], 0, 0, 0);
       }
     }
   }
-#undef SK_LOAD_A
+#undef SK_LOAD_W
 
   const bool to_part = part != nullptr;
   float* pout = to_part ? part + static_cast<size_t>(blockIdx.z) * M * N : nullptr;
@@ -217,30 +236,48 @@ __global__ void reduce_splits_kernel(const float* __restrict__ part, TO* __restr
 static int skinny_mt(int M) { return M <= 16 ? 1 : (M <= 32 ? 2 : 4); }
 
 // How the skinny kernel cuts the work for these sizes: waves per workgroup (each wave owns
-// 16 weight rows), the number of K slices and the length of one (a multiple of 256).  The
-// aim is at least two workgroups per compute unit with as many waves sharing one staging
-// of x as that allows, and at least 512 of K per workgroup.  A caller that takes the
-// slices unreduced needs splits * M * N floats.
+// 16 weight rows), the number of K slices and the length of one (a multiple of 256).
+// All workgroups do the same amount of work, so the time is that of the busiest compute
+// unit: (workgroups on it) x (waves each) x (K chunks each, plus a start-up of about one
+// and a half chunks), stretched when the unit has too few waves to keep memory busy.  The
+// plan minimises that over 1..8 waves and the slice counts that leave at least two chunks
+// per workgroup, with a small charge for narrow workgroups (every workgroup stages its own
+// copy of x) and for many slices (the consumer adds them).
+// A caller that takes the slices unreduced needs splits * M * N floats.
+constexpr int SK_CUS = 256;
+
 static int skinny_plan(int M, int N, int K, int* waves_out, int* k_block_out) {
   const int mt = skinny_mt(M);
   const long mtiles = (M + 16 * mt - 1) / (16 * mt);
-  const long max_by_k = std::max(1, K / 512);
-  int waves = 4;
-  long s = 1;
-  for (int w : {16, 8, 4}) {
-    if (w > 4 * mt && w > 8) continue;  // many waves only pay when x is wide
-    const long tiles = static_cast<long>((N + 16 * w - 1) / (16 * w)) * mtiles;
-    const long want = (512 + tiles - 1) / tiles;
-    waves = w;
-    s = std::max(1L, std::min(want, max_by_k));
-    if (tiles * s >= 512 || w == 4) break;
+  const long ntiles = (N + 15) / 16;
+  const long chunks = (K + SK_KC - 1) / SK_KC;
+  const long max_s = std::max(1L, std::min(32L, chunks / 2));
+  double best = 1e300;
+  int best_w = 4;
+  long best_s = 1;
+  for (int w = 1; w <= SK_MAX_WAVES; ++w) {
+    const long rblocks = (ntiles + w - 1) / w;
+    const double resident = std::min(20.0, static_cast<double>(160 * 1024 / skinny_lds_bytes(mt, w)) * w);
+    for (long s = 1; s <= max_s; ++s) {
+      const long per = (chunks + s - 1) / s;          // chunks per workgroup
+      const long real = (chunks + per - 1) / per;     // slices that are not empty
+      const long blocks = rblocks * mtiles * real;
+      const double busiest = static_cast<double>((blocks + SK_CUS - 1) / SK_CUS) * w * (per + 1.5);
+      // a compute unit streams at full rate only with about 12 waves' loads in flight
+      const double waves_cu = std::min(resident, static_cast<double>(blocks) * w / SK_CUS);
+      const double starved = std::max(1.0, 12.0 / waves_cu);
+      const double cost = busiest * starved * (1.0 + 0.25 * mt / w) * (1.0 + 0.01 * real);
+      if (cost < best * 0.999) {
+        best = cost;
+        best_w = w;
+        best_s = real;
+      }
+    }
   }
-  s = std::min(s, 32L);
-  int k_block = static_cast<int>((K + s - 1) / s);
-  k_block = (k_block + SK_KC - 1) / SK_KC * SK_KC;
-  if (waves_out) *waves_out = waves;
+  int k_block = static_cast<int>((chunks + best_s - 1) / best_s) * SK_KC;
+  if (waves_out) *waves_out = best_w;
   if (k_block_out) *k_block_out = k_block;
-  return (K + k_block - 1) / k_block;
+  return static_cast<int>((K + k_block - 1) / k_block);
 }
 
 extern "C" int yk_gemm_skinny_splits(int M, int N, int K) { return skinny_plan(M, N, K, nullptr, nullptr); }
@@ -252,12 +289,20 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, i
   dim3 grid((N + 16 * waves - 1) / (16 * waves), (M + 16 * mt - 1) / (16 * mt), splits);
   YK_REQUIRE(grid.y <= 65535, "gemm_mfma_skinny: too many rows for one launch");
   dim3 block(waves * 64);
-#define SK_GO(MT_, W_)                                                                                   \
-  if (mt == MT_ && waves == W_) {                                                                       \
-    gemm_mfma_skinny_kernel<MT_, W_, TO><<<grid, block, 0, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block); \
+  const size_t lds = skinny_lds_bytes(mt, waves);
+#define SK_GO(MT_)                                                                                       \
+  if (mt == MT_) {                                                                                      \
+    static bool raised = false; /* allow more than the default 64 KB of dynamic LDS, once */           \
+    if (!raised) {                                                                                      \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_kernel<MT_, TO>),         \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)    \
+        return yk_fail("gemm_mfma_skinny: cannot raise the LDS limit");                                 \
+      raised = true;                                                                                    \
+    }                                                                                                   \
+    gemm_mfma_skinny_kernel<MT_, TO><<<grid, block, lds, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block); \
     return yk_check_launch("gemm_mfma_skinny");                                                         \
   }
-  SK_GO(1, 4) SK_GO(1, 8) SK_GO(2, 4) SK_GO(2, 8) SK_GO(4, 4) SK_GO(4, 8) SK_GO(4, 16)
+  SK_GO(1) SK_GO(2) SK_GO(4)
 #undef SK_GO
   return yk_fail("gemm_mfma_skinny: no kernel for this plan");
 }
