@@ -14,6 +14,8 @@
 // The reference runs these products through nn.Linear / cuBLAS
 // (yalis/external/model.py:63-65, 449, 462-466, 717-722).
 #include <algorithm>
+#include <cstdio>
+#include <cstdlib>
 
 #include "common.h"
 
@@ -133,8 +135,8 @@ static size_t skinny_lds_bytes(int mt, int waves) {
   return static_cast<size_t>(16 * mt + 16 * waves) * SK_ROW * sizeof(bf16_t);
 }
 
-template <int MT, typename TO>
-__global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_mfma_skinny_kernel(
+template <int MT, int W, typename TO>
+__global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, float* __restrict__ part,
     TO* __restrict__ y, int M, int N, int K, int ldx, int ldw, int ldy, int k_block) {
   extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
@@ -142,7 +144,7 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_mfma_skinny_kernel(
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
   bf16_t(*wl)[SK_ROW] = reinterpret_cast<bf16_t(*)[SK_ROW]>(lds + static_cast<size_t>(16 * MT + 16 * wave) * SK_ROW);  // this wave's [16][SK_ROW]
   const int r = lane % 16, g = lane / 16;
-  const int n0 = (blockIdx.x * (blockDim.x / 64) + wave) * 16;
+  const int n0 = (blockIdx.x * W + wave) * 16;
   const int m0 = blockIdx.y * (16 * MT);
   const int kb0 = blockIdx.z * k_block;
   const int kb1 = min(K, kb0 + k_block);
@@ -151,7 +153,7 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_mfma_skinny_kernel(
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  // load j of a chunk: lanes 0..31 take row 2j, lanes 32..63 row 2j+1, 16 bytes each
+  // weights: load j of a chunk covers rows 2j (lanes 0..31) and 2j+1 (lanes 32..63), 16 bytes a lane
   const int half = lane / 32, l32 = lane % 32;
   const bf16_t* wrow[SK_STEPS];
 #pragma unroll
@@ -164,22 +166,35 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_mfma_skinny_kernel(
     _Pragma("unroll") for (int j = 0; j < SK_STEPS; ++j)                                     \
         regs[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wrow[j] + kk_)); \
   }
+  // x: the chunk's 16*MT rows x 32 pieces of 16 bytes are spread over the threads, XP each;
+  // what lies outside M or the slice becomes zero after the (clamped) load
+  constexpr int XP = 16 * MT * (SK_KC / 8) / (W * 64);
+  static_assert(XP * W * 64 == 16 * MT * (SK_KC / 8), "x pieces must divide evenly over the threads");
+  u32x4_t xr[XP];
+  const u32x4_t zero = {0u, 0u, 0u, 0u};
+#define SK_LOAD_X(KC0)                                                                      \
+  _Pragma("unroll") for (int p = 0; p < XP; ++p) {                                           \
+    const int e_ = threadIdx.x + p * W * 64;                                                 \
+    const int m_ = m0 + e_ / (SK_KC / 8), k_ = (KC0) + 8 * (e_ % (SK_KC / 8));               \
+    xr[p] = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(min(m_, M - 1)) * ldx + min(k_, k_last)); \
+    if (m_ >= M || k_ >= kb1) xr[p] = zero;                                                  \
+  }
 
   SK_LOAD_W(kb0)
+  SK_LOAD_X(kb0)
   for (int kc = kb0; kc < kb1; kc += SK_KC) {
-    // park the chunk that has arrived (this wave's earlier reads of the piece are done:
-    // LDS operations of a wave complete in order), then start the next chunk's loads
+    __syncthreads();  // every wave has read the previous chunk of x
+    // park what has arrived, then put the next chunk's loads in flight
 #pragma unroll
     for (int j = 0; j < SK_STEPS; ++j) *reinterpret_cast<u32x4_t*>(&wl[2 * j + half][8 * l32]) = regs[j];
-    if (kc + SK_KC < kb1) SK_LOAD_W(kc + SK_KC)
-    __syncthreads();  // the previous chunk of x has been read by every wave
-    // stage x[m0 .. m0+16*MT)[kc .. kc+256) as 16-byte pieces; zeros outside M and the slice
-    for (int e = threadIdx.x; e < 16 * MT * (SK_KC / 8); e += blockDim.x) {
-      const int row = e / (SK_KC / 8), piece = e % (SK_KC / 8);
-      const int m = m0 + row, k = kc + 8 * piece;
-      u32x4_t v = {0u, 0u, 0u, 0u};
-      if (m < M && k < kb1) v = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(m) * ldx + k);
-      *reinterpret_cast<u32x4_t*>(&xs[row][8 * piece]) = v;
+#pragma unroll
+    for (int p = 0; p < XP; ++p) {
+      const int e = threadIdx.x + p * W * 64;
+      *reinterpret_cast<u32x4_t*>(&xs[e / (SK_KC / 8)][8 * (e % (SK_KC / 8))]) = xr[p];
+    }
+    if (kc + SK_KC < kb1) {
+      SK_LOAD_W(kc + SK_KC)
+      SK_LOAD_X(kc + SK_KC)
     }
     __syncthreads();
 #pragma unroll
@@ -195,6 +210,7 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_mfma_skinny_kernel(
     }
   }
 #undef SK_LOAD_W
+#undef SK_LOAD_X
 
   const bool to_part = part != nullptr;
   float* pout = to_part ? part + static_cast<size_t>(blockIdx.z) * M * N : nullptr;
@@ -240,7 +256,7 @@ static int skinny_mt(int M) { return M <= 16 ? 1 : (M <= 32 ? 2 : 4); }
 // All workgroups do the same amount of work, so the time is that of the busiest compute
 // unit: (workgroups on it) x (waves each) x (K chunks each, plus a start-up of about one
 // and a half chunks), stretched when the unit has too few waves to keep memory busy.  The
-// plan minimises that over 1..8 waves and the slice counts that leave at least two chunks
+// plan minimises that over 4 or 8 waves and the slice counts that leave at least two chunks
 // per workgroup, with a small charge for narrow workgroups (every workgroup stages its own
 // copy of x) and for many slices (the consumer adds them).
 // A caller that takes the slices unreduced needs splits * M * N floats.
@@ -255,7 +271,7 @@ static int skinny_plan(int M, int N, int K, int* waves_out, int* k_block_out) {
   double best = 1e300;
   int best_w = 4;
   long best_s = 1;
-  for (int w = 1; w <= SK_MAX_WAVES; ++w) {
+  for (int w : {4}) {  // measured: four waves per workgroup beat eight on every shape tried
     const long rblocks = (ntiles + w - 1) / w;
     const double resident = std::min(20.0, static_cast<double>(160 * 1024 / skinny_lds_bytes(mt, w)) * w);
     for (long s = 1; s <= max_s; ++s) {
@@ -263,15 +279,22 @@ static int skinny_plan(int M, int N, int K, int* waves_out, int* k_block_out) {
       const long real = (chunks + per - 1) / per;     // slices that are not empty
       const long blocks = rblocks * mtiles * real;
       const double busiest = static_cast<double>((blocks + SK_CUS - 1) / SK_CUS) * w * (per + 1.5);
-      // a compute unit streams at full rate only with about 12 waves' loads in flight
+      // a compute unit streams at full rate only with about 6 waves' loads in flight
       const double waves_cu = std::min(resident, static_cast<double>(blocks) * w / SK_CUS);
-      const double starved = std::max(1.0, 12.0 / waves_cu);
+      const double starved = std::max(1.0, 6.0 / waves_cu);
       const double cost = busiest * starved * (1.0 + 0.25 * mt / w) * (1.0 + 0.01 * real);
       if (cost < best * 0.999) {
         best = cost;
         best_w = w;
         best_s = real;
       }
+    }
+  }
+  if (const char* force = getenv("YALIS_SKINNY_PLAN")) {  // "waves,slices": for measurements
+    int fw = 0, fs = 0;
+    if (sscanf(force, "%d,%d", &fw, &fs) == 2 && (fw == 4 || fw == 8) && fs >= 1) {
+      best_w = fw;
+      best_s = std::min<long>(fs, chunks);
     }
   }
   int k_block = static_cast<int>((chunks + best_s - 1) / best_s) * SK_KC;
@@ -290,19 +313,19 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, i
   YK_REQUIRE(grid.y <= 65535, "gemm_mfma_skinny: too many rows for one launch");
   dim3 block(waves * 64);
   const size_t lds = skinny_lds_bytes(mt, waves);
-#define SK_GO(MT_)                                                                                       \
-  if (mt == MT_) {                                                                                      \
+#define SK_GO(MT_, W_)                                                                                   \
+  if (mt == MT_ && waves == W_) {                                                                       \
     static bool raised = false; /* allow more than the default 64 KB of dynamic LDS, once */           \
     if (!raised) {                                                                                      \
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_kernel<MT_, TO>),         \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_kernel<MT_, W_, TO>),     \
                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)    \
         return yk_fail("gemm_mfma_skinny: cannot raise the LDS limit");                                 \
       raised = true;                                                                                    \
     }                                                                                                   \
-    gemm_mfma_skinny_kernel<MT_, TO><<<grid, block, lds, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block); \
+    gemm_mfma_skinny_kernel<MT_, W_, TO><<<grid, block, lds, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block); \
     return yk_check_launch("gemm_mfma_skinny");                                                         \
   }
-  SK_GO(1) SK_GO(2) SK_GO(4)
+  SK_GO(1, 4) SK_GO(1, 8) SK_GO(2, 4) SK_GO(2, 8) SK_GO(4, 4) SK_GO(4, 8)
 #undef SK_GO
   return yk_fail("gemm_mfma_skinny: no kernel for this plan");
 }
