@@ -104,7 +104,7 @@ def attention_paged(q, k_cache, v_cache, positions, token_seq, block_table, page
 
 
 def attention(qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size, scale,
-              window, ctx, group, tiles):
+              window, ctx, group, tiles, long_tiles=None):
     n = qkv.shape[0]
     q = qkv.view(n, -1, head_dim)[:, :n_heads]
     out = attention_paged(
@@ -139,6 +139,9 @@ class RefOps:
 
     def attention_tokens_per_tile(self, n_heads, n_kv):
         return 16 // min(n_heads // n_kv, 16)
+
+    def attention_long_span_tile(self, n_heads, n_kv):
+        return 4 * self.attention_tokens_per_tile(n_heads, n_kv)
 
     embed = staticmethod(embed)
     add_rmsnorm = staticmethod(add_rmsnorm)

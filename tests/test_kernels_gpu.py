@@ -254,7 +254,8 @@ def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True,
         seqs.append(SeqSpan(tokens=[0] * new, first_position=cached, block_tables=[table], state_slot=0))
     hb = build_host_batch(seqs, 1, page)
     tpt = ops.attention_tokens_per_tile(h, g)
-    arrays = named_arrays(hb, {f"tiles": lambda b: attention_tiles(b, tpt)})
+    big = ops.attention_long_span_tile(h, g)
+    arrays = named_arrays(hb, {"tiles": lambda b: attention_tiles(b, tpt, 1, big), "long_tiles": lambda b: attention_tiles(b, big, big + 1)})
     ctx = types.SimpleNamespace(
         arrays={k: torch.from_numpy(np.ascontiguousarray(v)).to(DEV) for k, v in arrays.items()},
         max_ctx=hb.max_ctx,
@@ -263,7 +264,7 @@ def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True,
     n = hb.n_tokens
     q = (torch.randn((n, h * d), generator=gen) * 1.5).to(dtype)
     scale = 1.0 / math.sqrt(d)
-    got = ops.attention(q.to(DEV), h, g, d, kc.to(DEV), vc.to(DEV), page, scale, window, ctx, 0, ctx.arrays["tiles"])
+    got = ops.attention(q.to(DEV), h, g, d, kc.to(DEV), vc.to(DEV), page, scale, window, ctx, 0, ctx.arrays["tiles"], ctx.arrays["long_tiles"])
     want = R.attention(q.float(), h, g, d, kc.float(), vc.float(), page, scale, window, ctx_cpu, 0, None)
     return got, want
 

@@ -137,9 +137,21 @@ union AFrag8 {
   bf16_t h[8];
 };
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+// two floats to two bfloat16 (round to nearest even) in one word: gfx950 converts in hardware
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return static_cast<uint32_t>(f32_to_bf16(lo)) | (static_cast<uint32_t>(f32_to_bf16(hi)) << 16);
+  union {
+    bf16x2_t v;
+    uint32_t u;
+  } c;
+  c.v = __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t);
+  return c.u;
 }
+
+// 2^x for scores: -inf gives 0, no denormal handling needed
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Layout of a tile row handed over by the host: (request, first token index in the
 // batch, token count, position of the first token).
@@ -240,22 +252,29 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
       }
     if (kb + 1 < my_hi) ATT_LOAD_K(kb + 1)
     float tmax = -INFINITY;
+    // a block that every column sees whole needs no mask (columns that stand for nothing
+    // compute on zeros and are never stored)
+    const bool whole = kb * 64 + 63 <= pos0 && (window == 0 || kb * 64 >= max(0, pos0 + ntok - window));
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
       for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int key = kb * 64 + 32 * u + 8 * gq + 4 * sb + i;
-          const bool ok = col_ok && key <= pos_c && key >= lo_c;
-          s[u][sb][i] = ok ? s[u][sb][i] * scale_log2 : -INFINITY;
+          if (whole) {
+            s[u][sb][i] *= scale_log2;
+          } else {
+            const int key = kb * 64 + 32 * u + 8 * gq + 4 * sb + i;
+            const bool ok = col_ok && key <= pos_c && key >= lo_c;
+            s[u][sb][i] = ok ? s[u][sb][i] * scale_log2 : -INFINITY;
+          }
           tmax = fmaxf(tmax, s[u][sb][i]);
         }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
     const float m_new = fmaxf(m, tmax);
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = exp2f(m - m_safe);
+    const float alpha = fast_exp2(m - m_safe);
     float psum = 0.f;
     AFrag8 pf[2];
 #pragma unroll
@@ -264,7 +283,7 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
       for (int sb = 0; sb < 2; ++sb) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          s[u][sb][i] = exp2f(s[u][sb][i] - m_safe);
+          s[u][sb][i] = fast_exp2(s[u][sb][i] - m_safe);
           psum += s[u][sb][i];
         }
         pf[u].u[2 * sb] = pack_bf16x2(s[u][sb][0], s[u][sb][1]);
@@ -318,6 +337,226 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
     if (gq == 0) {
       ws_ml[(widx * 16 + r) * 2] = m;
       ws_ml[(widx * 16 + r) * 2 + 1] = l;
+    }
+  }
+}
+
+// The same arithmetic for long spans (prompt portions): a workgroup of four waves owns four
+// consecutive tiles of one request (64 columns) and walks the keys once for all of them.
+// Each block of 64 keys and values is fetched from the pages with coalesced loads, parked
+// in LDS (keys in the row order the score products read them, so that the reads are free of
+// bank conflicts) and read from there by the four waves; the next block's loads are in
+// flight meanwhile.  No split of the keys: long spans bring enough workgroups.
+template <int D, bool BLOCK_IN_PAGE>
+__global__ __launch_bounds__(256) void attn_mfma_prefill_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
+    const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int32_t* __restrict__ tiles, const int32_t* __restrict__ block_table, int table_width,
+    int page_size, int n_heads, int n_kv, int hpt, int chunks, float scale_log2, int window) {
+  constexpr int KS = D / 32, DT = D / 16;
+  constexpr int KROW = D + 8;   // bf16 elements per parked key row
+  constexpr int VROW = 64 + 8;  // bf16 elements per parked value row
+  constexpr int PP = D / 32;    // 16-byte pieces of keys (and of values) per thread and block
+  __shared__ __attribute__((aligned(16))) bf16_t ks[64][KROW];
+  __shared__ __attribute__((aligned(16))) bf16_t vs[D][VROW];
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, gq = lane / 16;
+  const int t = blockIdx.x;
+  const int seq = tiles[4 * t], tile_tok0 = tiles[4 * t + 1], tile_ntok = tiles[4 * t + 2], tile_pos0 = tiles[4 * t + 3];
+  const int g = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+  const int qpk = n_heads / n_kv;
+  const int h_base = g * qpk + chunk * hpt;
+  const int heads_here = min(hpt, qpk - chunk * hpt);
+  const int tpt = 16 / hpt;  // tokens per wave
+  const int tt = r / hpt, hh = r % hpt;
+  const int tok_in_tile = wave * tpt + tt;
+  const bool col_ok = tt < tpt && tok_in_tile < tile_ntok && hh < heads_here;
+  const int pos_c = tile_pos0 + tok_in_tile;
+  const int lo_c = window > 0 ? max(0, pos_c - window + 1) : 0;
+  const int hi = tile_pos0 + tile_ntok;  // keys the workgroup may need
+  const int lo = window > 0 ? max(0, tile_pos0 - window + 1) : 0;
+  const int wave_hi = min(hi, tile_pos0 + (wave + 1) * tpt);  // keys this wave may need
+  const int kb_lo = lo / 64, kb_hi = (hi + 63) / 64;
+  const int32_t* bt = block_table + static_cast<size_t>(seq) * table_width;
+  const int last_page_col = min(table_width - 1, (hi - 1) / page_size);
+  // page ids of the keys this workgroup walks, once, into LDS (a lookup per fetched piece
+  // would put a dependent memory round trip before every load)
+  constexpr int PAGES_LDS = 2048;
+  __shared__ int32_t pages_s[PAGES_LDS];
+  const int first_col = min(last_page_col, kb_lo * 64 / page_size);
+  const bool pages_in_lds = last_page_col - first_col < PAGES_LDS;
+  if (pages_in_lds)
+    for (int c = first_col + threadIdx.x; c <= last_page_col; c += 256) pages_s[c - first_col] = max(0, bt[c]);
+  const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
+  auto page_col = [&](int key) { return min(page_shift >= 0 ? key >> page_shift : key / page_size, last_page_col); };
+  auto page_off = [&](int key) { return page_shift >= 0 ? key & (page_size - 1) : key % page_size; };
+  auto page_of = [&](int key) {
+    const int c = page_col(key);
+    return pages_in_lds ? pages_s[c - first_col] : max(0, bt[c]);
+  };
+  __syncthreads();
+
+  const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+  AFrag8 qf[KS];
+  {
+    const bf16_t* qp = q + static_cast<size_t>(tile_tok0 + (col_ok ? tok_in_tile : 0)) * q_stride +
+                       static_cast<size_t>(h_base + (col_ok ? hh : 0)) * D + 8 * gq;
+#pragma unroll
+    for (int ks_ = 0; ks_ < KS; ++ks_) {
+      qf[ks_].u = *reinterpret_cast<const u32x4_t*>(qp + 32 * ks_);
+      if (!col_ok) qf[ks_].u = zero4;
+    }
+  }
+  float m = -INFINITY, l = 0.f;
+  f32x4_t acc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  // what this thread fetches of every block: PP pieces of keys and PP pieces of values.
+  // With pages of a multiple of 64 tokens a block of keys lies in one page: the page id is
+  // looked up once per block and each thread adds offsets it computed once.
+  u32x4_t kreg[PP], vreg[PP];
+  constexpr bool block_in_page = BLOCK_IN_PAGE;  // chosen by the launcher: page_size % 64 == 0
+  size_t koff[PP], voff[PP];
+#pragma unroll
+  for (int p = 0; p < PP; ++p) {
+    const int e = threadIdx.x + 256 * p;
+    koff[p] = static_cast<size_t>(e / (D / 8)) * D + 8 * (e % (D / 8));
+    voff[p] = static_cast<size_t>(e / 8) * page_size + 8 * (e % 8);
+  }
+  const size_t page_elems = static_cast<size_t>(n_kv) * page_size * D;
+#define PF_LOAD(KB)                                                                                \
+  if (block_in_page) {                                                                              \
+    const int key0 = (KB) * 64;                                                                     \
+    const size_t base = static_cast<size_t>(page_of(key0)) * page_elems + static_cast<size_t>(g) * page_size * D; \
+    const int off = page_off(key0);                                                                 \
+    const bf16_t* kp = k_cache + base + static_cast<size_t>(off) * D;                               \
+    const bf16_t* vp = v_cache + base + off;                                                        \
+    _Pragma("unroll") for (int p = 0; p < PP; ++p) {                                                \
+      kreg[p] = *reinterpret_cast<const u32x4_t*>(kp + koff[p]);                                    \
+      vreg[p] = *reinterpret_cast<const u32x4_t*>(vp + voff[p]);                                    \
+    }                                                                                               \
+  } else {                                                                                          \
+    _Pragma("unroll") for (int p = 0; p < PP; ++p) {                                                \
+      const int e = threadIdx.x + 256 * p;                                                          \
+      {                                                                                             \
+        const int key = (KB) * 64 + e / (D / 8), piece = e % (D / 8);                               \
+        kreg[p] = *reinterpret_cast<const u32x4_t*>(                                                \
+            k_cache + ((static_cast<size_t>(page_of(key)) * n_kv + g) * page_size + page_off(key)) * D + 8 * piece); \
+      }                                                                                             \
+      {                                                                                             \
+        const int d = e / 8, key = (KB) * 64 + 8 * (e % 8);                                         \
+        vreg[p] = *reinterpret_cast<const u32x4_t*>(                                                \
+            v_cache + ((static_cast<size_t>(page_of(key)) * n_kv + g) * D + d) * page_size + page_off(key)); \
+      }                                                                                             \
+    }                                                                                               \
+  }
+
+  if (kb_lo < kb_hi) PF_LOAD(kb_lo)
+  for (int kb = kb_lo; kb < kb_hi; ++kb) {
+    __syncthreads();  // every wave is done with the previous block
+#pragma unroll
+    for (int p = 0; p < PP; ++p) {
+      const int e = threadIdx.x + 256 * p;
+      {
+        // key kappa = 32u + 8a + 4sb + c of the block is parked at row 32u + 16sb + 4a + c
+        const int kappa = e / (D / 8), piece = e % (D / 8);
+        const int row = (kappa & 32) | ((kappa & 4) << 2) | ((kappa & 24) >> 1) | (kappa & 3);
+        *reinterpret_cast<u32x4_t*>(&ks[row][8 * piece]) = kreg[p];
+      }
+      {
+        u32x4_t v = vreg[p];
+        const int key = kb * 64 + 8 * (e % 8);
+        if (key + 8 > hi) {  // values of keys that do not exist yet may be anything
+          AFrag8 f;
+          f.u = v;
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            if (key + i >= hi) f.h[i] = 0;
+          v = f.u;
+        }
+        *reinterpret_cast<u32x4_t*>(&vs[e / 8][8 * (e % 8)]) = v;
+      }
+    }
+    __syncthreads();
+    if (kb + 1 < kb_hi) PF_LOAD(kb + 1)  // in flight while this block is worked on
+    if (kb * 64 >= wave_hi) continue;  // nothing of this block is visible to this wave
+
+    f32x4_t s[2][2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int sb = 0; sb < 2; ++sb) {
+        s[u][sb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks_ = 0; ks_ < KS; ++ks_) {
+          AFrag8 a;
+          a.u = *reinterpret_cast<const u32x4_t*>(&ks[32 * u + 16 * sb + r][32 * ks_ + 8 * gq]);
+          s[u][sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[ks_].v, s[u][sb], 0, 0, 0);
+        }
+      }
+    float tmax = -INFINITY;
+    // a block that every column sees whole needs no mask (columns that stand for nothing
+    // compute on zeros and are never stored)
+    const bool whole = kb * 64 + 63 <= (tile_pos0 + wave * tpt) && (window == 0 || kb * 64 >= max(0, wave_hi - window));
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (whole) {
+            s[u][sb][i] *= scale_log2;
+          } else {
+            const int key = kb * 64 + 32 * u + 8 * gq + 4 * sb + i;
+            const bool ok = col_ok && key <= pos_c && key >= lo_c;
+            s[u][sb][i] = ok ? s[u][sb][i] * scale_log2 : -INFINITY;
+          }
+          tmax = fmaxf(tmax, s[u][sb][i]);
+        }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m, tmax);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = fast_exp2(m - m_safe);
+    float psum = 0.f;
+    AFrag8 pf[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int sb = 0; sb < 2; ++sb) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          s[u][sb][i] = fast_exp2(s[u][sb][i] - m_safe);
+          psum += s[u][sb][i];
+        }
+        pf[u].u[2 * sb] = pack_bf16x2(s[u][sb][0], s[u][sb][1]);
+        pf[u].u[2 * sb + 1] = pack_bf16x2(s[u][sb][2], s[u][sb][3]);
+      }
+    l = l * alpha + psum;
+    m = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      acc[dt] *= alpha;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        AFrag8 a;
+        a.u = *reinterpret_cast<const u32x4_t*>(&vs[16 * dt + r][32 * u + 8 * gq]);
+        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pf[u].v, acc[dt], 0, 0, 0);
+      }
+    }
+  }
+#undef PF_LOAD
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (col_ok) {
+    const float inv = 1.f / l;
+    bf16_t* op = out + (static_cast<size_t>(tile_tok0 + tok_in_tile) * n_heads + h_base + hh) * D + 4 * gq;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      u32x2_t w;
+      w[0] = pack_bf16x2(acc[dt][0] * inv, acc[dt][1] * inv);
+      w[1] = pack_bf16x2(acc[dt][2] * inv, acc[dt][3] * inv);
+      *reinterpret_cast<u32x2_t*>(op + 16 * dt) = w;
     }
   }
 }
@@ -378,6 +617,41 @@ extern "C" size_t yk_attn_mfma_workspace(int n_tiles, int n_heads, int n_kv, int
   const int chunks = (n_heads / n_kv + hpt - 1) / hpt;
   const size_t w = static_cast<size_t>(n_tiles) * n_kv * chunks * n_splits * 16;
   return w * head_dim + w * 2;
+}
+
+// Long spans: ``tiles`` hold up to 4 * tokens_per_tile tokens each (one workgroup a tile).
+extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, const void* k_cache,
+                                    const void* v_cache, const int32_t* tiles, int n_tiles,
+                                    const int32_t* block_table, int table_width, int page_size,
+                                    int head_dim, int n_heads, int n_kv, float scale, int window,
+                                    hipStream_t stream) {
+  YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_mfma_prefill: bad head counts");
+  YK_REQUIRE(yk_attn_mfma_supported(head_dim), "attn_mfma_prefill: head_dim must be 64 or 128");
+  YK_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_mfma_prefill: page_size must be a multiple of 16");
+  YK_REQUIRE(q_stride % 8 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0,
+             "attn_mfma_prefill: query rows must be 16-byte aligned");
+  YK_REQUIRE(reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0,
+             "attn_mfma_prefill: cache must be 16-byte aligned");
+  YK_REQUIRE(window >= 0 && table_width > 0, "attn_mfma_prefill: bad window or table");
+  if (n_tiles == 0) return 0;
+  const int hpt = yk_attn_heads_per_tile(n_heads, n_kv);
+  const int chunks = (n_heads / n_kv + hpt - 1) / hpt;
+  YK_REQUIRE(n_kv * chunks <= 65535, "attn_mfma_prefill: too many heads for one launch");
+  const float scale_log2 = scale * 1.4426950408889634f;
+  dim3 grid(n_tiles, n_kv * chunks), block(256);
+#define YK_PF(DD, BIP)                                                                                       \
+  attn_mfma_prefill_kernel<DD, BIP><<<grid, block, 0, stream>>>(                                                 \
+      static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),   \
+      static_cast<const bf16_t*>(v_cache), tiles, block_table, table_width, page_size, n_heads, n_kv, hpt, chunks, \
+      scale_log2, window)
+  const bool bip = page_size % 64 == 0;
+  if (head_dim == 64) {
+    if (bip) YK_PF(64, true); else YK_PF(64, false);
+  } else {
+    if (bip) YK_PF(128, true); else YK_PF(128, false);
+  }
+#undef YK_PF
+  return yk_check_launch("attn_mfma_prefill");
 }
 
 extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* k_cache,

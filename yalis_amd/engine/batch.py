@@ -143,14 +143,17 @@ def pack(arrays: Dict[str, np.ndarray]) -> Tuple[np.ndarray, Dict[str, Tuple[int
     return buf, layout
 
 
-def attention_tiles(hb: HostBatch, tokens_per_tile: int) -> np.ndarray:
+def attention_tiles(hb: HostBatch, tokens_per_tile: int, min_span: int = 1, max_span: int = 1 << 30) -> np.ndarray:
     """Cut every request's span into tiles of at most ``tokens_per_tile``
     consecutive tokens: rows of (request, first token index in the batch, token
-    count, first position)."""
+    count, first position).  Only spans of min_span..max_span tokens are cut (a kernel
+    for long spans and one for short ones each get their own list)."""
     rows = []
     for i in range(hb.n_seqs):
         q0 = int(hb.seq_qstart[i])
         ql = int(hb.seq_qlen[i])
+        if not min_span <= ql <= max_span:
+            continue
         p0 = int(hb.seq_ctx[i]) - ql
         for t in range(0, ql, tokens_per_tile):
             rows.append((i, q0 + t, min(tokens_per_tile, ql - t), p0 + t))

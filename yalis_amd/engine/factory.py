@@ -31,6 +31,9 @@ class _ShapeOnlyOps:
     def attention_tokens_per_tile(self, *a):
         return 1
 
+    def attention_long_span_tile(self, *a):
+        return 4
+
 
 def spec_from_config(config_dict: dict):
     arch = architecture_of(config_dict)

@@ -70,6 +70,10 @@ _SIGNATURES = {
     "yk_attn_heads_per_tile": ([_c_int, _c_int], _c_int),
     "yk_attn_tokens_per_tile": ([_c_int, _c_int], _c_int),
     "yk_attn_mfma_workspace": ([_c_int, _c_int, _c_int, _c_int, _c_int], _c_size_t),
+    "yk_attn_mfma_prefill": (
+        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp],
+        _c_int,
+    ),
     "yk_attn_mfma": (
         [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _vp, _c_size_t, _vp],
         _c_int,
@@ -168,6 +172,10 @@ class HipOps:
 
     def attention_tokens_per_tile(self, n_heads: int, n_kv: int) -> int:
         return self.lib.yk_attn_tokens_per_tile(n_heads, n_kv)
+
+    def attention_long_span_tile(self, n_heads: int, n_kv: int) -> int:
+        """Tokens per tile of the kernel for long spans (four waves of tokens_per_tile)."""
+        return 4 * self.lib.yk_attn_tokens_per_tile(n_heads, n_kv)
 
     # ------------------------------------------------------------------ embedding
     def embed(self, token_ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
@@ -309,7 +317,7 @@ class HipOps:
 
     # ------------------------------------------------------------------ attention
     def attention(self, qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size,
-                  scale, window, ctx, group, tiles) -> torch.Tensor:
+                  scale, window, ctx, group, tiles, long_tiles=None) -> torch.Tensor:
         """Queries are the first n_heads heads of each row of ``qkv`` (whatever follows
         them in the row is skipped); keys and values come from the cache through the
         block table of ``group``."""
@@ -327,6 +335,16 @@ class HipOps:
             and qkv.stride(0) % 8 == 0
             and qkv.data_ptr() % 16 == 0
         )
+        if use_mfma and long_tiles is not None and long_tiles.shape[0] > 0:
+            self._check(
+                self.lib.yk_attn_mfma_prefill(
+                    qkv.data_ptr(), qkv.stride(0), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                    long_tiles.data_ptr(), long_tiles.shape[0], bt.data_ptr(), bt.shape[1], page_size, head_dim,
+                    n_heads, n_kv, float(scale), int(window), self._stream(),
+                )
+            )
+        if use_mfma and tiles.shape[0] == 0:
+            return out
         if use_mfma:
             n_tiles = tiles.shape[0]
             hpt = self.lib.yk_attn_heads_per_tile(n_heads, n_kv)

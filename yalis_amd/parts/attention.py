@@ -50,6 +50,7 @@ class Attention(Mixer):
             raise ValueError("rotary_dim exceeds head_dim")
         rt.ops.check_attention_sizes(self.n_heads, self.n_kv, self.head_dim, rt.page_size)
         self.tokens_per_tile = rt.ops.attention_tokens_per_tile(self.n_heads, self.n_kv)
+        self.long_tile = rt.ops.attention_long_span_tile(self.n_heads, self.n_kv)
         self.group = None
         self.w_qkv = self.w_q = self.w_o = None
 
@@ -79,8 +80,14 @@ class Attention(Mixer):
         return KVNeed(self.n_kv, self.head_dim, self.window)
 
     def step_inputs(self):
+        # spans of more than one large tile go to the kernel for long spans, the rest
+        # (single decoded tokens, short portions) to the one that splits the keys
         tpt = self.tokens_per_tile
-        return {f"attention_tiles_{tpt}": lambda hb: attention_tiles(hb, tpt)}
+        big = self.rt.ops.attention_long_span_tile(self.n_heads, self.n_kv)
+        return {
+            f"attention_tiles_{tpt}_upto{big}": lambda hb: attention_tiles(hb, tpt, 1, big),
+            f"attention_long_tiles_{big}": lambda hb: attention_tiles(hb, big, big + 1),
+        }
 
     # ---- what it computes
     def forward(self, h: torch.Tensor, ctx, site) -> torch.Tensor:
@@ -122,6 +129,7 @@ class Attention(Mixer):
             0 if self.window is None else int(self.window),
             ctx,
             site.group,
-            ctx.arrays[f"attention_tiles_{self.tokens_per_tile}"],
+            ctx.arrays[f"attention_tiles_{self.tokens_per_tile}_upto{self.long_tile}"],
+            ctx.arrays[f"attention_long_tiles_{self.long_tile}"],
         )
         return ops.linear(out, self.w_o, self.rt.act_dtype, partial_ok=True)
