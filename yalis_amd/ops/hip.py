@@ -86,7 +86,7 @@ _SIGNATURES = {
 # above it the vendor library does.
 SKINNY_MAX_ROWS = 64
 # Waves the attention launch aims at when it decides how far to split the keys.
-ATTN_TARGET_WAVES = int(__import__('os').environ.get('YALIS_ATTN_WAVES', '2048'))
+ATTN_TARGET_WAVES = 1024
 
 
 class SplitSum:
