@@ -228,7 +228,7 @@ def test_rope_append(ops, dtype, h, g, d, rd, inter):
 
 
 # ------------------------------------------------------------------------- attention
-def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True, n_pages=64):
+def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True, n_pages=64, plan=None):
     """spans: list of (cached tokens before the step, new tokens).  Builds pages in a
     shuffled order, fills cache for the earlier tokens, runs rope-free attention."""
     gen = torch.Generator().manual_seed(seed)
@@ -264,7 +264,7 @@ def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True,
     n = hb.n_tokens
     q = (torch.randn((n, h * d), generator=gen) * 1.5).to(dtype)
     scale = 1.0 / math.sqrt(d)
-    got = ops.attention(q.to(DEV), h, g, d, kc.to(DEV), vc.to(DEV), page, scale, window, ctx, 0, ctx.arrays["tiles"], ctx.arrays["long_tiles"])
+    got = ops.attention(q.to(DEV), h, g, d, kc.to(DEV), vc.to(DEV), page, scale, window, ctx, 0, ctx.arrays["tiles"], ctx.arrays["long_tiles"], plan=plan)
     want = R.attention(q.float(), h, g, d, kc.float(), vc.float(), page, scale, window, ctx_cpu, 0, None)
     return got, want
 
@@ -301,6 +301,30 @@ def test_attention_mfma_long_context_splits(ops):
     close(got, want, 2e-2, 2**-6)
     got, want = _attention_case(ops, torch.bfloat16, 8, 2, 128, 64, spans, 700, seed=6, n_pages=48)
     close(got, want, 2e-2, 2**-6)
+
+
+@pytest.mark.parametrize("plan", [(1, 1), (4, 1), (1, 5), (4, 3), (4, 7)])
+@pytest.mark.parametrize("d", [64, 128])
+def test_attention_mfma_every_way_of_dividing_keys(ops, plan, d):
+    """Keys divided among the waves of a workgroup, among workgroups, or both, give the
+    same result; spans include ones with fewer key blocks than waves (idle waves hold
+    an empty part) and windows that cut the first block."""
+    spans = [(1500, 1), (900, 3), (0, 2), (63, 1), (64, 1), (200, 2)]
+    for window in (0, 700, 33):
+        got, want = _attention_case(ops, torch.bfloat16, 8, 2, d, 32, spans, window, seed=16, n_pages=96, plan=plan)
+        close(got, want, 2e-2, 2**-6)
+
+
+def test_attention_plan_covers_the_launch():
+    from yalis_amd.ops.hip import ATTN_TARGET_WAVES, HipOps
+
+    for groups in (1, 8, 64, 512, 5000):
+        for key_blocks in (1, 2, 5, 16, 128, 2048):
+            waves, splits = HipOps.attention_plan(groups, key_blocks)
+            assert waves in (1, 4) and 1 <= splits <= 256
+            if key_blocks == 1 or groups >= ATTN_TARGET_WAVES:
+                assert (waves, splits) == (1, 1)
+            assert waves * splits < 2 * 8 + max(key_blocks, 1) * 2
 
 
 def test_attention_far_key_stands_out(ops):

@@ -168,8 +168,14 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // row).  Every load is unconditional (addresses are clamped into allocated pages, what they
 // bring for keys that do not count is masked or zeroed), so that the values of a block and
 // the keys of the next are in flight while the block's scores are worked on.
-template <int D>
-__global__ __launch_bounds__(64) void attn_mfma_kernel(
+//
+// A workgroup has W waves that share the columns and divide the workgroup's key blocks
+// among themselves; at the end waves 1.. hand their running maximum, sum and output to
+// wave 0 through LDS (every lane to the same lane), and wave 0 merges and stores.  Across
+// workgroups (blockIdx.z) the keys are split further when the launch needs more waves;
+// those partial results go through the workspace to the combine kernel.
+template <int D, int W>
+__global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ block_table, int table_width,
@@ -177,7 +183,7 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
     int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml) {
   constexpr int KS = D / 32;  // matrix-core steps over the head dimension
   constexpr int DT = D / 16;  // output tiles over the head dimension
-  const int lane = threadIdx.x, r = lane % 16, gq = lane / 16;
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, gq = lane / 16;
   const int t = blockIdx.x;
   const int seq = tiles[4 * t], tok0 = tiles[4 * t + 1], ntok = tiles[4 * t + 2], pos0 = tiles[4 * t + 3];
   const int g = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
@@ -192,8 +198,11 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
   const int lo = window > 0 ? max(0, pos0 - window + 1) : 0;
   const int kb_lo = lo / 64, kb_hi = (hi + 63) / 64;
   const int per_split = (kb_hi - kb_lo + n_splits - 1) / n_splits;
-  const int my_lo = kb_lo + blockIdx.z * per_split;
-  const int my_hi = min(kb_hi, my_lo + per_split);
+  const int wg_lo = kb_lo + blockIdx.z * per_split;
+  const int wg_hi = min(kb_hi, wg_lo + per_split);
+  const int per_wave = (max(0, wg_hi - wg_lo) + W - 1) / W;
+  const int my_lo = wg_lo + wave * per_wave;
+  const int my_hi = min(wg_hi, my_lo + per_wave);
   const int32_t* bt = block_table + static_cast<size_t>(seq) * table_width;
   const int last_page_col = min(table_width - 1, (hi - 1) / page_size);
 
@@ -315,6 +324,36 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
 #undef ATT_LOAD_K
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
+
+  if (W > 1) {
+    constexpr int WP = W > 1 ? W - 1 : 1;
+    __shared__ f32x4_t part_o[WP][DT][64];
+    __shared__ float part_m[WP][64], part_l[WP][64];
+    if (wave > 0) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) part_o[wave - 1][dt][lane] = acc[dt];
+      part_m[wave - 1][lane] = m;
+      part_l[wave - 1][lane] = l;
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    float m_all = m;
+#pragma unroll
+    for (int w = 0; w < W - 1; ++w) m_all = fmaxf(m_all, part_m[w][lane]);
+    const float m_safe = m_all == -INFINITY ? 0.f : m_all;
+    const float a0 = fast_exp2(m - m_safe);
+    l *= a0;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[dt] *= a0;
+#pragma unroll
+    for (int w = 0; w < W - 1; ++w) {
+      const float aw = fast_exp2(part_m[w][lane] - m_safe);
+      l += aw * part_l[w][lane];
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) acc[dt] += aw * part_o[w][dt][lane];
+    }
+    m = m_all;
+  }
 
   if (n_splits == 1) {
     if (col_ok) {
@@ -658,9 +697,10 @@ extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* 
                             const void* v_cache, const int32_t* tiles, int n_tiles,
                             const int32_t* block_table, int table_width, int page_size,
                             int head_dim, int n_heads, int n_kv, float scale, int window,
-                            int n_splits, float* workspace, size_t workspace_floats,
+                            int n_waves, int n_splits, float* workspace, size_t workspace_floats,
                             hipStream_t stream) {
   YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_mfma: bad head counts");
+  YK_REQUIRE(n_waves == 1 || n_waves == 4, "attn_mfma: a workgroup has 1 or 4 waves");
   YK_REQUIRE(yk_attn_mfma_supported(head_dim), "attn_mfma: head_dim must be 64 or 128");
   YK_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_mfma: page_size must be a multiple of 16");
   YK_REQUIRE(q_stride % 8 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0,
@@ -678,12 +718,14 @@ extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* 
   float* ws_o = workspace;
   float* ws_ml = workspace ? workspace + (need / (head_dim + 2)) * head_dim : nullptr;
   const float scale_log2 = scale * 1.4426950408889634f;
-  dim3 grid(n_tiles, n_kv * chunks, n_splits), block(64);
-#define YK_LAUNCH(DD)                                                                              \
-  attn_mfma_kernel<DD><<<grid, block, 0, stream>>>(                                                \
+  dim3 grid(n_tiles, n_kv * chunks, n_splits), block(64 * n_waves);
+#define YK_ARGS                                                                                    \
       static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out),                          \
       static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), tiles, block_table, \
-      table_width, page_size, n_heads, n_kv, hpt, chunks, scale_log2, window, n_splits, ws_o, ws_ml); \
+      table_width, page_size, n_heads, n_kv, hpt, chunks, scale_log2, window, n_splits, ws_o, ws_ml
+#define YK_LAUNCH(DD)                                                                              \
+  if (n_waves == 1) attn_mfma_kernel<DD, 1><<<grid, block, 0, stream>>>(YK_ARGS);                  \
+  else attn_mfma_kernel<DD, 4><<<grid, block, 0, stream>>>(YK_ARGS);                               \
   if (yk_check_launch("attn_mfma")) return -1;                                                     \
   if (n_splits > 1) {                                                                              \
     attn_combine_kernel<DD><<<dim3(n_tiles, n_kv * chunks), 256, 0, stream>>>(                     \
@@ -696,5 +738,6 @@ extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* 
     YK_LAUNCH(128)
   }
 #undef YK_LAUNCH
+#undef YK_ARGS
   return 0;
 }

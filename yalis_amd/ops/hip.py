@@ -11,7 +11,7 @@ product and everything else are the hand-written kernels.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -75,7 +75,7 @@ _SIGNATURES = {
         _c_int,
     ),
     "yk_attn_mfma": (
-        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _vp, _c_size_t, _vp],
+        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _vp],
         _c_int,
     ),
     "yk_argmax": ([_vp, _vp, _c_int, _c_int, _vp, _c_size_t, _vp], _c_int),
@@ -316,11 +316,22 @@ class HipOps:
         return q_out
 
     # ------------------------------------------------------------------ attention
+    @staticmethod
+    def attention_plan(column_groups: int, key_blocks: int) -> Tuple[int, int]:
+        """(waves per workgroup, splits across workgroups) for the short-span kernel: the
+        keys of a column group are divided until the launch has about ATTN_TARGET_WAVES
+        waves, first among the waves of a workgroup (merged through LDS, no second kernel),
+        then across workgroups (merged by the combine kernel)."""
+        par = max(1, min(-(-ATTN_TARGET_WAVES // max(1, column_groups)), key_blocks))
+        if par == 1:
+            return 1, 1
+        return 4, max(1, min(-(-par // 4), 256))
+
     def attention(self, qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size,
-                  scale, window, ctx, group, tiles, long_tiles=None) -> torch.Tensor:
+                  scale, window, ctx, group, tiles, long_tiles=None, plan=None) -> torch.Tensor:
         """Queries are the first n_heads heads of each row of ``qkv`` (whatever follows
         them in the row is skipped); keys and values come from the cache through the
-        block table of ``group``."""
+        block table of ``group``.  ``plan`` overrides ``attention_plan`` (tests, measurements)."""
         self._rows(qkv, "qkv")
         n = qkv.shape[0]
         bt = ctx.arrays[f"block_table_g{group}"]
@@ -349,16 +360,15 @@ class HipOps:
             n_tiles = tiles.shape[0]
             hpt = self.lib.yk_attn_heads_per_tile(n_heads, n_kv)
             chunks = -(-(n_heads // n_kv) // hpt)
-            waves = n_tiles * n_kv * chunks
             key_blocks = max(1, -(-ctx.max_ctx // 64))
-            splits = max(1, min(-(-ATTN_TARGET_WAVES // waves), key_blocks, 256))
+            waves, splits = plan or self.attention_plan(n_tiles * n_kv * chunks, key_blocks)
             ws_floats = self.lib.yk_attn_mfma_workspace(n_tiles, n_heads, n_kv, head_dim, splits)
             ws = self._ws(ws_floats) if ws_floats else None
             self._check(
                 self.lib.yk_attn_mfma(
                     qkv.data_ptr(), qkv.stride(0), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                     tiles.data_ptr(), n_tiles, bt.data_ptr(), bt.shape[1], page_size, head_dim, n_heads, n_kv,
-                    float(scale), int(window), splits, _ptr(ws), 0 if ws is None else ws.numel(), self._stream(),
+                    float(scale), int(window), waves, splits, _ptr(ws), 0 if ws is None else ws.numel(), self._stream(),
                 )
             )
         else:
