@@ -255,7 +255,7 @@ def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True,
     hb = build_host_batch(seqs, 1, page)
     tpt = ops.attention_tokens_per_tile(h, g)
     big = ops.attention_long_span_tile(h, g)
-    arrays = named_arrays(hb, {"tiles": lambda b: attention_tiles(b, tpt, 1, big), "long_tiles": lambda b: attention_tiles(b, big, big + 1)})
+    arrays = named_arrays(hb, {"tiles": lambda b: attention_tiles(b, tpt, 1, big), "long_tiles": lambda b: attention_tiles(b, big, big + 1, longest_first=(seed % 2 == 0))})
     ctx = types.SimpleNamespace(
         arrays={k: torch.from_numpy(np.ascontiguousarray(v)).to(DEV) for k, v in arrays.items()},
         max_ctx=hb.max_ctx,

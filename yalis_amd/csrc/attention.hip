@@ -380,40 +380,58 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
   }
 }
 
-// The same arithmetic for long spans (prompt portions): a workgroup of four waves owns four
-// consecutive tiles of one request (64 columns) and walks the keys once for all of them.
-// Each block of 64 keys and values is fetched from the pages with coalesced loads, parked
-// in LDS (keys in the row order the score products read them, so that the reads are free of
-// bank conflicts) and read from there by the four waves; the next block's loads are in
-// flight meanwhile.  No split of the keys: long spans bring enough workgroups.
+// The same arithmetic for long spans (prompt portions): a workgroup of four waves owns one
+// long tile of a request; every wave has PF_CT column tiles of 16 (consecutive tokens), so
+// the workgroup walks the keys once for 64 * PF_CT columns and every key or value operand
+// read from LDS feeds PF_CT products.  Each block of 64 keys and values is fetched from the
+// pages with coalesced loads, parked in LDS (keys in the row order the score products read
+// them, so that the reads are free of bank conflicts) and read from there by the four
+// waves; the next block's loads are in flight meanwhile.  No split of the keys: long spans
+// bring enough workgroups.  Measured on 2,048-token prompts: one column tile per wave with
+// three workgroups resident per CU (the launch bound below keeps the registers to that) is
+// the fastest; more columns per wave save LDS reads but leave too few workgroups to balance
+// the triangle of a causal prompt.
+constexpr int PF_CT = 1;
+
 template <int D, bool BLOCK_IN_PAGE>
-__global__ __launch_bounds__(256) void attn_mfma_prefill_kernel(
+__global__ __launch_bounds__(256, 3) void attn_mfma_prefill_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ block_table, int table_width,
     int page_size, int n_heads, int n_kv, int hpt, int chunks, float scale_log2, int window) {
-  constexpr int KS = D / 32, DT = D / 16;
+  constexpr int KS = D / 32, DT = D / 16, CT = PF_CT;
   constexpr int KROW = D + 8;   // bf16 elements per parked key row
   constexpr int VROW = 64 + 8;  // bf16 elements per parked value row
   constexpr int PP = D / 32;    // 16-byte pieces of keys (and of values) per thread and block
   __shared__ __attribute__((aligned(16))) bf16_t ks[64][KROW];
   __shared__ __attribute__((aligned(16))) bf16_t vs[D][VROW];
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, gq = lane / 16;
-  const int t = blockIdx.x;
+  // Workgroups start in the order of blockIdx.x: heads vary fastest, so that the tiles the
+  // host put first (those with the most keys) start first on every head and the short ones
+  // fill the gaps at the end; consecutive workgroups, which land on different dies, hold
+  // different kv heads.
+  const int n_y = n_kv * chunks;
+  const int t = blockIdx.x / n_y, by = blockIdx.x % n_y;
   const int seq = tiles[4 * t], tile_tok0 = tiles[4 * t + 1], tile_ntok = tiles[4 * t + 2], tile_pos0 = tiles[4 * t + 3];
-  const int g = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+  const int g = by / chunks, chunk = by % chunks;
   const int qpk = n_heads / n_kv;
   const int h_base = g * qpk + chunk * hpt;
   const int heads_here = min(hpt, qpk - chunk * hpt);
-  const int tpt = 16 / hpt;  // tokens per wave
+  const int tpt = 16 / hpt;  // tokens per column tile
   const int tt = r / hpt, hh = r % hpt;
-  const int tok_in_tile = wave * tpt + tt;
-  const bool col_ok = tt < tpt && tok_in_tile < tile_ntok && hh < heads_here;
-  const int pos_c = tile_pos0 + tok_in_tile;
-  const int lo_c = window > 0 ? max(0, pos_c - window + 1) : 0;
+  const int wave_tok0 = wave * CT * tpt;  // first token of this wave within the tile
+  int tok_c[CT], pos_c[CT], lo_c[CT];
+  bool col_ok[CT];
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    tok_c[c] = wave_tok0 + c * tpt + tt;
+    col_ok[c] = tt < tpt && tok_c[c] < tile_ntok && hh < heads_here;
+    pos_c[c] = tile_pos0 + tok_c[c];
+    lo_c[c] = window > 0 ? max(0, pos_c[c] - window + 1) : 0;
+  }
   const int hi = tile_pos0 + tile_ntok;  // keys the workgroup may need
   const int lo = window > 0 ? max(0, tile_pos0 - window + 1) : 0;
-  const int wave_hi = min(hi, tile_pos0 + (wave + 1) * tpt);  // keys this wave may need
+  const int wave_hi = min(hi, tile_pos0 + wave_tok0 + CT * tpt);  // keys this wave may need
   const int kb_lo = lo / 64, kb_hi = (hi + 63) / 64;
   const int32_t* bt = block_table + static_cast<size_t>(seq) * table_width;
   const int last_page_col = min(table_width - 1, (hi - 1) / page_size);
@@ -435,20 +453,26 @@ __global__ __launch_bounds__(256) void attn_mfma_prefill_kernel(
   __syncthreads();
 
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
-  AFrag8 qf[KS];
-  {
-    const bf16_t* qp = q + static_cast<size_t>(tile_tok0 + (col_ok ? tok_in_tile : 0)) * q_stride +
-                       static_cast<size_t>(h_base + (col_ok ? hh : 0)) * D + 8 * gq;
+  AFrag8 qf[CT][KS];
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    const bf16_t* qp = q + static_cast<size_t>(tile_tok0 + (col_ok[c] ? tok_c[c] : 0)) * q_stride +
+                       static_cast<size_t>(h_base + (col_ok[c] ? hh : 0)) * D + 8 * gq;
 #pragma unroll
     for (int ks_ = 0; ks_ < KS; ++ks_) {
-      qf[ks_].u = *reinterpret_cast<const u32x4_t*>(qp + 32 * ks_);
-      if (!col_ok) qf[ks_].u = zero4;
+      qf[c][ks_].u = *reinterpret_cast<const u32x4_t*>(qp + 32 * ks_);
+      if (!col_ok[c]) qf[c][ks_].u = zero4;
     }
   }
-  float m = -INFINITY, l = 0.f;
-  f32x4_t acc[DT];
+  float m[CT], l[CT];
+  f32x4_t acc[CT][DT];
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int c = 0; c < CT; ++c) {
+    m[c] = -INFINITY;
+    l[c] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[c][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
 
   // what this thread fetches of every block: PP pieces of keys and PP pieces of values.
   // With pages of a multiple of 64 tokens a block of keys lies in one page: the page id is
@@ -520,82 +544,96 @@ __global__ __launch_bounds__(256) void attn_mfma_prefill_kernel(
     if (kb + 1 < kb_hi) PF_LOAD(kb + 1)  // in flight while this block is worked on
     if (kb * 64 >= wave_hi) continue;  // nothing of this block is visible to this wave
 
-    f32x4_t s[2][2];
+    f32x4_t s[CT][2][2];
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
       for (int sb = 0; sb < 2; ++sb) {
-        s[u][sb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < CT; ++c) s[c][u][sb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks_ = 0; ks_ < KS; ++ks_) {
           AFrag8 a;
           a.u = *reinterpret_cast<const u32x4_t*>(&ks[32 * u + 16 * sb + r][32 * ks_ + 8 * gq]);
-          s[u][sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[ks_].v, s[u][sb], 0, 0, 0);
+#pragma unroll
+          for (int c = 0; c < CT; ++c)
+            s[c][u][sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[c][ks_].v, s[c][u][sb], 0, 0, 0);
         }
       }
-    float tmax = -INFINITY;
     // a block that every column sees whole needs no mask (columns that stand for nothing
     // compute on zeros and are never stored)
-    const bool whole = kb * 64 + 63 <= (tile_pos0 + wave * tpt) && (window == 0 || kb * 64 >= max(0, wave_hi - window));
+    const bool whole = kb * 64 + 63 <= (tile_pos0 + wave_tok0) && (window == 0 || kb * 64 >= max(0, wave_hi - window));
+    AFrag8 pf[CT][2];
+    float alpha[CT];
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
+    for (int c = 0; c < CT; ++c) {
+      float tmax = -INFINITY;
 #pragma unroll
-      for (int sb = 0; sb < 2; ++sb)
+      for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          if (whole) {
-            s[u][sb][i] *= scale_log2;
-          } else {
-            const int key = kb * 64 + 32 * u + 8 * gq + 4 * sb + i;
-            const bool ok = col_ok && key <= pos_c && key >= lo_c;
-            s[u][sb][i] = ok ? s[u][sb][i] * scale_log2 : -INFINITY;
+        for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            if (whole) {
+              s[c][u][sb][i] *= scale_log2;
+            } else {
+              const int key = kb * 64 + 32 * u + 8 * gq + 4 * sb + i;
+              const bool ok = col_ok[c] && key <= pos_c[c] && key >= lo_c[c];
+              s[c][u][sb][i] = ok ? s[c][u][sb][i] * scale_log2 : -INFINITY;
+            }
+            tmax = fmaxf(tmax, s[c][u][sb][i]);
           }
-          tmax = fmaxf(tmax, s[u][sb][i]);
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(m[c], tmax);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      alpha[c] = fast_exp2(m[c] - m_safe);
+      float psum = 0.f;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            s[c][u][sb][i] = fast_exp2(s[c][u][sb][i] - m_safe);
+            psum += s[c][u][sb][i];
+          }
+          pf[c][u].u[2 * sb] = pack_bf16x2(s[c][u][sb][0], s[c][u][sb][1]);
+          pf[c][u].u[2 * sb + 1] = pack_bf16x2(s[c][u][sb][2], s[c][u][sb][3]);
         }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float m_new = fmaxf(m, tmax);
-    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = fast_exp2(m - m_safe);
-    float psum = 0.f;
-    AFrag8 pf[2];
-#pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-      for (int sb = 0; sb < 2; ++sb) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          s[u][sb][i] = fast_exp2(s[u][sb][i] - m_safe);
-          psum += s[u][sb][i];
-        }
-        pf[u].u[2 * sb] = pack_bf16x2(s[u][sb][0], s[u][sb][1]);
-        pf[u].u[2 * sb + 1] = pack_bf16x2(s[u][sb][2], s[u][sb][3]);
-      }
-    l = l * alpha + psum;
-    m = m_new;
+      l[c] = l[c] * alpha[c] + psum;
+      m[c] = m_new;
+    }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      acc[dt] *= alpha;
+#pragma unroll
+      for (int c = 0; c < CT; ++c) acc[c][dt] *= alpha[c];
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         AFrag8 a;
         a.u = *reinterpret_cast<const u32x4_t*>(&vs[16 * dt + r][32 * u + 8 * gq]);
-        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pf[u].v, acc[dt], 0, 0, 0);
+#pragma unroll
+        for (int c = 0; c < CT; ++c)
+          acc[c][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pf[c][u].v, acc[c][dt], 0, 0, 0);
       }
     }
   }
 #undef PF_LOAD
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
-  if (col_ok) {
-    const float inv = 1.f / l;
-    bf16_t* op = out + (static_cast<size_t>(tile_tok0 + tok_in_tile) * n_heads + h_base + hh) * D + 4 * gq;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      u32x2_t w;
-      w[0] = pack_bf16x2(acc[dt][0] * inv, acc[dt][1] * inv);
-      w[1] = pack_bf16x2(acc[dt][2] * inv, acc[dt][3] * inv);
-      *reinterpret_cast<u32x2_t*>(op + 16 * dt) = w;
+  for (int c = 0; c < CT; ++c) {
+    float lc = l[c];
+    lc += __shfl_xor(lc, 16, 64);
+    lc += __shfl_xor(lc, 32, 64);
+    if (col_ok[c]) {
+      const float inv = 1.f / lc;
+      bf16_t* op = out + (static_cast<size_t>(tile_tok0 + tok_c[c]) * n_heads + h_base + hh) * D + 4 * gq;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        u32x2_t w;
+        w[0] = pack_bf16x2(acc[c][dt][0] * inv, acc[c][dt][1] * inv);
+        w[1] = pack_bf16x2(acc[c][dt][2] * inv, acc[c][dt][3] * inv);
+        *reinterpret_cast<u32x2_t*>(op + 16 * dt) = w;
+      }
     }
   }
 }
@@ -647,6 +685,10 @@ extern "C" int yk_attn_heads_per_tile(int n_heads, int n_kv) {
 extern "C" int yk_attn_tokens_per_tile(int n_heads, int n_kv) {
   return 16 / yk_attn_heads_per_tile(n_heads, n_kv);
 }
+// Tokens of one long tile (a workgroup of the long-span kernel): four waves of PF_CT column tiles.
+extern "C" int yk_attn_long_tile_tokens(int n_heads, int n_kv) {
+  return 4 * PF_CT * yk_attn_tokens_per_tile(n_heads, n_kv);
+}
 
 // Floats of workspace for a launch with n_splits > 1: outputs, then (max, sum) pairs.
 extern "C" size_t yk_attn_mfma_workspace(int n_tiles, int n_heads, int n_kv, int head_dim,
@@ -658,7 +700,7 @@ extern "C" size_t yk_attn_mfma_workspace(int n_tiles, int n_heads, int n_kv, int
   return w * head_dim + w * 2;
 }
 
-// Long spans: ``tiles`` hold up to 4 * tokens_per_tile tokens each (one workgroup a tile).
+// Long spans: ``tiles`` hold up to yk_attn_long_tile_tokens tokens each (one workgroup a tile).
 extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, const void* k_cache,
                                     const void* v_cache, const int32_t* tiles, int n_tiles,
                                     const int32_t* block_table, int table_width, int page_size,
@@ -675,9 +717,9 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
   if (n_tiles == 0) return 0;
   const int hpt = yk_attn_heads_per_tile(n_heads, n_kv);
   const int chunks = (n_heads / n_kv + hpt - 1) / hpt;
-  YK_REQUIRE(n_kv * chunks <= 65535, "attn_mfma_prefill: too many heads for one launch");
+  YK_REQUIRE(static_cast<long long>(n_tiles) * n_kv * chunks <= 0x7fffffffLL, "attn_mfma_prefill: too many tiles for one launch");
   const float scale_log2 = scale * 1.4426950408889634f;
-  dim3 grid(n_tiles, n_kv * chunks), block(256);
+  dim3 grid(n_tiles * n_kv * chunks), block(256);
 #define YK_PF(DD, BIP)                                                                                       \
   attn_mfma_prefill_kernel<DD, BIP><<<grid, block, 0, stream>>>(                                                 \
       static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),   \

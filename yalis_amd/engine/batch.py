@@ -143,11 +143,14 @@ def pack(arrays: Dict[str, np.ndarray]) -> Tuple[np.ndarray, Dict[str, Tuple[int
     return buf, layout
 
 
-def attention_tiles(hb: HostBatch, tokens_per_tile: int, min_span: int = 1, max_span: int = 1 << 30) -> np.ndarray:
+def attention_tiles(hb: HostBatch, tokens_per_tile: int, min_span: int = 1, max_span: int = 1 << 30,
+                    longest_first: bool = False) -> np.ndarray:
     """Cut every request's span into tiles of at most ``tokens_per_tile``
     consecutive tokens: rows of (request, first token index in the batch, token
     count, first position).  Only spans of min_span..max_span tokens are cut (a kernel
-    for long spans and one for short ones each get their own list)."""
+    for long spans and one for short ones each get their own list).  ``longest_first``
+    orders the tiles by the keys they see, most first: workgroups start in that order,
+    and the short ones then fill the end of the launch."""
     rows = []
     for i in range(hb.n_seqs):
         q0 = int(hb.seq_qstart[i])
@@ -157,4 +160,6 @@ def attention_tiles(hb: HostBatch, tokens_per_tile: int, min_span: int = 1, max_
         p0 = int(hb.seq_ctx[i]) - ql
         for t in range(0, ql, tokens_per_tile):
             rows.append((i, q0 + t, min(tokens_per_tile, ql - t), p0 + t))
+    if longest_first:
+        rows.sort(key=lambda row: -(row[3] + row[2]))
     return np.array(rows, dtype=np.int32).reshape(-1, 4)

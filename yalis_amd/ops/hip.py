@@ -68,6 +68,7 @@ _SIGNATURES = {
     ),
     "yk_attn_mfma_supported": ([_c_int], _c_int),
     "yk_attn_heads_per_tile": ([_c_int, _c_int], _c_int),
+    "yk_attn_long_tile_tokens": ([_c_int, _c_int], _c_int),
     "yk_attn_tokens_per_tile": ([_c_int, _c_int], _c_int),
     "yk_attn_mfma_workspace": ([_c_int, _c_int, _c_int, _c_int, _c_int], _c_size_t),
     "yk_attn_mfma_prefill": (
@@ -174,8 +175,8 @@ class HipOps:
         return self.lib.yk_attn_tokens_per_tile(n_heads, n_kv)
 
     def attention_long_span_tile(self, n_heads: int, n_kv: int) -> int:
-        """Tokens per tile of the kernel for long spans (four waves of tokens_per_tile)."""
-        return 4 * self.lib.yk_attn_tokens_per_tile(n_heads, n_kv)
+        """Tokens per tile of the kernel for long spans (one workgroup a tile)."""
+        return self.lib.yk_attn_long_tile_tokens(n_heads, n_kv)
 
     # ------------------------------------------------------------------ embedding
     def embed(self, token_ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:

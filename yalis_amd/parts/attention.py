@@ -86,7 +86,7 @@ class Attention(Mixer):
         big = self.rt.ops.attention_long_span_tile(self.n_heads, self.n_kv)
         return {
             f"attention_tiles_{tpt}_upto{big}": lambda hb: attention_tiles(hb, tpt, 1, big),
-            f"attention_long_tiles_{big}": lambda hb: attention_tiles(hb, big, big + 1),
+            f"attention_long_tiles_{big}": lambda hb: attention_tiles(hb, big, big + 1, longest_first=True),
         }
 
     # ---- what it computes
