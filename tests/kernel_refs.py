@@ -152,7 +152,7 @@ class RefOps:
     gated_act = staticmethod(gated_act)
     argmax = staticmethod(argmax)
 
-    def sample(self, logits, temperature, top_k, top_p, seeds, draws):
+    def sample(self, logits, temperature, top_k, top_p, seeds, draws, whole_row=False):
         from plain_llama import sample_token
 
         out = []

@@ -384,12 +384,12 @@ def test_argmax_lowest_index_on_ties(ops):
     assert torch.equal(got[2:].long(), want[2:])
 
 
-def _sample(ops, logits, temperature, top_k, top_p, seed, draw):
+def _sample(ops, logits, temperature, top_k, top_p, seed, draw, whole_row=False):
     rows = logits.shape[0]
     f = lambda v, dt: torch.full((rows,), v, dtype=dt, device=DEV)
     return ops.sample(
         logits, f(temperature, torch.float32), f(top_k, torch.int32), f(top_p, torch.float32),
-        f(seed, torch.int32), torch.arange(draw, draw + rows, dtype=torch.int32, device=DEV),
+        f(seed, torch.int32), torch.arange(draw, draw + rows, dtype=torch.int32, device=DEV), whole_row=whole_row,
     ).cpu()
 
 
@@ -402,6 +402,54 @@ def test_sample_matches_plain(ops):
             got = _sample(ops, logits, temperature, top_k, top_p, 99, draw)[0].item()
             want = P.sample_token(logits[0].cpu(), temperature, top_k or None, top_p, 99, draw)
             assert got == want, (temperature, top_k, top_p, draw)
+
+
+SAMPLE_SETTINGS = [(0.7, 0, 1.0), (1.0, 5, 1.0), (1.3, 0, 0.8), (0.9, 50, 0.5), (1.0, 1, 1.0), (1.0, 0, 0.0),
+                   (0.8, 3000, 0.95), (1.0, 6000, 0.9), (2.0, 0, 0.999), (1.1, 700, 1.0), (0.6, 5000, 1.0)]
+
+
+@pytest.mark.parametrize("vocab,kind", [(32003, "peaked"), (128256, "peaked"), (20000, "flat"), (9001, "ties")])
+def test_sample_large_vocabulary_matches_plain(ops, vocab, kind):
+    """Rows larger than the candidate store: peaked rows narrow down to a few tokens, a
+    flat row under top_p alone and a row of thousands of equal logits fall back to the
+    whole-row path; every way gives the plain implementation's token, and the forced
+    whole-row path agrees."""
+    import plain_llama as P
+
+    gen = torch.Generator().manual_seed(vocab)
+    if kind == "peaked":
+        logits = torch.randn((1, vocab), generator=gen) * 3.0
+    elif kind == "flat":
+        logits = torch.randn((1, vocab), generator=gen) * 0.01
+    else:
+        logits = torch.randn((1, vocab), generator=gen).round()  # a handful of distinct values
+    logits = logits.to(DEV)
+    for temperature, top_k, top_p in SAMPLE_SETTINGS:
+        if kind == "ties" and top_p < 1.0:
+            # which of several equally likely tokens top_p keeps is left to the sort in the
+            # reference (yalis/external/sampling.py:24); the kernel drops them together
+            continue
+        for draw in range(4):
+            want = P.sample_token(logits[0].cpu(), temperature, top_k or None, top_p, 7, draw)
+            got = _sample(ops, logits, temperature, top_k, top_p, 7, draw)[0].item()
+            slow = _sample(ops, logits, temperature, top_k, top_p, 7, draw, whole_row=True)[0].item()
+            assert got == want and slow == want, (kind, temperature, top_k, top_p, draw, got, slow, want)
+
+
+def test_sample_rows_are_independent(ops):
+    """Many rows with different settings in one launch give what each gives alone."""
+    vocab = 50000
+    logits = rnd((6, vocab), torch.float32, 41, scale=2.5)
+    temperature = torch.tensor([0.0, 0.7, 1.0, 1.2, 0.9, 1.0], dtype=torch.float32, device=DEV)
+    top_k = torch.tensor([0, 40, 0, 5000, 0, 1], dtype=torch.int32, device=DEV)
+    top_p = torch.tensor([1.0, 0.9, 0.5, 1.0, 1.0, 0.3], dtype=torch.float32, device=DEV)
+    seeds = torch.arange(6, dtype=torch.int32, device=DEV) + 100
+    draws = torch.arange(6, dtype=torch.int32, device=DEV) * 3
+    both = ops.sample(logits, temperature, top_k, top_p, seeds, draws).cpu()
+    for i in range(6):
+        alone = ops.sample(logits[i : i + 1].contiguous(), temperature[i : i + 1], top_k[i : i + 1], top_p[i : i + 1],
+                           seeds[i : i + 1], draws[i : i + 1]).cpu()
+        assert both[i].item() == alone[0].item()
 
 
 def test_sample_frequencies(ops):

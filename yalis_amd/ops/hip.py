@@ -80,7 +80,7 @@ _SIGNATURES = {
         _c_int,
     ),
     "yk_argmax": ([_vp, _vp, _c_int, _c_int, _vp, _c_size_t, _vp], _c_int),
-    "yk_sample": ([_vp, _vp, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _vp], _c_int),
+    "yk_sample": ([_vp, _vp, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _vp], _c_int),
 }
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
@@ -420,9 +420,10 @@ class HipOps:
                                        ws.data_ptr(), ws.numel(), self._stream()))
         return out
 
-    def sample(self, logits, temperature, top_k, top_p, seeds, draws) -> torch.Tensor:
+    def sample(self, logits, temperature, top_k, top_p, seeds, draws, whole_row: bool = False) -> torch.Tensor:
         """Per row: temperature (float32; 0 = greedy), top_k (int32; 0 = off), top_p
-        (float32), seed and draw number (int32).  Returns int32 token ids."""
+        (float32), seed and draw number (int32).  Returns int32 token ids.  ``whole_row``
+        forces the path that never narrows the row down to candidates (for tests)."""
         if logits.dtype != torch.float32 or not logits.is_contiguous() or logits.dim() != 2:
             raise KernelError("sample takes contiguous float32 logits [rows, vocab]")
         rows = logits.shape[0]
@@ -434,7 +435,7 @@ class HipOps:
         self._check(
             self.lib.yk_sample(
                 logits.data_ptr(), out.data_ptr(), rows, logits.shape[1], temperature.data_ptr(), top_k.data_ptr(),
-                top_p.data_ptr(), seeds.data_ptr(), draws.data_ptr(), self._stream(),
+                top_p.data_ptr(), seeds.data_ptr(), draws.data_ptr(), int(bool(whole_row)), self._stream(),
             )
         )
         return out
