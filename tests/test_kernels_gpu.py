@@ -227,6 +227,43 @@ def test_rope_append(ops, dtype, h, g, d, rd, inter):
         assert torch.equal(vc.cpu(), vc_r), "values are copied, not changed"
 
 
+@pytest.mark.parametrize("h,g,d,rd,page", [(8, 2, 128, 128, 64), (6, 3, 64, 32, 16), (4, 4, 48, 48, 32), (5, 1, 80, 16, 16)])
+def test_rope_append_prompt_portions(ops, h, g, d, rd, page):
+    """Many bfloat16 tokens: portions whose slots run on from a multiple of 8 (values stored
+    as 16-byte pieces), portions that start anywhere, scattered single tokens, a token count
+    that is no multiple of 8; everything else in the pages stays as it was."""
+    u = 64  # slots are laid out in units of 64 whatever the page size
+    n_pages = 12 * u // page
+    runs = [(3 * u, 40), (7 * u + 5, 19), (0, u), (9 * u + 8, 11)]  # (first slot, tokens)
+    slots, positions = [], []
+    for first, count in runs:
+        slots += list(range(first, first + count))
+        positions += list(range(first % 50, first % 50 + count))
+    scattered = [5 * u + 3, 2 * u + 9, 11 * u + 1]
+    slots += scattered
+    positions += [190, 0, 77]
+    n = len(slots)
+    assert n % 8 != 0 and len(set(slots)) == n
+    qkv = rnd((n, (h + 2 * g) * d), torch.bfloat16, 40)
+    cos, sin = _tables(rd, 200)
+    positions = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    slots = torch.tensor(slots, dtype=torch.int32, device=DEV)
+    kc = rnd((n_pages, g, page, d), torch.bfloat16, 41)
+    vc = rnd((n_pages, g, d, page), torch.bfloat16, 42)
+    kc_r, vc_r, qkv_r = kc.cpu().clone(), vc.cpu().clone(), qkv.cpu().clone()
+    ops.rope_append(qkv, h, g, d, positions, cos, sin, rd, False, kc, vc, slots, page)
+    R.rope_append(qkv_r, h, g, d, positions.cpu(), cos.cpu(), sin.cpu(), rd, False, kc_r, vc_r, slots.cpu(), page)
+    close(qkv.view(n, -1, d)[:, :h], qkv_r.view(n, -1, d)[:, :h], 2**-7, 2**-7)
+    close(kc, kc_r, 2**-7, 2**-7)
+    assert torch.equal(vc.cpu(), vc_r), "values are copied, not changed"
+    # the same rows one token at a time (the scalar kernel) give the same bits
+    qkv1 = rnd((n, (h + 2 * g) * d), torch.bfloat16, 40)
+    kc1, vc1 = rnd((n_pages, g, page, d), torch.bfloat16, 41), rnd((n_pages, g, d, page), torch.bfloat16, 42)
+    for i in range(n):
+        ops.rope_append(qkv1[i : i + 1], h, g, d, positions[i : i + 1], cos, sin, rd, False, kc1, vc1, slots[i : i + 1], page)
+    assert torch.equal(qkv1.view(n, -1, d)[:, :h], qkv.view(n, -1, d)[:, :h]) and torch.equal(kc1, kc) and torch.equal(vc1, vc)
+
+
 # ------------------------------------------------------------------------- attention
 def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True, n_pages=64, plan=None):
     """spans: list of (cached tokens before the step, new tokens).  Builds pages in a

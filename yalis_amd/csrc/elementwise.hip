@@ -295,6 +295,11 @@ extern "C" int yk_add_rmsnorm(float* residual, const void* delta, int delta_dtyp
 // (position, pair index i): a' = a cos - b sin, b' = b cos + a sin; pairs are
 // (i, i + rotary_dim/2) ("half") or (2i, 2i + 1) ("interleaved"); elements beyond
 // rotary_dim pass unchanged.
+// one rounding of b*s (or a*s), then a fused multiply-add: written out so that every kernel
+// that rotates gives the same bits
+__device__ __forceinline__ float rot_first(float a, float b, float c, float s) { return fmaf(a, c, -__fmul_rn(b, s)); }
+__device__ __forceinline__ float rot_second(float a, float b, float c, float s) { return fmaf(b, c, __fmul_rn(a, s)); }
+
 template <typename TS, typename T>
 __global__ void rope_append_kernel(const TS* src, int n_splits, size_t split_stride,
                                    int src_stride, T* q_out, int q_stride, int n_heads,
@@ -344,10 +349,115 @@ __global__ void rope_append_kernel(const TS* src, int n_splits, size_t split_str
     const int ib = interleaved ? 2 * i + 1 : i + half;
     const float a = value(base + ia), b = value(base + ib);
     const float c = cs[i], s = sn[i];
-    dst[ia] = from_f32<T>(a * c - b * s);
-    dst[ib] = from_f32<T>(b * c + a * s);
+    dst[ia] = from_f32<T>(rot_first(a, b, c, s));
+    dst[ib] = from_f32<T>(rot_second(a, b, c, s));
   }
   for (int d = rotary_dim + threadIdx.x; d < head_dim; d += blockDim.x) dst[d] = from_f32<T>(value(base + d));
+}
+
+// The same for many tokens of plain bfloat16 rows with "half" pairs: a workgroup takes
+// ROPE_TOK consecutive tokens of one head and moves 16 bytes per access.  Value heads
+// (blockIdx.y beyond the query and key heads) gather the tokens' elements of one value row
+// and, where the tokens' slots are consecutive and start at a multiple of ROPE_TOK (a
+// prompt portion that starts on such a boundary), store them as one 16-byte piece of the
+// transposed page instead of ROPE_TOK separate elements.
+constexpr int ROPE_TOK = 8;
+
+__device__ __forceinline__ void rope_rotate8(const uint4& a, const uint4& b, const float* __restrict__ c,
+                                             const float* __restrict__ s, uint4& oa, uint4& ob) {
+  const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+  uint32_t ra[4], rb[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float a0 = __uint_as_float(aw[j] << 16), a1 = __uint_as_float(aw[j] & 0xffff0000u);
+    const float b0 = __uint_as_float(bw[j] << 16), b1 = __uint_as_float(bw[j] & 0xffff0000u);
+    const float c0 = c[2 * j], c1 = c[2 * j + 1], s0 = s[2 * j], s1 = s[2 * j + 1];
+    ra[j] = static_cast<uint32_t>(from_f32<bf16_t>(rot_first(a0, b0, c0, s0))) |
+            (static_cast<uint32_t>(from_f32<bf16_t>(rot_first(a1, b1, c1, s1))) << 16);
+    rb[j] = static_cast<uint32_t>(from_f32<bf16_t>(rot_second(a0, b0, c0, s0))) |
+            (static_cast<uint32_t>(from_f32<bf16_t>(rot_second(a1, b1, c1, s1))) << 16);
+  }
+  oa = make_uint4(ra[0], ra[1], ra[2], ra[3]);
+  ob = make_uint4(rb[0], rb[1], rb[2], rb[3]);
+}
+
+__global__ __launch_bounds__(64) void rope_append_vec_kernel(
+    const bf16_t* src, int src_stride, bf16_t* q_out, int q_stride, int n_tokens, int n_heads,
+    int n_kv, int head_dim, const int32_t* __restrict__ positions, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, int rotary_dim, int max_positions, bf16_t* __restrict__ k_cache,
+    bf16_t* __restrict__ v_cache, const int32_t* __restrict__ slots, int page_size) {
+  const int n0 = blockIdx.x * ROPE_TOK, h = blockIdx.y;
+  const int n_here = min(ROPE_TOK, n_tokens - n0);
+  const int half = rotary_dim / 2;
+  if (h >= n_heads + n_kv) {
+    // value head g of these tokens, transposed into the pages
+    const int g = h - n_heads - n_kv;
+    const int vbase = (n_heads + n_kv + g) * head_dim;
+    const int slot0 = slots[n0];
+    bool together = n_here == ROPE_TOK && slot0 % ROPE_TOK == 0;
+    for (int t = 1; t < n_here; ++t) together = together && slots[n0 + t] == slot0 + t;
+    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+      bf16_t v[ROPE_TOK];
+#pragma unroll
+      for (int t = 0; t < ROPE_TOK; ++t)
+        v[t] = src[static_cast<size_t>(n0 + min(t, n_here - 1)) * src_stride + vbase + d];
+      if (together) {
+        const size_t page = static_cast<size_t>(slot0 / page_size);
+        bf16_t* vdst = v_cache + ((page * n_kv + g) * head_dim + d) * page_size + slot0 % page_size;
+        uint4 w;
+        w.x = v[0] | (static_cast<uint32_t>(v[1]) << 16);
+        w.y = v[2] | (static_cast<uint32_t>(v[3]) << 16);
+        w.z = v[4] | (static_cast<uint32_t>(v[5]) << 16);
+        w.w = v[6] | (static_cast<uint32_t>(v[7]) << 16);
+        *reinterpret_cast<uint4*>(vdst) = w;
+      } else {
+        for (int t = 0; t < n_here; ++t) {
+          const int slot = slots[n0 + t];
+          const size_t page = static_cast<size_t>(slot / page_size);
+          v_cache[((page * n_kv + g) * head_dim + d) * page_size + slot % page_size] = v[t];
+        }
+      }
+    }
+    return;
+  }
+  const bool is_q = h < n_heads;
+  const int pieces = half / 8;                      // rotated pairs of 16-byte pieces per head
+  const int tail = (head_dim - rotary_dim) / 8;     // pieces beyond the rotated part
+  const int per_tok = pieces + tail;
+  for (int item = threadIdx.x; item < n_here * per_tok; item += blockDim.x) {
+    const int t = item / per_tok, pc = item % per_tok;
+    const int n = n0 + t;
+    const bf16_t* row = src + static_cast<size_t>(n) * src_stride + static_cast<size_t>(h) * head_dim;
+    bf16_t* dst;
+    if (is_q) {
+      dst = q_out + static_cast<size_t>(n) * q_stride + static_cast<size_t>(h) * head_dim;
+    } else {
+      const int slot = slots[n];
+      const size_t page = static_cast<size_t>(slot / page_size);
+      dst = k_cache + ((page * n_kv + (h - n_heads)) * page_size + slot % page_size) * head_dim;
+    }
+    if (pc < pieces) {
+      int pos = positions[n];
+      pos = pos < 0 ? 0 : (pos >= max_positions ? max_positions - 1 : pos);
+      const float* cs = cos_t + static_cast<size_t>(pos) * half + 8 * pc;
+      const float* sn = sin_t + static_cast<size_t>(pos) * half + 8 * pc;
+      const uint4 a = *reinterpret_cast<const uint4*>(row + 8 * pc);
+      const uint4 b = *reinterpret_cast<const uint4*>(row + half + 8 * pc);
+      float c[8], s_[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        c[j] = cs[j];
+        s_[j] = sn[j];
+      }
+      uint4 oa, ob;
+      rope_rotate8(a, b, c, s_, oa, ob);
+      *reinterpret_cast<uint4*>(dst + 8 * pc) = oa;
+      *reinterpret_cast<uint4*>(dst + half + 8 * pc) = ob;
+    } else {
+      const int d = rotary_dim + 8 * (pc - pieces);
+      *reinterpret_cast<uint4*>(dst + d) = *reinterpret_cast<const uint4*>(row + d);
+    }
+  }
 }
 
 // src_dtype/n_splits describe `src`; act_dtype is the dtype of q_out and of the cache.
@@ -367,6 +477,18 @@ extern "C" int yk_rope_append(const void* src, int src_dtype, int n_splits, int 
   YK_REQUIRE(n_splits >= 1 && (n_splits == 1 || src_dtype == YK_F32), "rope_append: unreduced slices must be float32");
   YK_REQUIRE(n_heads + n_kv <= 65535, "rope_append: too many heads for one launch");
   if (n_tokens == 0 || n_heads + n_kv == 0) return 0;
+  const auto aligned16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  if (src_dtype == YK_BF16 && act_dtype == YK_BF16 && n_splits == 1 && !interleaved && n_tokens >= 4 * ROPE_TOK &&
+      rotary_dim % 16 == 0 && head_dim % 8 == 0 && src_stride % 8 == 0 && q_stride % 8 == 0 && page_size % ROPE_TOK == 0 &&
+      aligned16(src) && aligned16(q_out) && (n_kv == 0 || (aligned16(k_cache) && aligned16(v_cache))) &&
+      (rotary_dim == 0 || (aligned16(cos_t) && aligned16(sin_t))) && n_heads + 2 * n_kv <= 65535) {
+    dim3 vgrid((n_tokens + ROPE_TOK - 1) / ROPE_TOK, n_heads + 2 * n_kv);
+    rope_append_vec_kernel<<<vgrid, 64, 0, stream>>>(
+        static_cast<const bf16_t*>(src), src_stride, static_cast<bf16_t*>(q_out), q_stride, n_tokens, n_heads, n_kv,
+        head_dim, positions, cos_t, sin_t, rotary_dim, max_positions, static_cast<bf16_t*>(k_cache),
+        static_cast<bf16_t*>(v_cache), slots, page_size);
+    return yk_check_launch("rope_append_vec");
+  }
   dim3 grid(n_tokens, n_heads + n_kv), block(head_dim <= 128 ? 64 : 128);
   const size_t stride = static_cast<size_t>(n_tokens) * src_stride;
 #define YK_CASE(SD, TS, AD, T)                                                                          \
