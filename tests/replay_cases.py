@@ -157,22 +157,22 @@ def plain_logits(cfg, weights, reqs, bf16: bool) -> Dict[str, torch.Tensor]:
     return {rid: P.forward(cfg, weights, toks) for rid, toks in reqs.items()}
 
 
-def tolerance(want: torch.Tensor, bf16: bool) -> float:
+def tolerance(want: torch.Tensor, bf16: bool, f32_tol: float = 2e-5) -> float:
     """float32: the plain implementation's own rounding noise at these sizes, with a
     margin (the engine sums in another order).  bfloat16: activations carry 8 bits; a
     logit gathers a few roundings per layer, so a few times 2^-8 of the logits' scale."""
     if not bf16:
-        return 2e-5
+        return f32_tol
     return 4 * 2.0**-8 * float(want.abs().max())
 
 
-def assert_matches(got: Dict[str, torch.Tensor], want: Dict[str, torch.Tensor], bf16: bool, what: str) -> None:
+def assert_matches(got: Dict[str, torch.Tensor], want: Dict[str, torch.Tensor], bf16: bool, what: str, f32_tol: float = 2e-5) -> None:
     for rid, w in want.items():
         g = got[rid]
         assert g.shape == w.shape, f"{what}: request {rid} has {tuple(g.shape)} logits, expected {tuple(w.shape)}"
         assert torch.isfinite(g).all(), f"{what}: request {rid} has non-finite logits"
         err = (g - w).abs().max(dim=1).values
-        tol = tolerance(w, bf16)
+        tol = tolerance(w, bf16, f32_tol)
         if (err > tol).any():
             first = int(torch.nonzero(err > tol)[0])
             raise AssertionError(

@@ -76,6 +76,47 @@ def test_replay_modes(backend, name, mode):
         assert reused, "the trace was meant to reuse pages"
 
 
+# The widths of the Llama-3-8B shape (hidden size, heads and groups, head size, feed-forward
+# width, vocabulary, rotary base) with two layers: the kernels meet inside the engine the
+# sizes they are measured at, a vocabulary that is no power of two and products split over K.
+FULL_WIDTH = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 4096, "num_hidden_layers": 2,
+    "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 14336,
+    "vocab_size": 128256, "rms_norm_eps": 1e-5, "rope_theta": 500000.0, "rope_scaling": None,
+    "max_position_embeddings": 8192, "tie_word_embeddings": False,
+}
+_full_width = {}
+
+
+def full_width_setup(bf16):
+    if "weights" not in _full_width:
+        _full_width["weights"] = P.random_weights(FULL_WIDTH, seed=8)
+        _full_width["reqs"] = C.make_requests(FULL_WIDTH, [100, 37, 70, 5, 66], seed=11)
+    if bf16 not in _full_width:
+        _full_width[bf16] = C.plain_logits(FULL_WIDTH, _full_width["weights"], _full_width["reqs"], bf16)
+    return _full_width["weights"], _full_width["reqs"], _full_width[bf16]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_full_width_replay(dtype):
+    """Every way of cutting the work at the widths of the 8B shape.  The float32 bound is
+    1e-4 absolute: sums over 4,096 and 14,336 terms in another order than the plain
+    implementation's carry more rounding than the tiny models' (whose bound stays 2e-5)."""
+    bf16 = dtype == "bfloat16"
+    weights, reqs, want = full_width_setup(bf16)
+    runner = None
+    for mode, make in (("whole", C.trace_whole), ("tail", C.trace_tail), ("portions", C.trace_portions), ("mixed", C.trace_mixed)):
+        steps = make(reqs)
+        n_pages = C.pages_needed(steps, reqs, 64)
+        del runner
+        runner = C.make_runner(FULL_WIDTH, weights, dtype, "cuda:0", ops_for("cuda:0"), 64, n_pages)
+        got, _ = C.run_trace(runner, steps)
+        C.assert_matches(got, want, bf16, f"full width/{mode}", f32_tol=1e-4)
+        runner.pages.audit()
+        assert runner.pages.live_requests() == 0
+
+
 @pytest.mark.parametrize("backend", BACKENDS)
 def test_readmission_reproduces(backend):
     """Release a request half way (as a preemption does) and replay it from the start:

@@ -144,31 +144,34 @@ def test_gemm_mfma_operand_order(ops):
 
 def test_split_sums_feed_their_consumers(ops):
     """A few-row product may stay as unreduced K slices; norm, rotary + append and the
-    gated activation add them up themselves and must agree with the reduced path."""
+    gated activation add them up themselves, round the sum as the product's output would
+    have been rounded, and so give the same bits as the reduced path."""
     from yalis_amd.ops.hip import SplitSum
 
     m, k = 5, 4096
     x = rnd((m, k), torch.bfloat16, 20, 0.5)
-    # norm
     w = rnd((256, k), torch.bfloat16, 21, 0.05)
     part = ops.linear(x, w, torch.bfloat16, partial_ok=True)
     assert isinstance(part, SplitSum) and part.n_splits > 1, "this shape was meant to split K"
+    assert part.out_dtype == torch.bfloat16
     full = part.tensor.sum(0)
     assert (full.cpu() - (x.double().cpu() @ w.double().cpu().T).float()).abs().max() < 1e-3
+    reduced = ops.linear(x, w, torch.bfloat16)  # the same slices, summed and rounded by the product
+    assert torch.equal(part.reduce(), reduced.float())
+    # norm
     res = rnd((m, 256), torch.float32, 22)
     nw = (1 + 0.1 * rnd((256,), torch.float32, 23)).to(torch.bfloat16)
     r1, r2 = res.clone(), res.clone()
     got = ops.add_rmsnorm(r1, part, nw, 1e-5, False, torch.bfloat16)
-    want = ops.add_rmsnorm(r2, full, nw, 1e-5, False, torch.bfloat16)
-    close(r1, r2, 2e-6, 2e-6)
-    close(got, want, 1e-2, 2**-7)
+    want = ops.add_rmsnorm(r2, reduced, nw, 1e-5, False, torch.bfloat16)
+    assert torch.equal(r1, r2) and torch.equal(got, want)
+    close(r1, res.cpu() + full.cpu(), 1e-2, 2**-7)
     rows = torch.tensor([4, 0], dtype=torch.int32, device=DEV)
-    # two float32 summation orders: a few units in the last place
-    close(ops.gather_add_rmsnorm(res, part, rows, nw, 1e-5, False, torch.float32),
-          ops.gather_add_rmsnorm(res, full, rows, nw, 1e-5, False, torch.float32), 2e-6, 2e-6)
+    assert torch.equal(ops.gather_add_rmsnorm(res, part, rows, nw, 1e-5, False, torch.float32),
+                       ops.gather_add_rmsnorm(res, reduced, rows, nw, 1e-5, False, torch.float32))
     # gated activation
-    close(ops.gated_act(part, "silu", torch.bfloat16), ops.gated_act(full.to(torch.bfloat16), "silu"), 1e-2, 2**-7)
-    close(ops.gated_act(part, "silu", torch.float32), R.gated_act(full.cpu(), "silu"), 1e-5, 1e-5)
+    assert torch.equal(ops.gated_act(part, "silu", torch.bfloat16), ops.gated_act(reduced, "silu"))
+    close(ops.gated_act(part, "silu", torch.float32), R.gated_act(reduced.float().cpu(), "silu"), 1e-5, 1e-5)
     # rotary + append: 2 query heads, 1 kv head of 64 -> 256 columns
     cos, sin = _tables(64, 100)
     positions = torch.tensor([3, 4, 50, 0, 99], dtype=torch.int32, device=DEV)
@@ -177,12 +180,21 @@ def test_split_sums_feed_their_consumers(ops):
     vc = torch.zeros((4, 1, 64, 16), dtype=torch.bfloat16, device=DEV)
     q = ops.rope_append(part, 2, 1, 64, positions, cos, sin, 64, False, kc, vc, slots, 16)
     assert q.shape == (m, 128) and q.dtype == torch.bfloat16
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    q2 = ops.rope_append(reduced.clone(), 2, 1, 64, positions, cos, sin, 64, False, kc2, vc2, slots, 16)
+    assert torch.equal(q, q2[:, :128]) and torch.equal(kc, kc2) and torch.equal(vc, vc2)
     kr, vr = torch.zeros((4, 1, 16, 64)), torch.zeros((4, 1, 64, 16))
     ref2 = full.clone().cpu()
     R.rope_append(ref2, 2, 1, 64, positions.cpu(), cos.cpu(), sin.cpu(), 64, False, kr, vr, slots.cpu(), 16)
     close(q, ref2[:, :128], 1e-2, 2**-7)
     close(kc, kr, 1e-2, 2**-7)
     close(vc, vr, 1e-2, 2**-7)
+    # slices of a product asked for in float32 are added without rounding
+    part32 = ops.linear(x, w, torch.float32, partial_ok=True)
+    assert isinstance(part32, SplitSum) and part32.out_dtype == torch.float32
+    r3 = res.clone()
+    ops.add_rmsnorm(r3, part32, nw, 1e-5, False, torch.bfloat16)
+    close(r3, res.cpu() + full.cpu(), 2e-6, 2e-6)
 
 
 def test_linear_dispatch(ops):

@@ -25,7 +25,7 @@ int yk_check_launch(const char* what) {
   return 0;
 }
 extern "C" const char* yk_last_error() { return yk_error_slot().c_str(); }
-extern "C" int yk_abi_version() { return 2; }
+extern "C" int yk_abi_version() { return 3; }
 
 // ------------------------------------------------------------------------- embedding
 // out[n, :] = float(table[ids[n], :])
@@ -119,6 +119,13 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float4 v) {
   *reinterpret_cast<uint2*>(p) = raw;
 }
 
+// The sum of a product's K slices stands for the product's output: with `round_sum` it is
+// rounded to bfloat16 as that output would have been, so that what follows does not depend
+// on whether the product came reduced (bfloat16) or as slices.
+__device__ __forceinline__ float as_output(float v, int round_sum) {
+  return round_sum ? to_f32<bf16_t>(from_f32<bf16_t>(v)) : v;
+}
+
 // ------------------------------------------------------------- residual add + RMS norm
 // For row r (source row rows[r] when rows is given):
 //   v = residual[src] + sum over s of delta[s][src]   (float32; delta may be absent;
@@ -128,7 +135,7 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float4 v) {
 // General form: any width, two passes over the row.
 template <typename TD, typename TW, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
-                                   int n_splits, size_t split_stride,
+                                   int n_splits, size_t split_stride, int round_sum,
                                    const int32_t* __restrict__ rows, const TW* __restrict__ weight,
                                    TO* __restrict__ out, int width, float eps, int unit_offset) {
   __shared__ float scratch[17];
@@ -140,7 +147,9 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
     float v = res[c];
     if (del) {
-      for (int s = 0; s < n_splits; ++s) v += to_f32<TD>(del[s * split_stride + c]);
+      float d = 0.f;
+      for (int s = 0; s < n_splits; ++s) d += to_f32<TD>(del[s * split_stride + c]);
+      v += as_output(d, round_sum);
       if (!rows) res[c] = v;
     }
     ss += v * v;
@@ -150,8 +159,11 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
   TO* o = out + static_cast<size_t>(r) * width;
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
     float v = res[c];
-    if (del && rows)  // not written back in the gathered form
-      for (int s = 0; s < n_splits; ++s) v += to_f32<TD>(del[s * split_stride + c]);
+    if (del && rows) {  // not written back in the gathered form
+      float d = 0.f;
+      for (int s = 0; s < n_splits; ++s) d += to_f32<TD>(del[s * split_stride + c]);
+      v += as_output(d, round_sum);
+    }
     float w = to_f32<TW>(weight[c]);
     if (unit_offset) w += 1.f;
     o[c] = from_f32<TO>(v * inv * w);
@@ -159,19 +171,20 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
 }
 
 // Fast form: width a multiple of 4 and at most 4 * NORM_IT * blockDim; the row stays in
-// registers, every load of a thread is issued before the first use.
-constexpr int NORM_IT = 8;
-template <typename TD, typename TW, typename TO>
+// registers, every load of a thread is issued before the first use.  NORM_IT (four-wide
+// pieces per thread) is chosen by the launcher as small as the width allows.
+constexpr int NORM_IT_MAX = 8;
+template <typename TD, typename TW, typename TO, int NORM_IT>
 __global__ __launch_bounds__(512) void add_rmsnorm_vec_kernel(
     float* __restrict__ residual, const TD* __restrict__ delta, int n_splits, size_t split_stride,
-    const int32_t* __restrict__ rows, const TW* __restrict__ weight, TO* __restrict__ out,
+    int round_sum, const int32_t* __restrict__ rows, const TW* __restrict__ weight, TO* __restrict__ out,
     int width, float eps, int unit_offset) {
   __shared__ float scratch[17];
   const int r = blockIdx.x;
   const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
   float* res = residual + src * width;
   const TD* del = delta ? delta + src * width : nullptr;
-  float4 v[NORM_IT], w[NORM_IT];
+  float4 v[NORM_IT], w[NORM_IT], ds[NORM_IT];
   float ss = 0.f;
 #pragma unroll
   for (int it = 0; it < NORM_IT; ++it) {
@@ -184,6 +197,8 @@ __global__ __launch_bounds__(512) void add_rmsnorm_vec_kernel(
   if (del) {
     // four slices at a time, all loads issued before the first sum; a slice index beyond
     // the last is clamped and its value dropped, so that the loads carry no condition
+#pragma unroll
+    for (int it = 0; it < NORM_IT; ++it) ds[it] = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int s0 = 0; s0 < n_splits; s0 += 4) {
 #pragma unroll
       for (int it = 0; it < NORM_IT; ++it) {
@@ -195,14 +210,21 @@ __global__ __launch_bounds__(512) void add_rmsnorm_vec_kernel(
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             if (s0 + j < n_splits) {
-              v[it].x += d[j].x;
-              v[it].y += d[j].y;
-              v[it].z += d[j].z;
-              v[it].w += d[j].w;
+              ds[it].x += d[j].x;
+              ds[it].y += d[j].y;
+              ds[it].z += d[j].z;
+              ds[it].w += d[j].w;
             }
           }
         }
       }
+    }
+#pragma unroll
+    for (int it = 0; it < NORM_IT; ++it) {
+      v[it].x += as_output(ds[it].x, round_sum);
+      v[it].y += as_output(ds[it].y, round_sum);
+      v[it].z += as_output(ds[it].z, round_sum);
+      v[it].w += as_output(ds[it].w, round_sum);
     }
   }
 #pragma unroll
@@ -233,30 +255,38 @@ __global__ __launch_bounds__(512) void add_rmsnorm_vec_kernel(
 
 template <typename TD, typename TW, typename TO>
 static int launch_add_rmsnorm(float* residual, const void* delta, int n_splits, size_t split_stride,
-                              const int32_t* rows, const void* weight, void* out, int n_rows,
+                              int round_sum, const int32_t* rows, const void* weight, void* out, int n_rows,
                               int width, float eps, int unit_offset, hipStream_t stream) {
   const bool aligned = width % 4 == 0 && reinterpret_cast<uintptr_t>(residual) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(delta) % 16 == 0 && reinterpret_cast<uintptr_t>(weight) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(out) % 16 == 0 && split_stride % 4 == 0;
-  if (aligned && width <= 4 * NORM_IT * 512) {
+  if (aligned && width <= 4 * NORM_IT_MAX * 512) {
     // two four-wide chunks per thread where the row allows, at most 512 threads
     int threads = ((width / 4 + 1) / 2 + 63) / 64 * 64;
     threads = std::max(64, std::min(threads, 512));
-    add_rmsnorm_vec_kernel<TD, TW, TO><<<n_rows, threads, 0, stream>>>(
-        residual, static_cast<const TD*>(delta), n_splits, split_stride, rows,
-        static_cast<const TW*>(weight), static_cast<TO*>(out), width, eps, unit_offset);
+    const int pieces = (width / 4 + threads - 1) / threads;
+#define YK_NORM(IT)                                                                           \
+    add_rmsnorm_vec_kernel<TD, TW, TO, IT><<<n_rows, threads, 0, stream>>>(                   \
+        residual, static_cast<const TD*>(delta), n_splits, split_stride, round_sum, rows,     \
+        static_cast<const TW*>(weight), static_cast<TO*>(out), width, eps, unit_offset)
+    if (pieces <= 1) YK_NORM(1);
+    else if (pieces <= 2) YK_NORM(2);
+    else if (pieces <= 4) YK_NORM(4);
+    else YK_NORM(8);
+#undef YK_NORM
   } else {
     add_rmsnorm_kernel<TD, TW, TO><<<n_rows, width >= 2048 ? 512 : 256, 0, stream>>>(
-        residual, static_cast<const TD*>(delta), n_splits, split_stride, rows,
+        residual, static_cast<const TD*>(delta), n_splits, split_stride, round_sum, rows,
         static_cast<const TW*>(weight), static_cast<TO*>(out), width, eps, unit_offset);
   }
   return yk_check_launch("add_rmsnorm");
 }
 
 // delta may be null (then delta_dtype is ignored); rows may be null.  n_splits > 1 needs
-// float32 delta laid out [n_splits][rows of the residual][width].
+// float32 delta laid out [n_splits][rows of the residual][width]; round_sum: the slices' sum
+// is rounded to bfloat16 before it is added.
 extern "C" int yk_add_rmsnorm(float* residual, const void* delta, int delta_dtype, int n_splits,
-                              const int32_t* rows, const void* weight, int weight_dtype, void* out,
+                              int round_sum, const int32_t* rows, const void* weight, int weight_dtype, void* out,
                               int out_dtype, int n_rows, int n_residual_rows, int width, float eps,
                               int unit_offset, hipStream_t stream) {
   YK_REQUIRE(n_rows >= 0 && width > 0 && n_residual_rows >= 0, "add_rmsnorm: bad sizes");
@@ -271,7 +301,7 @@ extern "C" int yk_add_rmsnorm(float* residual, const void* delta, int delta_dtyp
   const size_t stride = static_cast<size_t>(n_residual_rows) * width;
 #define YK_CASE(DD, TD, WD, TW, OD, TO)                                  \
   if (delta_dtype == DD && weight_dtype == WD && out_dtype == OD)        \
-    return launch_add_rmsnorm<TD, TW, TO>(residual, delta, n_splits, stride, rows, weight, out, n_rows, width, eps, unit_offset, stream);
+    return launch_add_rmsnorm<TD, TW, TO>(residual, delta, n_splits, stride, round_sum, rows, weight, out, n_rows, width, eps, unit_offset, stream);
   YK_CASE(YK_F32, float, YK_F32, float, YK_F32, float)
   YK_CASE(YK_F32, float, YK_F32, float, YK_BF16, bf16_t)
   YK_CASE(YK_F32, float, YK_BF16, bf16_t, YK_F32, float)
@@ -301,7 +331,7 @@ __device__ __forceinline__ float rot_first(float a, float b, float c, float s) {
 __device__ __forceinline__ float rot_second(float a, float b, float c, float s) { return fmaf(b, c, __fmul_rn(a, s)); }
 
 template <typename TS, typename T>
-__global__ void rope_append_kernel(const TS* src, int n_splits, size_t split_stride,
+__global__ void rope_append_kernel(const TS* src, int n_splits, size_t split_stride, int round_sum,
                                    int src_stride, T* q_out, int q_stride, int n_heads,
                                    int n_kv, int head_dim, const int32_t* __restrict__ positions,
                                    const float* __restrict__ cos_t, const float* __restrict__ sin_t,
@@ -325,7 +355,7 @@ __global__ void rope_append_kernel(const TS* src, int n_splits, size_t split_str
       for (int j = 0; j < 4; ++j)
         if (s0 + j < n_splits) a += d[j];
     }
-    return a;
+    return as_output(a, round_sum);
   };
   const bool is_q = h < n_heads;
   T* dst;
@@ -461,7 +491,7 @@ __global__ __launch_bounds__(64) void rope_append_vec_kernel(
 }
 
 // src_dtype/n_splits describe `src`; act_dtype is the dtype of q_out and of the cache.
-extern "C" int yk_rope_append(const void* src, int src_dtype, int n_splits, int src_stride,
+extern "C" int yk_rope_append(const void* src, int src_dtype, int n_splits, int round_sum, int src_stride,
                               void* q_out, int act_dtype, int q_stride, int n_tokens, int n_heads,
                               int n_kv, int head_dim, const int32_t* positions, const float* cos_t,
                               const float* sin_t, int rotary_dim, int interleaved,
@@ -494,7 +524,7 @@ extern "C" int yk_rope_append(const void* src, int src_dtype, int n_splits, int 
 #define YK_CASE(SD, TS, AD, T)                                                                          \
   if (src_dtype == SD && act_dtype == AD) {                                                             \
     rope_append_kernel<TS, T><<<grid, block, 0, stream>>>(                                              \
-        static_cast<const TS*>(src), n_splits, stride, src_stride, static_cast<T*>(q_out), q_stride,    \
+        static_cast<const TS*>(src), n_splits, stride, round_sum, src_stride, static_cast<T*>(q_out), q_stride, \
         n_heads, n_kv, head_dim, positions, cos_t, sin_t, rotary_dim, interleaved, max_positions,       \
         static_cast<T*>(k_cache), static_cast<T*>(v_cache), slots, page_size);                          \
     return yk_check_launch("rope_append");                                                              \
@@ -517,7 +547,7 @@ __device__ __forceinline__ float act_gelu_tanh(float z) {
 __device__ __forceinline__ float act_apply(float z, int act) { return act == 0 ? act_silu(z) : act_gelu_tanh(z); }
 
 template <typename TS, typename TO>
-__global__ void gated_act_kernel(const TS* __restrict__ gu, int n_splits, size_t split_stride,
+__global__ void gated_act_kernel(const TS* __restrict__ gu, int n_splits, size_t split_stride, int round_sum,
                                  TO* __restrict__ out, int inter, size_t total, int act) {
   for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total;
        i += static_cast<size_t>(gridDim.x) * blockDim.x) {
@@ -527,13 +557,15 @@ __global__ void gated_act_kernel(const TS* __restrict__ gu, int n_splits, size_t
       g += to_f32<TS>(gu[s * split_stride + n * 2 * inter + j]);
       u += to_f32<TS>(gu[s * split_stride + n * 2 * inter + inter + j]);
     }
+    g = as_output(g, round_sum);
+    u = as_output(u, round_sum);
     out[i] = from_f32<TO>(act_apply(g, act) * u);
   }
 }
 
 // four outputs per thread, no loop (inter a multiple of 4)
 template <typename TS, typename TO>
-__global__ void gated_act_vec_kernel(const TS* __restrict__ gu, int n_splits, size_t split_stride,
+__global__ void gated_act_vec_kernel(const TS* __restrict__ gu, int n_splits, size_t split_stride, int round_sum,
                                      TO* __restrict__ out, int inter, size_t total_vec, int act) {
   const size_t v = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
   if (v >= total_vec) return;
@@ -554,15 +586,15 @@ __global__ void gated_act_vec_kernel(const TS* __restrict__ gu, int n_splits, si
     }
   }
   float4 y;
-  y.x = act_apply(g.x, act) * u.x;
-  y.y = act_apply(g.y, act) * u.y;
-  y.z = act_apply(g.z, act) * u.z;
-  y.w = act_apply(g.w, act) * u.w;
+  y.x = act_apply(as_output(g.x, round_sum), act) * as_output(u.x, round_sum);
+  y.y = act_apply(as_output(g.y, round_sum), act) * as_output(u.y, round_sum);
+  y.z = act_apply(as_output(g.z, round_sum), act) * as_output(u.z, round_sum);
+  y.w = act_apply(as_output(g.w, round_sum), act) * as_output(u.w, round_sum);
   store4<TO>(out + n * inter + j, y);
 }
 
 template <typename TS, typename TO>
-static int launch_gated_act(const void* gu, int n_splits, void* out, int n_rows, int inter, int act,
+static int launch_gated_act(const void* gu, int n_splits, int round_sum, void* out, int n_rows, int inter, int act,
                             hipStream_t stream) {
   const size_t stride = static_cast<size_t>(n_rows) * 2 * inter;
   const bool aligned = inter % 4 == 0 && reinterpret_cast<uintptr_t>(gu) % 16 == 0 &&
@@ -571,24 +603,24 @@ static int launch_gated_act(const void* gu, int n_splits, void* out, int n_rows,
     const size_t total_vec = static_cast<size_t>(n_rows) * (inter / 4);
     YK_REQUIRE((total_vec + 255) / 256 < (1ull << 31), "gated_act: too large for one launch");
     gated_act_vec_kernel<TS, TO><<<static_cast<unsigned>((total_vec + 255) / 256), 256, 0, stream>>>(
-        static_cast<const TS*>(gu), n_splits, stride, static_cast<TO*>(out), inter, total_vec, act);
+        static_cast<const TS*>(gu), n_splits, stride, round_sum, static_cast<TO*>(out), inter, total_vec, act);
   } else {
     const size_t total = static_cast<size_t>(n_rows) * inter;
     const int grid = static_cast<int>(std::min<size_t>((total + 255) / 256, 65535));
-    gated_act_kernel<TS, TO><<<grid, 256, 0, stream>>>(static_cast<const TS*>(gu), n_splits, stride,
+    gated_act_kernel<TS, TO><<<grid, 256, 0, stream>>>(static_cast<const TS*>(gu), n_splits, stride, round_sum,
                                                         static_cast<TO*>(out), inter, total, act);
   }
   return yk_check_launch("gated_act");
 }
 
-extern "C" int yk_gated_act(const void* gu, int src_dtype, int n_splits, void* out, int out_dtype,
+extern "C" int yk_gated_act(const void* gu, int src_dtype, int n_splits, int round_sum, void* out, int out_dtype,
                             int n_rows, int inter, int act, hipStream_t stream) {
   YK_REQUIRE(n_rows >= 0 && inter > 0, "gated_act: bad sizes");
   YK_REQUIRE(act == 0 || act == 1, "gated_act: unknown activation");
   YK_REQUIRE(n_splits >= 1 && (n_splits == 1 || src_dtype == YK_F32), "gated_act: unreduced slices must be float32");
   if (n_rows == 0) return 0;
-  if (src_dtype == YK_F32 && out_dtype == YK_F32) return launch_gated_act<float, float>(gu, n_splits, out, n_rows, inter, act, stream);
-  if (src_dtype == YK_F32 && out_dtype == YK_BF16) return launch_gated_act<float, bf16_t>(gu, n_splits, out, n_rows, inter, act, stream);
-  if (src_dtype == YK_BF16 && out_dtype == YK_BF16) return launch_gated_act<bf16_t, bf16_t>(gu, n_splits, out, n_rows, inter, act, stream);
+  if (src_dtype == YK_F32 && out_dtype == YK_F32) return launch_gated_act<float, float>(gu, n_splits, round_sum, out, n_rows, inter, act, stream);
+  if (src_dtype == YK_F32 && out_dtype == YK_BF16) return launch_gated_act<float, bf16_t>(gu, n_splits, round_sum, out, n_rows, inter, act, stream);
+  if (src_dtype == YK_BF16 && out_dtype == YK_BF16) return launch_gated_act<bf16_t, bf16_t>(gu, n_splits, round_sum, out, n_rows, inter, act, stream);
   return yk_fail("gated_act: unsupported dtype combination");
 }

@@ -44,15 +44,15 @@ _SIGNATURES = {
     "yk_abi_version": ([], _c_int),
     "yk_embed": ([_vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_add_rmsnorm": (
-        [_vp, _vp, _c_int, _c_int, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp],
+        [_vp, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp],
         _c_int,
     ),
     "yk_rope_append": (
-        [_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp,
+        [_vp, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp,
          _c_int, _c_int, _c_int, _vp, _vp, _vp, _c_int, _vp],
         _c_int,
     ),
-    "yk_gated_act": ([_vp, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _vp], _c_int),
+    "yk_gated_act": ([_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_gemm_fma": (
         [_vp, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
         _c_int,
@@ -94,19 +94,26 @@ class SplitSum:
     """The unreduced K slices of a product: float32 [slices, rows, columns] whose sum over
     the first axis is the result.  The kernels that consume a projection (norm, rotary +
     append, gated activation) add the slices themselves, which saves a pass over memory
-    and a rounding.  It lives in the library's workspace: consume it before the next
-    product is launched."""
+    of its own.  ``out_dtype`` is the dtype the product was asked for: the consumers round
+    the sum to it, so that a value does not depend on whether its product came reduced or
+    as slices.  It lives in the library's workspace: consume it before the next product
+    is launched."""
 
-    def __init__(self, tensor: torch.Tensor):
+    def __init__(self, tensor: torch.Tensor, out_dtype: torch.dtype = torch.float32):
         self.tensor = tensor
         self.shape = tuple(tensor.shape[1:])
         self.n_splits = tensor.shape[0]
+        self.out_dtype = out_dtype
         self.dtype = torch.float32
         self.device = tensor.device
 
+    @property
+    def round_sum(self) -> int:
+        return int(self.out_dtype == torch.bfloat16)
+
     def reduce(self) -> torch.Tensor:
         """The product itself, float32 (for code that does not add the slices itself)."""
-        return self.tensor.sum(0)
+        return self.tensor.sum(0).to(self.out_dtype).float()
 
     def float(self) -> torch.Tensor:
         return self.reduce()
@@ -123,7 +130,7 @@ class HipOps:
             fn = getattr(self.lib, name)
             fn.argtypes = args
             fn.restype = res
-        if self.lib.yk_abi_version() != 2:
+        if self.lib.yk_abi_version() != 3:
             raise KernelError("kernel library and bindings disagree; rebuild (python -c 'import __graft_entry__ as g; g.build()')")
         self._workspace: Optional[torch.Tensor] = None  # attention splits, argmax parts
         self._gemm_workspace: Optional[torch.Tensor] = None  # K slices of products
@@ -199,9 +206,9 @@ class HipOps:
         width = residual.shape[1]
         if weight.numel() != width:
             raise KernelError(f"norm weight has {weight.numel()} elements, rows have {width}")
-        n_splits = 1
+        n_splits, round_sum = 1, 0
         if isinstance(delta, SplitSum):
-            n_splits, delta = delta.n_splits, delta.tensor
+            n_splits, round_sum, delta = delta.n_splits, delta.round_sum, delta.tensor
             if tuple(delta.shape[1:]) != tuple(residual.shape):
                 raise KernelError(f"delta {tuple(delta.shape[1:])} does not match the residual {tuple(residual.shape)}")
         elif delta is not None and (tuple(delta.shape) != tuple(residual.shape) or not delta.is_contiguous()):
@@ -209,7 +216,7 @@ class HipOps:
         out = torch.empty((n_out, width), dtype=out_dtype, device=residual.device)
         self._check(
             self.lib.yk_add_rmsnorm(
-                residual.data_ptr(), _ptr(delta), 0 if delta is None else _code(delta.dtype), n_splits,
+                residual.data_ptr(), _ptr(delta), 0 if delta is None else _code(delta.dtype), n_splits, round_sum,
                 _ptr(rows), weight.data_ptr(), _code(weight.dtype), out.data_ptr(), _code(out_dtype),
                 n_out, residual.shape[0], width, float(eps), int(bool(unit_offset)), self._stream(),
             )
@@ -268,7 +275,7 @@ class HipOps:
         if rc < 0:
             raise KernelError(self.lib.yk_last_error().decode())
         if keep:
-            return SplitSum(ws[: splits * m * n].view(splits, m, n))
+            return SplitSum(ws[: splits * m * n].view(splits, m, n), out_dtype)
         return y
 
     # ------------------------------------------------- rotary + append to the cache
@@ -277,10 +284,10 @@ class HipOps:
         """Rotates the query heads, appends rotated keys and values to the pages; returns
         the tensor whose rows start with the rotated queries (``qkv`` itself, rotated in
         place, or a new [N, n_heads * head_dim] tensor when ``qkv`` is a SplitSum)."""
-        n_splits = 1
+        n_splits, round_sum = 1, 0
         src = qkv
         if isinstance(qkv, SplitSum):
-            n_splits, src = qkv.n_splits, qkv.tensor
+            n_splits, round_sum, src = qkv.n_splits, qkv.round_sum, qkv.tensor
             n, cols = qkv.shape
             act = k_cache.dtype if n_kv else torch.bfloat16
             q_out = torch.empty((n, n_heads * head_dim), dtype=act, device=src.device)
@@ -306,7 +313,7 @@ class HipOps:
                 raise KernelError(f"cache pages have shapes {tuple(k_cache.shape)}, {tuple(v_cache.shape)}")
         self._check(
             self.lib.yk_rope_append(
-                src.data_ptr(), _code(src.dtype), n_splits, src_stride, q_out.data_ptr(), _code(q_out.dtype),
+                src.data_ptr(), _code(src.dtype), n_splits, round_sum, src_stride, q_out.data_ptr(), _code(q_out.dtype),
                 q_out.stride(0), n, n_heads, n_kv, head_dim,
                 positions.data_ptr(), _ptr(cos) if rotary_dim else None, _ptr(sin) if rotary_dim else None,
                 rotary_dim, int(bool(interleaved)), max_pos,
@@ -385,10 +392,10 @@ class HipOps:
 
     # ----------------------------------------------------------------- activation
     def gated_act(self, gu, activation: str, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-        n_splits = 1
+        n_splits, round_sum = 1, 0
         src = gu
         if isinstance(gu, SplitSum):
-            n_splits, src = gu.n_splits, gu.tensor
+            n_splits, round_sum, src = gu.n_splits, gu.round_sum, gu.tensor
             rows, cols = gu.shape
             out_dtype = out_dtype or torch.bfloat16
         else:
@@ -405,7 +412,7 @@ class HipOps:
         inter = cols // 2
         out = torch.empty((rows, inter), dtype=out_dtype, device=src.device)
         self._check(
-            self.lib.yk_gated_act(src.data_ptr(), _code(src.dtype), n_splits, out.data_ptr(), _code(out_dtype),
+            self.lib.yk_gated_act(src.data_ptr(), _code(src.dtype), n_splits, round_sum, out.data_ptr(), _code(out_dtype),
                                   rows, inter, act, self._stream())
         )
         return out
