@@ -32,6 +32,14 @@ LLAMA3_8B = {
     "max_position_embeddings": 8192,
     "tie_word_embeddings": False,
 }
+_LLAMA3_SCALING = {"rope_type": "llama3", "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                   "original_max_position_embeddings": 8192}
+# further shapes (not the default): --shape 3b / 70b
+LLAMA32_3B = dict(LLAMA3_8B, hidden_size=3072, num_hidden_layers=28, num_attention_heads=24, intermediate_size=8192,
+                  rope_scaling=dict(_LLAMA3_SCALING, factor=32.0), tie_word_embeddings=True)
+LLAMA31_70B = dict(LLAMA3_8B, hidden_size=8192, num_hidden_layers=80, num_attention_heads=64, intermediate_size=28672,
+                   rope_scaling=dict(_LLAMA3_SCALING, factor=8.0))
+SHAPES = {"8b": ("Llama-3-8B", LLAMA3_8B), "3b": ("Llama-3.2-3B", LLAMA32_3B), "70b": ("Llama-3.1-70B", LLAMA31_70B)}
 
 
 def main() -> int:
@@ -45,6 +53,7 @@ def main() -> int:
     ap.add_argument("--prefill-len", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--only-prefill", action="store_true", help="measure the prefill only (for profiling)")
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="8b", help="layer sizes (default: the 8B shape of the headline)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
@@ -56,7 +65,8 @@ def main() -> int:
     from yalis_amd.engine.factory import random_runner
     from yalis_amd.engine.step import StepEntry
 
-    cfg = dict(LLAMA3_8B)
+    shape_name, shape_cfg = SHAPES[args.shape]
+    cfg = dict(shape_cfg)
     full_layers = cfg["num_hidden_layers"]
     if args.layers is not None:
         cfg["num_hidden_layers"] = args.layers
@@ -113,6 +123,8 @@ def main() -> int:
 
     c, h, g, d, inter = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["intermediate_size"]
     layer_params = c * (h + 2 * g) * d + h * d * c + 3 * c * inter
+    # every weight a decode step reads once: the layers, the final norm, the output head (the
+    # embedding table itself when tied; of a separate table only a row per token is read)
     weight_bytes = 2 * (layers * (layer_params + 2 * c) + c + vocab * c)
 
     def step_bytes(batch, mean_ctx_tokens):
@@ -138,7 +150,7 @@ def main() -> int:
     achieved = step_bytes(args.batch, mean_ctx) / (dt / args.steps) / 1e9
 
     result = {
-        "metric": "decode tok/s (Llama-3-8B shape, batch 8, 1,024-token prompts)",
+        "metric": f"decode tok/s ({shape_name} shape, batch {args.batch}, {args.prompt_len:,}-token prompts)",
         "value": round(value, 2),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -151,7 +163,7 @@ def main() -> int:
         "dtype": "bf16",
         "data": "synthetic: random N(0,0.02) bf16 weights, seeded uniform-random token ids",
         "config": {
-            "model": "Llama-3-8B shape",
+            "model": f"{shape_name} shape",
             "layers": layers,
             "layers_of_full_model": full_layers,
             "hidden_size": c,

@@ -191,3 +191,40 @@ def test_one_error_lists_everything_wrong(tmp_path):
     msg = str(err)
     for piece in ("missing tensors (2)", "unexpected tensors (1)", "model.norm.weight has (65,), the model needs (64,)", "wrong type"):
         assert piece in msg
+
+
+def test_tensors_are_made_when_a_part_asks(tmp_path):
+    """The loader hands the model a source that reads a tensor when a part asks for it: each
+    tensor is read once, a tied table is read once and shared by the embedding and the head,
+    nothing is kept afterwards, and the folder is still checked as a whole first."""
+    from kernel_refs import RefOps
+    from yalis_amd.engine.factory import build_model, load_runner
+    from yalis_amd.weights import loader
+
+    folder = write_random_model(str(tmp_path / "m"), TINY_B, seed=5)
+    eng = EngineConfig(page_size=16, num_pages=4, max_num_seqs=2, max_model_len=64, dtype="float32", device="cpu")
+    model = build_model(TINY_B, eng, ops=RefOps())
+    uses = model.tensor_uses()
+    assert uses["model.embed_tokens.weight"] == 2 and uses["model.norm.weight"] == 1
+    reads = []
+    real = loader.read_tensor
+    loader.read_tensor = lambda e: (reads.append(e.name), real(e))[1]
+    try:
+        src = loader.open_tensors(folder, model.tensor_specs(), uses, "float32", "cpu")
+        model.load(src)
+    finally:
+        loader.read_tensor = real
+    assert sorted(reads) == sorted(model.tensor_specs()), "every tensor is read exactly once"
+    assert not src._kept, "nothing is held once every part has its tensors"
+    assert model.head.weight.data_ptr() == model.embedding.table.data_ptr(), "the tied table is shared"
+    # the same through the factory, and the one error still comes before anything is read
+    runner = load_runner(folder, eng, ops=RefOps())
+    assert runner.model.head.weight.data_ptr() == runner.model.embedding.table.data_ptr()
+    t = {n: read_tensor(e) for n, e in index_folder(folder).items()}
+    del t["model.norm.weight"]
+    bad = str(tmp_path / "bad")
+    os.makedirs(bad)
+    json.dump(TINY_B, open(os.path.join(bad, "config.json"), "w"))
+    write_dict(os.path.join(bad, "model.safetensors"), t)
+    with pytest.raises(WeightsError, match="model.norm.weight"):
+        load_runner(bad, eng, ops=RefOps())

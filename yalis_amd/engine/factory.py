@@ -16,8 +16,8 @@ from ..config.registry import architecture_of
 from ..config.runtime import EngineConfig
 from ..models.decoder import DecoderModel
 from ..parts.base import Runtime
-from ..weights.loader import TensorSpec, load_tensors
-from ..weights.random_init import random_tensors
+from ..weights.loader import TensorSource, TensorSpec, open_tensors
+from ..weights.random_init import random_tensor
 from .step import ModelRunner
 
 
@@ -77,8 +77,7 @@ def build_model(
 def load_runner(model_dir: str, engine: EngineConfig, ops=None, progress=None) -> ModelRunner:
     """A runner over the checkpoint in ``model_dir``."""
     model = build_model(read_config_json(model_dir), engine, ops)
-    tensors = load_tensors(model_dir, model.tensor_specs(), engine.dtype, engine.device, progress)
-    model.load(tensors)
+    model.load(open_tensors(model_dir, model.tensor_specs(), model.tensor_uses(), engine.dtype, engine.device, progress))
     return ModelRunner(model, engine)
 
 
@@ -88,8 +87,9 @@ def random_runner(config_dict: dict, engine: EngineConfig, seed: int, ops=None, 
     model = build_model(config_dict, engine, ops)
     wdtype = torch.float32 if engine.dtype == "float32" else torch.bfloat16
     gen_device = engine.device if on_device else "cpu"
-    tensors = {}
-    for name, t in random_tensors(model.tensor_specs(), seed, wdtype, gen_device):
-        tensors[name] = t.to(engine.device)
-    model.load(tensors)
+    specs = model.tensor_specs()
+    model.load(TensorSource(
+        model.tensor_uses(),
+        lambda name: random_tensor(name, specs[name], seed, wdtype, gen_device).to(engine.device),
+    ))
     return ModelRunner(model, engine)

@@ -8,7 +8,7 @@ on the wanted rows, the head (the order of yalis/external/model.py:122-197).
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Callable, Dict, List, Optional, Tuple
+from typing import Callable, Dict, List, Mapping, Optional, Tuple
 
 import torch
 
@@ -126,7 +126,17 @@ class DecoderModel:
                 out.setdefault(name, spec)
         return out
 
-    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+    def tensor_uses(self) -> Dict[str, int]:
+        """How many parts ask for each tensor (a tied table is asked for twice)."""
+        out: Dict[str, int] = {}
+        for p in self.all_parts():
+            for name in p.tensor_specs():
+                out[name] = out.get(name, 0) + 1
+        return out
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        """Every part takes its tensors from ``tensors``: a dict, or a source that makes
+        each tensor when it is asked for (each part asks once for each of its names)."""
         for p in self.all_parts():
             p.load(tensors)
 

@@ -14,7 +14,7 @@ tensor is widened to float32 (exact).
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Callable, Dict, Iterable, Optional, Tuple
+from typing import Callable, Dict, Iterable, Mapping, Optional, Tuple
 
 import torch
 
@@ -92,6 +92,61 @@ def check_against(entries: Dict[str, TensorEntry], wanted: Dict[str, TensorSpec]
                 wrong_kind.append((n, tag, s.kind))
     if missing or unexpected or wrong_shape or wrong_kind:
         raise WeightsError(where, sorted(missing), sorted(unexpected), wrong_shape, wrong_kind)
+
+
+class TensorSource(Mapping):
+    """Tensors made when a part asks for them, so that a large model never holds both the
+    checkpoint's tensors and what the parts fuse from them.  ``uses`` says how many parts
+    ask for each name: a tensor that several parts take (a tied table) is made once and
+    kept until the last of them has had it."""
+
+    def __init__(self, uses: Dict[str, int], make: Callable[[str], torch.Tensor]):
+        self._left = dict(uses)
+        self._make = make
+        self._kept: Dict[str, torch.Tensor] = {}
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        if name not in self._left:
+            raise KeyError(name)
+        t = self._kept.pop(name, None)
+        if t is None:
+            t = self._make(name)
+        self._left[name] -= 1
+        if self._left[name] > 0:
+            self._kept[name] = t
+        return t
+
+    def __iter__(self):
+        return iter(self._left)
+
+    def __len__(self) -> int:
+        return len(self._left)
+
+
+def open_tensors(
+    model_dir: str,
+    wanted: Dict[str, TensorSpec],
+    uses: Dict[str, int],
+    engine_dtype: str,
+    device: str,
+    progress: Optional[Callable[[str], None]] = None,
+) -> TensorSource:
+    """Check the folder against ``wanted`` (the one error lists everything that is wrong)
+    and return a source that reads each tensor onto ``device`` when it is asked for."""
+    entries = index_folder(model_dir)
+    check_against(entries, wanted, model_dir)
+    done = [0]
+
+    def make(name: str) -> torch.Tensor:
+        e = entries[name]
+        dt = target_dtype(e.dtype, wanted[name].kind, engine_dtype)
+        t = read_tensor(e).to(device=device, dtype=dt).contiguous()
+        done[0] += 1
+        if progress is not None and done[0] % 32 == 1:
+            progress(f"loaded {done[0]}/{len(wanted)} tensors")
+        return t
+
+    return TensorSource(uses, make)
 
 
 def load_tensors(
