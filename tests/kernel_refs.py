@@ -114,10 +114,15 @@ def attention(qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size, scale,
     return out.reshape(n, n_heads * head_dim).to(qkv.dtype)
 
 
-def gated_act(gu, activation, out_dtype=None):
+def gated_act(gu, activation, out_dtype=None, group=0):
     inter = gu.shape[1] // 2
-    g = gu[:, :inter].to(torch.float32)
-    u = gu[:, inter:].to(torch.float32)
+    if group:
+        pairs = gu.reshape(gu.shape[0], inter // group, 2, group)
+        g = pairs[:, :, 0, :].reshape(gu.shape[0], inter).to(torch.float32)
+        u = pairs[:, :, 1, :].reshape(gu.shape[0], inter).to(torch.float32)
+    else:
+        g = gu[:, :inter].to(torch.float32)
+        u = gu[:, inter:].to(torch.float32)
     if activation == "silu":
         a = g * torch.sigmoid(g)
     elif activation == "gelu_tanh":
@@ -151,6 +156,14 @@ class RefOps:
     attention = staticmethod(attention)
     gated_act = staticmethod(gated_act)
     argmax = staticmethod(argmax)
+
+    @staticmethod
+    def pack_gate_up(w_gate, w_up):
+        return torch.cat([w_gate, w_up], dim=0).contiguous(), 0
+
+    @staticmethod
+    def gate_up_act(x, w_gate_up, group, activation, out_dtype):
+        return gated_act(linear(x, w_gate_up, out_dtype), activation, out_dtype, group)
 
     def sample(self, logits, temperature, top_k, top_p, seeds, draws, whole_row=False):
         from plain_llama import sample_token

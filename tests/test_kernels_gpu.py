@@ -197,6 +197,42 @@ def test_split_sums_feed_their_consumers(ops):
     close(r3, res.cpu() + full.cpu(), 2e-6, 2e-6)
 
 
+@pytest.mark.parametrize("act", ["silu", "gelu_tanh"])
+@pytest.mark.parametrize("m,k,inter", [(1, 4096, 1024), (8, 512, 2048), (40, 320, 520), (64, 4096, 14336 // 4),
+                                       (5, 8192, 64), (70, 256, 328), (9, 192, 100)])
+def test_gate_up_act(ops, act, m, k, inter):
+    """Both projections and the activation: as one kernel where the product has few rows and
+    is not split over K, else product + activation kernel over the packed columns; the
+    same bits either way, and the plain arithmetic on [gate; up] within rounding."""
+    x = rnd((m, k), torch.bfloat16, 30, 0.7)
+    wg = rnd((inter, k), torch.bfloat16, 31, 0.05)
+    wu = rnd((inter, k), torch.bfloat16, 32, 0.05)
+    packed, group = ops.pack_gate_up(wg, wu)
+    assert group == (8 if inter % 8 == 0 else 0) and packed.shape == (2 * inter, k)
+    got = ops.gate_up_act(x, packed, group, act, torch.bfloat16)
+    assert got.shape == (m, inter)
+    # product, then the activation kernel on the packed columns
+    gu = ops.linear(x, packed, torch.bfloat16)
+    two_steps = ops.gated_act(gu, act, torch.bfloat16, group=group)
+    assert torch.equal(got, two_steps)
+    gate = (x.double().cpu() @ wg.double().cpu().T).to(torch.bfloat16)
+    up = (x.double().cpu() @ wu.double().cpu().T).to(torch.bfloat16)
+    want = R.gated_act(torch.cat([gate, up], dim=1).float(), act)
+    close(got, want, 3e-2, 2**-7)
+    # float32 weights are never packed
+    assert ops.pack_gate_up(wg.float(), wu.float())[1] == 0
+
+
+def test_gated_act_grouped_columns(ops):
+    gu = rnd((7, 2 * 72), torch.bfloat16, 33, 2.0)
+    for group in (0, 4, 8, 24):
+        close(ops.gated_act(gu, "silu", group=group), R.gated_act(gu.float().cpu(), "silu", group=group), 1e-2, 2**-7)
+    part = rnd((3, 7, 2 * 72), torch.float32, 34, 1.0)
+    from yalis_amd.ops.hip import SplitSum
+    close(ops.gated_act(SplitSum(part, torch.bfloat16), "silu", torch.bfloat16, group=8),
+          R.gated_act(part.sum(0).to(torch.bfloat16).float().cpu(), "silu", group=8), 1e-2, 2**-7)
+
+
 def test_linear_dispatch(ops):
     x = rnd((200, 192), torch.bfloat16, 8)
     w = rnd((515, 192), torch.bfloat16, 9)

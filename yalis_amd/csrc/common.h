@@ -76,6 +76,21 @@ __device__ __forceinline__ float wave_max(float v) {
 
 // Sum over a block of up to 1024 threads; every thread gets the result.
 // `scratch` is shared memory for 17 floats.
+// Gated activations: 0 = silu, 1 = gelu (tanh form); float32.
+__device__ __forceinline__ float act_silu(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float act_gelu_tanh(float z) {
+  const float k = 0.7978845608028654f;  // sqrt(2/pi)
+  return 0.5f * z * (1.f + tanhf(k * (z + 0.044715f * z * z * z)));
+}
+__device__ __forceinline__ float act_apply(float z, int act) { return act == 0 ? act_silu(z) : act_gelu_tanh(z); }
+
+// The sum of a product's K slices (or an accumulator) stands for the product's output: with
+// `round_sum` it is rounded to bfloat16 as that output would have been, so that what follows
+// does not depend on whether the product came reduced (bfloat16), as slices, or fused.
+__device__ __forceinline__ float as_output(float v, int round_sum) {
+  return round_sum ? to_f32<bf16_t>(from_f32<bf16_t>(v)) : v;
+}
+
 __device__ __forceinline__ float block_sum(float v, float* scratch) {
   v = wave_sum(v);
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;

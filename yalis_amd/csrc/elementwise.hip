@@ -25,7 +25,7 @@ int yk_check_launch(const char* what) {
   return 0;
 }
 extern "C" const char* yk_last_error() { return yk_error_slot().c_str(); }
-extern "C" int yk_abi_version() { return 3; }
+extern "C" int yk_abi_version() { return 4; }
 
 // ------------------------------------------------------------------------- embedding
 // out[n, :] = float(table[ids[n], :])
@@ -119,12 +119,8 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float4 v) {
   *reinterpret_cast<uint2*>(p) = raw;
 }
 
-// The sum of a product's K slices stands for the product's output: with `round_sum` it is
-// rounded to bfloat16 as that output would have been, so that what follows does not depend
-// on whether the product came reduced (bfloat16) or as slices.
-__device__ __forceinline__ float as_output(float v, int round_sum) {
-  return round_sum ? to_f32<bf16_t>(from_f32<bf16_t>(v)) : v;
-}
+// (as_output, in common.h: the sum of a product's K slices is rounded as the product's
+// output would have been)
 
 // ------------------------------------------------------------- residual add + RMS norm
 // For row r (source row rows[r] when rows is given):
@@ -537,25 +533,27 @@ extern "C" int yk_rope_append(const void* src, int src_dtype, int n_splits, int 
 }
 
 // ------------------------------------------------------------------ gated activation
-// out[n, j] = act(gu[n, j]) * gu[n, inter + j]; act 0 = silu, 1 = gelu (tanh form).
+// out[n, j] = act(gate[n, j]) * up[n, j]; act 0 = silu, 1 = gelu (tanh form).  The columns
+// of gu are [gate | up] (group 0) or alternate in groups: `group` gate columns, then the
+// `group` up columns that belong to them, and so on (the layout the fused product uses).
 // With n_splits > 1, gu holds unreduced float32 K slices [n_splits][rows][2 * inter].
-__device__ __forceinline__ float act_silu(float z) { return z / (1.f + expf(-z)); }
-__device__ __forceinline__ float act_gelu_tanh(float z) {
-  const float k = 0.7978845608028654f;  // sqrt(2/pi)
-  return 0.5f * z * (1.f + tanhf(k * (z + 0.044715f * z * z * z)));
+__device__ __forceinline__ size_t gate_col(size_t j, int inter, int group) {
+  return group ? (j / group) * 2 * group + j % group : j;
 }
-__device__ __forceinline__ float act_apply(float z, int act) { return act == 0 ? act_silu(z) : act_gelu_tanh(z); }
+__device__ __forceinline__ size_t up_offset(int inter, int group) { return group ? group : inter; }
+
 
 template <typename TS, typename TO>
 __global__ void gated_act_kernel(const TS* __restrict__ gu, int n_splits, size_t split_stride, int round_sum,
-                                 TO* __restrict__ out, int inter, size_t total, int act) {
+                                 TO* __restrict__ out, int inter, size_t total, int act, int group) {
   for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total;
        i += static_cast<size_t>(gridDim.x) * blockDim.x) {
     const size_t n = i / inter, j = i % inter;
     float g = 0.f, u = 0.f;
+    const size_t gc = n * 2 * inter + gate_col(j, inter, group);
     for (int s = 0; s < n_splits; ++s) {
-      g += to_f32<TS>(gu[s * split_stride + n * 2 * inter + j]);
-      u += to_f32<TS>(gu[s * split_stride + n * 2 * inter + inter + j]);
+      g += to_f32<TS>(gu[s * split_stride + gc]);
+      u += to_f32<TS>(gu[s * split_stride + gc + up_offset(inter, group)]);
     }
     g = as_output(g, round_sum);
     u = as_output(u, round_sum);
@@ -566,18 +564,19 @@ __global__ void gated_act_kernel(const TS* __restrict__ gu, int n_splits, size_t
 // four outputs per thread, no loop (inter a multiple of 4)
 template <typename TS, typename TO>
 __global__ void gated_act_vec_kernel(const TS* __restrict__ gu, int n_splits, size_t split_stride, int round_sum,
-                                     TO* __restrict__ out, int inter, size_t total_vec, int act) {
+                                     TO* __restrict__ out, int inter, size_t total_vec, int act, int group) {
   const size_t v = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
   if (v >= total_vec) return;
   const int per_row = inter / 4;
   const size_t n = v / per_row;
   const int j = static_cast<int>(v % per_row) * 4;
-  const TS* p = gu + n * 2 * inter + j;
-  float4 g = load4<TS>(p), u = load4<TS>(p + inter);
+  const TS* p = gu + n * 2 * inter + gate_col(j, inter, group);  // four columns of one group (group % 4 == 0)
+  const size_t up = up_offset(inter, group);
+  float4 g = load4<TS>(p), u = load4<TS>(p + up);
   for (int s0 = 1; s0 < n_splits; s0 += 2) {  // two slices in flight
     const int s1 = min(s0 + 1, n_splits - 1);
-    const float4 g2 = load4<TS>(p + s0 * split_stride), u2 = load4<TS>(p + s0 * split_stride + inter);
-    const float4 g3 = load4<TS>(p + s1 * split_stride), u3 = load4<TS>(p + s1 * split_stride + inter);
+    const float4 g2 = load4<TS>(p + s0 * split_stride), u2 = load4<TS>(p + s0 * split_stride + up);
+    const float4 g3 = load4<TS>(p + s1 * split_stride), u3 = load4<TS>(p + s1 * split_stride + up);
     g.x += g2.x; g.y += g2.y; g.z += g2.z; g.w += g2.w;
     u.x += u2.x; u.y += u2.y; u.z += u2.z; u.w += u2.w;
     if (s0 + 1 < n_splits) {
@@ -595,7 +594,7 @@ __global__ void gated_act_vec_kernel(const TS* __restrict__ gu, int n_splits, si
 
 template <typename TS, typename TO>
 static int launch_gated_act(const void* gu, int n_splits, int round_sum, void* out, int n_rows, int inter, int act,
-                            hipStream_t stream) {
+                            int group, hipStream_t stream) {
   const size_t stride = static_cast<size_t>(n_rows) * 2 * inter;
   const bool aligned = inter % 4 == 0 && reinterpret_cast<uintptr_t>(gu) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(out) % 16 == 0;
@@ -603,24 +602,25 @@ static int launch_gated_act(const void* gu, int n_splits, int round_sum, void* o
     const size_t total_vec = static_cast<size_t>(n_rows) * (inter / 4);
     YK_REQUIRE((total_vec + 255) / 256 < (1ull << 31), "gated_act: too large for one launch");
     gated_act_vec_kernel<TS, TO><<<static_cast<unsigned>((total_vec + 255) / 256), 256, 0, stream>>>(
-        static_cast<const TS*>(gu), n_splits, stride, round_sum, static_cast<TO*>(out), inter, total_vec, act);
+        static_cast<const TS*>(gu), n_splits, stride, round_sum, static_cast<TO*>(out), inter, total_vec, act, group);
   } else {
     const size_t total = static_cast<size_t>(n_rows) * inter;
     const int grid = static_cast<int>(std::min<size_t>((total + 255) / 256, 65535));
     gated_act_kernel<TS, TO><<<grid, 256, 0, stream>>>(static_cast<const TS*>(gu), n_splits, stride, round_sum,
-                                                        static_cast<TO*>(out), inter, total, act);
+                                                        static_cast<TO*>(out), inter, total, act, group);
   }
   return yk_check_launch("gated_act");
 }
 
 extern "C" int yk_gated_act(const void* gu, int src_dtype, int n_splits, int round_sum, void* out, int out_dtype,
-                            int n_rows, int inter, int act, hipStream_t stream) {
+                            int n_rows, int inter, int act, int group, hipStream_t stream) {
   YK_REQUIRE(n_rows >= 0 && inter > 0, "gated_act: bad sizes");
+  YK_REQUIRE(group == 0 || (group % 4 == 0 && inter % group == 0), "gated_act: groups are multiples of 4 that divide the width");
   YK_REQUIRE(act == 0 || act == 1, "gated_act: unknown activation");
   YK_REQUIRE(n_splits >= 1 && (n_splits == 1 || src_dtype == YK_F32), "gated_act: unreduced slices must be float32");
   if (n_rows == 0) return 0;
-  if (src_dtype == YK_F32 && out_dtype == YK_F32) return launch_gated_act<float, float>(gu, n_splits, round_sum, out, n_rows, inter, act, stream);
-  if (src_dtype == YK_F32 && out_dtype == YK_BF16) return launch_gated_act<float, bf16_t>(gu, n_splits, round_sum, out, n_rows, inter, act, stream);
-  if (src_dtype == YK_BF16 && out_dtype == YK_BF16) return launch_gated_act<bf16_t, bf16_t>(gu, n_splits, round_sum, out, n_rows, inter, act, stream);
+  if (src_dtype == YK_F32 && out_dtype == YK_F32) return launch_gated_act<float, float>(gu, n_splits, round_sum, out, n_rows, inter, act, group, stream);
+  if (src_dtype == YK_F32 && out_dtype == YK_BF16) return launch_gated_act<float, bf16_t>(gu, n_splits, round_sum, out, n_rows, inter, act, group, stream);
+  if (src_dtype == YK_BF16 && out_dtype == YK_BF16) return launch_gated_act<bf16_t, bf16_t>(gu, n_splits, round_sum, out, n_rows, inter, act, group, stream);
   return yk_fail("gated_act: unsupported dtype combination");
 }

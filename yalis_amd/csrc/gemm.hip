@@ -131,18 +131,22 @@ constexpr int SK_PAD = 8;             // bf16 elements of padding per LDS row (k
 constexpr int SK_ROW = SK_KC + SK_PAD;
 constexpr int SK_MAX_WAVES = 8;
 
+// x is parked in two buffers by turns where that costs no resident workgroup (up to 16 rows
+// of x): then one barrier a chunk is enough.  Measured: 2 to 5 % on the 8B shapes.
+static constexpr int skinny_x_buffers(int mt) { return mt == 1 ? 2 : 1; }
 static size_t skinny_lds_bytes(int mt, int waves) {
-  return static_cast<size_t>(16 * mt + 16 * waves) * SK_ROW * sizeof(bf16_t);
+  return static_cast<size_t>(16 * mt * skinny_x_buffers(mt) + 16 * waves) * SK_ROW * sizeof(bf16_t);
 }
 
-template <int MT, int W, typename TO>
+template <int MT, int W, typename TO, int GATED>
 __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, float* __restrict__ part,
     TO* __restrict__ y, int M, int N, int K, int ldx, int ldw, int ldy, int k_block) {
   extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
-  bf16_t(*xs)[SK_ROW] = reinterpret_cast<bf16_t(*)[SK_ROW]>(lds);  // [16 * MT][SK_ROW]
+  constexpr int XB = skinny_x_buffers(MT);
+  bf16_t(*xs0)[SK_ROW] = reinterpret_cast<bf16_t(*)[SK_ROW]>(lds);  // XB x [16 * MT][SK_ROW]
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
-  bf16_t(*wl)[SK_ROW] = reinterpret_cast<bf16_t(*)[SK_ROW]>(lds + static_cast<size_t>(16 * MT + 16 * wave) * SK_ROW);  // this wave's [16][SK_ROW]
+  bf16_t(*wl)[SK_ROW] = reinterpret_cast<bf16_t(*)[SK_ROW]>(lds + static_cast<size_t>(16 * MT * XB + 16 * wave) * SK_ROW);  // this wave's [16][SK_ROW]
   const int r = lane % 16, g = lane / 16;
   const int n0 = (blockIdx.x * W + wave) * 16;
   const int m0 = blockIdx.y * (16 * MT);
@@ -167,7 +171,7 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
         regs[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wrow[j] + kk_)); \
   }
   // x: the chunk's 16*MT rows x 32 pieces of 16 bytes are spread over the threads, XP each;
-  // what lies outside M or the slice becomes zero after the (clamped) load
+  // what lies outside M or the slice is loaded from a clamped address and parked as zero
   constexpr int XP = 16 * MT * (SK_KC / 8) / (W * 64);
   static_assert(XP * W * 64 == 16 * MT * (SK_KC / 8), "x pieces must divide evenly over the threads");
   u32x4_t xr[XP];
@@ -177,20 +181,27 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
     const int e_ = threadIdx.x + p * W * 64;                                                 \
     const int m_ = m0 + e_ / (SK_KC / 8), k_ = (KC0) + 8 * (e_ % (SK_KC / 8));               \
     xr[p] = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(min(m_, M - 1)) * ldx + min(k_, k_last)); \
-    if (m_ >= M || k_ >= kb1) xr[p] = zero;                                                  \
   }
 
   SK_LOAD_W(kb0)
   SK_LOAD_X(kb0)
-  for (int kc = kb0; kc < kb1; kc += SK_KC) {
-    __syncthreads();  // every wave has read the previous chunk of x
+  int turn = 0;
+  for (int kc = kb0; kc < kb1; kc += SK_KC, turn ^= 1) {
+    // With one buffer every wave must have read the previous chunk of x before it is
+    // overwritten.  With two, the buffer written now was last read two chunks ago, and every
+    // wave finished that before it passed the previous chunk's barrier.
+    if (XB == 1) __syncthreads();
+    bf16_t(*xs)[SK_ROW] = xs0 + (XB == 2 ? turn * 16 * MT : 0);
     // park what has arrived, then put the next chunk's loads in flight
 #pragma unroll
     for (int j = 0; j < SK_STEPS; ++j) *reinterpret_cast<u32x4_t*>(&wl[2 * j + half][8 * l32]) = regs[j];
 #pragma unroll
     for (int p = 0; p < XP; ++p) {
+      // (zeroed here, not at the load: a select right behind the load would make the wave
+      // wait for everything it has just put in flight)
       const int e = threadIdx.x + p * W * 64;
-      *reinterpret_cast<u32x4_t*>(&xs[e / (SK_KC / 8)][8 * (e % (SK_KC / 8))]) = xr[p];
+      const bool outside = m0 + e / (SK_KC / 8) >= M || kc + 8 * (e % (SK_KC / 8)) >= kb1;
+      *reinterpret_cast<u32x4_t*>(&xs[e / (SK_KC / 8)][8 * (e % (SK_KC / 8))]) = outside ? zero : xr[p];
     }
     if (kc + SK_KC < kb1) {
       SK_LOAD_W(kc + SK_KC)
@@ -212,6 +223,26 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
 #undef SK_LOAD_W
 #undef SK_LOAD_X
 
+  if (GATED) {
+    // The weight's rows alternate: 8 gate rows, then the 8 up rows that belong to them.  A
+    // wave's tile holds one such pair of groups: lane groups 0 and 1 have the gate features
+    // 0..7 of a token, groups 2 and 3 the up features, 32 lanes further.  Both are rounded
+    // as the product's output would have been, then out = act(gate) * up, 8 columns a tile.
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      f32x4_t up;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) up[e] = __shfl_xor(acc[t][e], 32, 64);
+      const int m = m0 + 16 * t + r;
+      if (g < 2 && m < M && n0 < N) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          y[static_cast<size_t>(m) * ldy + n0 / 2 + 4 * g + e] =
+              from_f32<TO>(act_apply(as_output(acc[t][e], 1), GATED - 1) * as_output(up[e], 1));
+      }
+    }
+    return;
+  }
   const bool to_part = part != nullptr;
   float* pout = to_part ? part + static_cast<size_t>(blockIdx.z) * M * N : nullptr;
   const int n = n0 + 4 * g;
@@ -307,25 +338,28 @@ extern "C" int yk_gemm_skinny_splits(int M, int N, int K) { return skinny_plan(M
 
 template <typename TO>
 static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, int M, int N, int K,
-                         int ldx, int ldw, int ldy, int waves, int k_block, int splits, hipStream_t stream) {
+                         int ldx, int ldw, int ldy, int waves, int k_block, int splits, int gated, hipStream_t stream) {
   const int mt = skinny_mt(M);
   dim3 grid((N + 16 * waves - 1) / (16 * waves), (M + 16 * mt - 1) / (16 * mt), splits);
   YK_REQUIRE(grid.y <= 65535, "gemm_mfma_skinny: too many rows for one launch");
   dim3 block(waves * 64);
   const size_t lds = skinny_lds_bytes(mt, waves);
-#define SK_GO(MT_, W_)                                                                                   \
-  if (mt == MT_ && waves == W_) {                                                                       \
+#define SK_GO(MT_, W_, G_)                                                                               \
+  if (mt == MT_ && waves == W_ && gated == G_) {                                                        \
     static bool raised = false; /* allow more than the default 64 KB of dynamic LDS, once */           \
     if (!raised) {                                                                                      \
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_kernel<MT_, W_, TO>),     \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_kernel<MT_, W_, TO, G_>), \
                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)    \
         return yk_fail("gemm_mfma_skinny: cannot raise the LDS limit");                                 \
       raised = true;                                                                                    \
     }                                                                                                   \
-    gemm_mfma_skinny_kernel<MT_, W_, TO><<<grid, block, lds, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block); \
+    gemm_mfma_skinny_kernel<MT_, W_, TO, G_><<<grid, block, lds, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block); \
     return yk_check_launch("gemm_mfma_skinny");                                                         \
   }
-  SK_GO(1, 4) SK_GO(1, 8) SK_GO(2, 4) SK_GO(2, 8) SK_GO(4, 4) SK_GO(4, 8)
+  SK_GO(1, 4, 0) SK_GO(2, 4, 0) SK_GO(4, 4, 0)
+  if constexpr (sizeof(TO) == 2) {  // gated results are bfloat16 only
+    SK_GO(1, 4, 1) SK_GO(2, 4, 1) SK_GO(4, 4, 1) SK_GO(1, 4, 2) SK_GO(2, 4, 2) SK_GO(4, 4, 2)
+  }
 #undef SK_GO
   return yk_fail("gemm_mfma_skinny: no kernel for this plan");
 }
@@ -334,31 +368,37 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, i
 // a consumer that sums them itself (y is not written unless there is a single slice and
 // y is given).  Returns the number of slices written to the workspace (0: y holds the
 // result), or a negative number on error.
+// gated: 0 = y is the product [M, N].  1 (silu) or 2 (gelu-tanh): the rows of w alternate in
+// groups of 8 gate rows and their 8 up rows, and y [M, N / 2] = act(gate) * up; only where the
+// plan does not split K (yk_gemm_skinny_splits == 1), and N a multiple of 16.
 extern "C" int yk_gemm_mfma_skinny(const void* x, const void* w, void* y, int y_dtype,
                                    float* workspace, size_t workspace_floats, int M, int N, int K,
-                                   int ldx, int ldw, int ldy, int keep_splits,
+                                   int ldx, int ldw, int ldy, int keep_splits, int gated,
                                    hipStream_t stream) {
   YK_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_mfma_skinny: bad sizes");
   YK_REQUIRE(K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0,
              "gemm_mfma_skinny: K and the leading dimensions must be multiples of 8");
   YK_REQUIRE((reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(w) % 16 == 0),
              "gemm_mfma_skinny: operands must be 16-byte aligned");
-  YK_REQUIRE(ldx >= K && ldw >= K && ldy >= N, "gemm_mfma_skinny: leading dimensions too small");
+  YK_REQUIRE(gated >= 0 && gated <= 2, "gemm_mfma_skinny: unknown activation");
+  YK_REQUIRE(ldx >= K && ldw >= K && ldy >= (gated ? N / 2 : N), "gemm_mfma_skinny: leading dimensions too small");
+  YK_REQUIRE(!gated || (N % 16 == 0 && y_dtype == YK_BF16 && !keep_splits), "gemm_mfma_skinny: a gated product needs N % 16 == 0 and a bfloat16 result");
   YK_REQUIRE(y_dtype == YK_F32 || y_dtype == YK_BF16, "gemm_mfma_skinny: unsupported output dtype");
   if (M == 0) return 0;
   int k_block = 0, waves = 4;
   const int splits = skinny_plan(M, N, K, &waves, &k_block);
+  YK_REQUIRE(!gated || splits == 1, "gemm_mfma_skinny: a gated product cannot split K");
   const bf16_t* xp = static_cast<const bf16_t*>(x);
   const bf16_t* wp = static_cast<const bf16_t*>(w);
   if (splits == 1 && !keep_splits) {
     int rc = y_dtype == YK_F32
-                 ? launch_skinny<float>(xp, wp, nullptr, static_cast<float*>(y), M, N, K, ldx, ldw, ldy, waves, k_block, 1, stream)
-                 : launch_skinny<bf16_t>(xp, wp, nullptr, static_cast<bf16_t*>(y), M, N, K, ldx, ldw, ldy, waves, k_block, 1, stream);
+                 ? launch_skinny<float>(xp, wp, nullptr, static_cast<float*>(y), M, N, K, ldx, ldw, ldy, waves, k_block, 1, gated, stream)
+                 : launch_skinny<bf16_t>(xp, wp, nullptr, static_cast<bf16_t*>(y), M, N, K, ldx, ldw, ldy, waves, k_block, 1, gated, stream);
     return rc;
   }
   YK_REQUIRE(workspace && workspace_floats >= static_cast<size_t>(splits) * M * N,
              "gemm_mfma_skinny: workspace too small");
-  if (launch_skinny<float>(xp, wp, workspace, nullptr, M, N, K, ldx, ldw, ldy, waves, k_block, splits, stream)) return -1;
+  if (launch_skinny<float>(xp, wp, workspace, nullptr, M, N, K, ldx, ldw, ldy, waves, k_block, splits, 0, stream)) return -1;
   if (keep_splits) return splits;
   const size_t total = static_cast<size_t>(M) * N;
   const int rb = 256;

@@ -52,14 +52,14 @@ _SIGNATURES = {
          _c_int, _c_int, _c_int, _vp, _vp, _vp, _c_int, _vp],
         _c_int,
     ),
-    "yk_gated_act": ([_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _vp], _c_int),
+    "yk_gated_act": ([_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_gemm_fma": (
         [_vp, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
         _c_int,
     ),
     "yk_gemm_skinny_splits": ([_c_int, _c_int, _c_int], _c_int),
     "yk_gemm_mfma_skinny": (
-        [_vp, _vp, _vp, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
+        [_vp, _vp, _vp, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
         _c_int,
     ),
     "yk_attn_generic": (
@@ -130,7 +130,7 @@ class HipOps:
             fn = getattr(self.lib, name)
             fn.argtypes = args
             fn.restype = res
-        if self.lib.yk_abi_version() != 3:
+        if self.lib.yk_abi_version() != 4:
             raise KernelError("kernel library and bindings disagree; rebuild (python -c 'import __graft_entry__ as g; g.build()')")
         self._workspace: Optional[torch.Tensor] = None  # attention splits, argmax parts
         self._gemm_workspace: Optional[torch.Tensor] = None  # K slices of products
@@ -261,6 +261,49 @@ class HipOps:
         )
         return y
 
+    # ---------------------------------------------------------- gate/up + activation
+    GATE_UP_GROUP = 8  # rows of the packed matrix alternate: 8 of gate, their 8 of up
+
+    def pack_gate_up(self, w_gate: torch.Tensor, w_up: torch.Tensor) -> Tuple[torch.Tensor, int]:
+        """One matrix for both projections and the group size of its row order: 0 = [gate; up];
+        8 = eight gate rows, then their eight up rows, and so on, which lets the few-row
+        product apply the activation itself (the reference keeps gate and up in one matrix
+        with rows interleaved too, yalis/external/model.py:717-722)."""
+        inter = w_gate.shape[0]
+        g = self.GATE_UP_GROUP
+        if w_gate.dtype == torch.bfloat16 and w_up.dtype == torch.bfloat16 and inter % g == 0:
+            packed = torch.stack([w_gate.view(inter // g, g, -1), w_up.view(inter // g, g, -1)], dim=1)
+            return packed.reshape(2 * inter, -1).contiguous(), g
+        return torch.cat([w_gate, w_up], dim=0).contiguous(), 0
+
+    def gate_up_act(self, x: torch.Tensor, w_gate_up: torch.Tensor, group: int, activation: str, out_dtype: torch.dtype) -> torch.Tensor:
+        """act(x . gate^T) * (x . up^T) -> [M, intermediate], ``w_gate_up`` and ``group`` as
+        ``pack_gate_up`` gave them.  Few rows of bfloat16 whose product is not split over K
+        run as one kernel; otherwise the product, then the activation kernel."""
+        act = {"silu": 1, "gelu_tanh": 2}.get(activation)
+        if act is None:
+            raise KernelError(f"unknown activation {activation!r}")
+        self._rows(x, "gate/up input")
+        m, k = x.shape
+        n = w_gate_up.shape[0]
+        bf = torch.bfloat16
+        fused = (
+            group == self.GATE_UP_GROUP and 0 < m <= SKINNY_MAX_ROWS and x.dtype == bf and w_gate_up.dtype == bf and out_dtype == bf
+            and w_gate_up.shape[1] == k and k % 8 == 0 and x.stride(0) % 8 == 0 and w_gate_up.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0 and n % 16 == 0
+            and self.lib.yk_gemm_skinny_splits(m, n, k) == 1
+        )
+        if not fused:
+            return self.gated_act(self.linear(x, w_gate_up, out_dtype, partial_ok=True), activation, out_dtype, group=group)
+        y = torch.empty((m, n // 2), dtype=bf, device=x.device)
+        rc = self.lib.yk_gemm_mfma_skinny(
+            x.data_ptr(), w_gate_up.data_ptr(), y.data_ptr(), _code(bf), None, 0,
+            m, n, k, x.stride(0), w_gate_up.stride(0), n // 2, 0, act, self._stream(),
+        )
+        if rc < 0:
+            self._check(rc)
+        return y
+
     def gemm_mfma_skinny(self, x, w, out_dtype, partial_ok: bool = False):
         m, k = x.shape
         n = w.shape[0]
@@ -270,7 +313,7 @@ class HipOps:
         y = None if keep else torch.empty((m, n), dtype=out_dtype, device=x.device)
         rc = self.lib.yk_gemm_mfma_skinny(
             x.data_ptr(), w.data_ptr(), _ptr(y), _code(out_dtype), _ptr(ws), 0 if ws is None else ws.numel(),
-            m, n, k, x.stride(0), w.stride(0), n, int(keep), self._stream(),
+            m, n, k, x.stride(0), w.stride(0), n, int(keep), 0, self._stream(),
         )
         if rc < 0:
             raise KernelError(self.lib.yk_last_error().decode())
@@ -391,7 +434,9 @@ class HipOps:
         return out
 
     # ----------------------------------------------------------------- activation
-    def gated_act(self, gu, activation: str, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    def gated_act(self, gu, activation: str, out_dtype: Optional[torch.dtype] = None, group: int = 0) -> torch.Tensor:
+        """act(gate) * up for gate/up columns [gate | up] (group 0) or alternating in groups
+        of ``group`` columns (see ``pack_gate_up``)."""
         n_splits, round_sum = 1, 0
         src = gu
         if isinstance(gu, SplitSum):
@@ -413,7 +458,7 @@ class HipOps:
         out = torch.empty((rows, inter), dtype=out_dtype, device=src.device)
         self._check(
             self.lib.yk_gated_act(src.data_ptr(), _code(src.dtype), n_splits, round_sum, out.data_ptr(), _code(out_dtype),
-                                  rows, inter, act, self._stream())
+                                  rows, inter, act, int(group), self._stream())
         )
         return out
 

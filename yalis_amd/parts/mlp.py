@@ -1,9 +1,10 @@
 """Gated feed-forward (SwiGLU for Llama).
 
 Reference: yalis/external/model.py:710-744: down(act(gate(x)) * up(x)) without
-biases; the reference interleaves gate and up rows in one matrix (:717-722,
-:741-743), here they are stacked [gate; up], which is the same arithmetic.  The
-activation and product are computed in float32 on the projection's output.
+biases.  The reference keeps gate and up in one matrix with rows interleaved (:717-722,
+:741-743); here the kernel library packs the two (``ops.pack_gate_up``) in the row order
+its products want, which is the same arithmetic.  The activation and product are computed
+in float32 on the projection's output.
 
 params: prefix, hidden_size, intermediate_size, activation ("silu"), names
 (optional overrides of the three tensor names below the prefix).
@@ -36,6 +37,7 @@ class GatedMLP(FeedForward):
         names.update(params.get("names", {}))
         self.names = {k: f"{self.prefix}.{v}" for k, v in names.items()}
         self.w_gate_up = self.w_down = None
+        self.gate_up_group = 0
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         return {
@@ -45,11 +47,10 @@ class GatedMLP(FeedForward):
         }
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        self.w_gate_up = torch.cat([tensors[self.names["gate"]], tensors[self.names["up"]]], dim=0).contiguous()
+        self.w_gate_up, self.gate_up_group = self.rt.ops.pack_gate_up(tensors[self.names["gate"]], tensors[self.names["up"]])
         self.w_down = tensors[self.names["down"]]
 
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
         ops = self.rt.ops
-        gu = ops.linear(h, self.w_gate_up, self.rt.act_dtype, partial_ok=True)
-        a = ops.gated_act(gu, self.activation, self.rt.act_dtype)
+        a = ops.gate_up_act(h, self.w_gate_up, self.gate_up_group, self.activation, self.rt.act_dtype)
         return ops.linear(a, self.w_down, self.rt.act_dtype, partial_ok=True)
