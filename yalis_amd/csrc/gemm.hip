@@ -174,13 +174,15 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
   // what lies outside M or the slice is loaded from a clamped address and parked as zero
   constexpr int XP = 16 * MT * (SK_KC / 8) / (W * 64);
   static_assert(XP * W * 64 == 16 * MT * (SK_KC / 8), "x pieces must divide evenly over the threads");
-  u32x4_t xr[XP];
   const u32x4_t zero = {0u, 0u, 0u, 0u};
+  u32x4_t xr[XP];
+#pragma unroll
+  for (int p = 0; p < XP; ++p) xr[p] = zero;
 #define SK_LOAD_X(KC0)                                                                      \
   _Pragma("unroll") for (int p = 0; p < XP; ++p) {                                           \
     const int e_ = threadIdx.x + p * W * 64;                                                 \
     const int m_ = m0 + e_ / (SK_KC / 8), k_ = (KC0) + 8 * (e_ % (SK_KC / 8));               \
-    xr[p] = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(min(m_, M - 1)) * ldx + min(k_, k_last)); \
+    if (m_ < M) xr[p] = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(m_) * ldx + min(k_, k_last)); \
   }
 
   SK_LOAD_W(kb0)
