@@ -97,6 +97,30 @@ def test_greedy_matches_plain(tmp_path, backend, engine_kw):
     assert eng.runner.pages.live_requests() == 0
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_bfloat16_follows_float32_by_the_reference_rule(tmp_path, name):
+    """The reference compares two implementations' greedy tokens until they first differ
+    and then asks that each one's token is among the other's five most likely
+    (tests/basic_correctness/test_yalis_vs_hf.py:163-185, NUM_LOGPROBS = 5 at :7); here the bfloat16 engine against the true float32 engine."""
+    n_new = 24
+    outs = {}
+    for precision in ("fp32", "bf16"):
+        eng, cfg, _ = make_engine(tmp_path / precision, name, ("cuda:0", precision), 4, temperature=0.0,
+                                  page_size=16, num_pages=64, max_num_batched_tokens=2048)
+        prompts = prompts_for(cfg, [9, 33, 70, 2], seed=21)
+        toks, _, logits = eng.generate(prompts, tokens_to_generate=n_new, get_logits=True)
+        outs[precision] = (toks.tolist(), [step.float().cpu() for step in logits])
+    for r in range(4):
+        a, b = outs["fp32"][0][r], outs["bf16"][0][r]
+        for i in range(n_new):
+            if a[i] != b[i]:
+                top_a = torch.topk(outs["fp32"][1][i][r], 5).indices.tolist()
+                top_b = torch.topk(outs["bf16"][1][i][r], 5).indices.tolist()
+                assert a[i] in top_b and b[i] in top_a, (r, i, a[i], b[i], top_a, top_b)
+                break
+
+
 @pytest.mark.parametrize("backend", BACKENDS[:2])
 def test_temperature_sampling_matches_plain(tmp_path, backend):
     """Tiny B, prompts of 1/40/130 tokens, temperature 0.7, 24 tokens, page size 32: the
