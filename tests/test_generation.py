@@ -171,3 +171,32 @@ def test_engine_refuses_what_it_cannot_run(tmp_path):
         eng.generate(prompts_for(cfg, [60]), tokens_to_generate=30)
     with pytest.raises(ValueError, match="tokenizer"):
         eng.generate(["text"], tokens_to_generate=2)
+
+
+@pytest.mark.gpu
+def test_command_line(tmp_path):
+    """``python -m yalis_amd.infer`` on a random model folder: prompts as ids on the command
+    line and from a file, greedy, float32; the printed tokens are the plain implementation's."""
+    import ast
+    import subprocess
+    import sys
+
+    from yalis_amd.weights.random_init import write_random_model
+    from yalis_amd.weights.safetensors_io import index_folder, read_tensor
+
+    cfg = ALL["C"]
+    folder = write_random_model(str(tmp_path / "m"), cfg, seed=4, dtype="float32")
+    weights = {n: read_tensor(e).float() for n, e in index_folder(folder).items()}
+    prompts = prompts_for(cfg, [6, 19], seed=8)
+    ids = [",".join(str(t) for t in p) for p in prompts]
+    listing = tmp_path / "prompts.txt"
+    listing.write_text("\n".join(ids) + "\n")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    base = [sys.executable, "-m", "yalis_amd.infer", "--model", folder, "--dtype", "float32", "--temperature", "0",
+            "--max-tokens", "8", "--max-num-seqs", "2", "--max-length-of-generated-sequences", "128", "--page-size", "16"]
+    for how in (["--prompt-ids", ids[0], "--prompt-ids", ids[1]], ["--prompt-file", str(listing)]):
+        run = subprocess.run(base + how, cwd=root, capture_output=True, text=True, timeout=300)
+        assert run.returncode == 0, run.stderr[-2000:]
+        outs = [ast.literal_eval(ln.split("=", 1)[1].strip()) for ln in run.stdout.splitlines() if ln.startswith("output =")]
+        assert outs == [P.greedy_generate(cfg, weights, p, 8) for p in prompts]
+        assert "metrics = " in run.stdout and "Number of prompts = 2" in run.stdout

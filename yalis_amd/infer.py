@@ -14,11 +14,13 @@ from typing import List
 
 import torch
 
+# used when no prompt is given and the folder has a tokenizer (the reference's script has a
+# list of its own built in, examples/infer.py:18-35)
 DEFAULT_PROMPTS = [
-    "How to bake a cake?",
-    "Explain quantum mechanics in simple terms.",
-    "What are the benefits of a balanced diet?",
-    "How can I learn to play the guitar?",
+    "Describe how a paged key-value cache hands out and takes back its pages.",
+    "Why does decoding one token at a time read every weight of the model?",
+    "Write a short note on what limits the speed of a matrix product with few rows.",
+    "Name three things a scheduler must decide when the cache is full.",
 ]
 
 
@@ -26,12 +28,13 @@ def parse_args(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--model", "--model-path", dest="model_path", required=True, help="folder with config.json, model.safetensors (and a tokenizer for text prompts)")
     ap.add_argument("--model-name", default=None)
-    ap.add_argument("--precision", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--precision", "--dtype", dest="precision", default="bf16", choices=["bf16", "fp32", "bfloat16", "float32"])
     ap.add_argument("--prompt", action="append", default=[], help="a text prompt (repeatable; needs a tokenizer)")
     ap.add_argument("--prompt-ids", action="append", default=[], help="a prompt as comma-separated token ids (repeatable)")
     ap.add_argument("--random-prompts", default=None, metavar="N,LEN", help="N prompts of LEN seeded random token ids")
-    ap.add_argument("--tokens-to-generate", type=int, default=50)
-    ap.add_argument("--max-batch-size", type=int, default=32)
+    ap.add_argument("--prompt-file", default=None, help="a file with one prompt a line: text, or comma-separated token ids")
+    ap.add_argument("--tokens-to-generate", "--max-tokens", dest="tokens_to_generate", type=int, default=50)
+    ap.add_argument("--max-batch-size", "--max-num-seqs", dest="max_batch_size", type=int, default=32)
     ap.add_argument("--max-length-of-generated-sequences", type=int, default=1024)
     ap.add_argument("--temperature", type=float, default=1.0)
     ap.add_argument("--top-k", type=int, default=None)
@@ -39,11 +42,12 @@ def parse_args(argv=None):
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--iters", type=int, default=1, help="timed generate calls (the reference script runs 10)")
     ap.add_argument("--no-ignore-eos", action="store_true", help="stop a request at its EOS token")
+    ap.add_argument("--ignore-eos", action="store_true", help="generate past EOS (the default, as in the reference)")
     ap.add_argument("--report-throughput", action="store_true")
     ap.add_argument("--random-weights-seed", type=int, default=None, help="ignore the folder's weights; random ones from this seed")
     ap.add_argument("--page-size", type=int, default=64)
     ap.add_argument("--num-pages", type=int, default=None)
-    ap.add_argument("--max-num-batched-tokens", type=int, default=2048)
+    ap.add_argument("--max-num-batched-tokens", "--max-batched-tokens", dest="max_num_batched_tokens", type=int, default=2048)
     return ap.parse_args(argv)
 
 
@@ -81,6 +85,11 @@ def main(argv=None) -> int:
         g = torch.Generator().manual_seed(args.seed)
         vocab = engine.model.spec.vocab_size
         prompts = [torch.randint(0, vocab, (length,), generator=g).tolist() for _ in range(n)]
+    elif args.prompt_file:
+        with open(args.prompt_file, encoding="utf-8") as f:
+            lines = [ln.strip() for ln in f if ln.strip()]
+        as_ids = all(all(t.strip().isdigit() for t in ln.split(",")) for ln in lines)
+        prompts = [[int(t) for t in ln.split(",")] for ln in lines] if as_ids else lines
     elif args.prompt:
         prompts = list(args.prompt)
     else:
