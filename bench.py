@@ -7,7 +7,10 @@ batch x tokens / time, TBT = mean time of a decode step: yalis/engine.py:531-557
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L]
 
 A step is one decode step through the engine's own path: page reservation, the step
-function over the paged cache, greedy sampling, the token back on the host.
+function over the paged cache, greedy sampling.  As in ``LLMEngine.generate``, steps that need
+no decision of the scheduler are launched one behind the other, each feeding on the tokens the
+step before left on the device; the tokens of all timed steps are on the host when the clock
+stops.
 """
 import argparse
 import json
@@ -109,12 +112,19 @@ def main() -> int:
 
         for _ in range(warmup):
             toks = one_step(toks)
+        entries = [StepEntry(r, [0], [0]) for r in range(batch)]
+        last = torch.tensor(toks, dtype=torch.int32, device="cuda")
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         ctx_sum = 0
+        run = []
+        for r in range(batch):
+            assert runner.reserve(r, steps)
         for _ in range(steps):
             ctx_sum += sum(runner.cached[r] + 1 for r in range(batch))
-            toks = one_step(toks)
+            last = ops.argmax(runner.step(entries, token_source=last))
+            run.append(last)
+        toks = torch.stack(run).tolist()[-1]
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         for r in range(batch):

@@ -97,6 +97,26 @@ def test_greedy_matches_plain(tmp_path, backend, engine_kw):
     assert eng.runner.pages.live_requests() == 0
 
 
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("temperature,top_k,top_p", [(0.0, None, 1.0), (0.9, 12, 0.8)])
+def test_steps_launched_ahead_change_nothing(tmp_path, backend, temperature, top_k, top_p):
+    """Decode steps that need no decision are launched without waiting for the tokens of the
+    step before; asking for the logits switches that off.  Both ways give the same tokens,
+    also when requests have different lengths to go and finish at different steps."""
+    eng, cfg, _ = make_engine(tmp_path, "C", backend, 3, temperature=temperature, top_k=top_k, top_p=top_p,
+                              page_size=16, num_pages=40, max_num_batched_tokens=64)
+    prompts = prompts_for(cfg, [7, 40, 21], seed=31)
+    ahead, m1 = eng.generate(prompts, tokens_to_generate=20)
+    plain, m2, _ = eng.generate(prompts, tokens_to_generate=20, get_logits=True)
+    assert m1["StepsLaunchedAhead"] >= 15 and m2["StepsLaunchedAhead"] == 0
+    assert torch.equal(ahead, plain)
+    # a request that stops at EOS needs its tokens on the host: nothing is launched ahead
+    _, m3 = eng.generate(prompts, tokens_to_generate=6, ignore_eos=False)
+    assert m3["StepsLaunchedAhead"] == 0
+    eng.runner.pages.audit()
+    assert eng.runner.pages.live_requests() == 0
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", ["B", "C"])
 def test_bfloat16_follows_float32_by_the_reference_rule(tmp_path, name):

@@ -124,3 +124,44 @@ def test_requests_that_can_never_run_are_refused():
     assert r.params.max_tokens == 13
     sched2, _ = make(num_pages=16)
     assert sched2.add(list(range(100)), greedy(500)).params.max_tokens == 28, "clamped to the context"
+
+
+def test_steps_that_need_no_decision():
+    """``run_ahead_steps``: how many single-token steps may follow a launched plan before the
+    scheduler has anything to decide; it reserves their pages."""
+    sched, runner = make(num_pages=16, max_seqs=4, budget=64)
+    a = sched.add(list(range(1, 11)), SamplingParams(temperature=0.0, max_tokens=9))
+    b = sched.add(list(range(1, 31)), SamplingParams(temperature=0.0, max_tokens=5))
+    plan = sched.schedule()
+    for s in plan:
+        runner.cached[s.request.rid] += s.n_tokens
+    # both prompts whole, both sample: b needs 4 more tokens after this step's, a needs 8
+    assert [s.samples for s in plan] == [True, True]
+    assert sched.run_ahead_steps(plan) == 4
+    assert sched.run_ahead_steps(plan, limit=3) == 3
+    # pages for those steps are there: 10 + 4 and 30 + 4 tokens
+    assert runner.pages.reserve(a.rid, 14) and runner.pages.reserve(b.rid, 34)
+    sched.update(plan, [1, 1])
+    # a third request waits: the next step must admit it, nothing runs ahead
+    sched.add([1, 2, 3], SamplingParams(temperature=0.0, max_tokens=4))
+    assert sched.run_ahead_steps(plan) == 0
+    # EOS may stop a request: its tokens are needed on the host
+    sched2, runner2 = make()
+    sched2.add([1, 2, 3], SamplingParams(temperature=0.0, max_tokens=9, ignore_eos=False))
+    plan2 = sched2.schedule()
+    for s in plan2:
+        runner2.cached[s.request.rid] += s.n_tokens
+    assert sched2.run_ahead_steps(plan2) == 0
+    # a portion of a prompt that does not sample yet: no
+    sched3, runner3 = make(budget=8)
+    sched3.add(list(range(1, 21)), SamplingParams(temperature=0.0, max_tokens=9))
+    plan3 = sched3.schedule()
+    assert not plan3[0].samples and sched3.run_ahead_steps(plan3) == 0
+    # a pool that cannot hold all the steps of both requests: as many as it can (halving)
+    sched4, runner4 = make(num_pages=3, page=16)
+    for _ in range(2):
+        sched4.add(list(range(1, 15)), SamplingParams(temperature=0.0, max_tokens=18))
+    plan4 = sched4.schedule()
+    for s in plan4:
+        runner4.cached[s.request.rid] += s.n_tokens
+    assert len(plan4) == 2 and sched4.run_ahead_steps(plan4) == 2  # 14 + 2 tokens fill each one's first page

@@ -16,7 +16,8 @@ from ..config.reader import read_config_json
 from ..config.runtime import EngineConfig, InferenceConfig, ModelConfig
 from ..sampling.sampler import Sampler, SamplingParams
 from .factory import load_runner, random_runner
-from .scheduler import Request, Scheduler
+from .scheduler import Request, Scheduled, Scheduler
+from .step import StepEntry
 
 
 def print_rank0(*args, **kwargs) -> None:
@@ -130,31 +131,66 @@ class LLMEngine:
 
         cuda = torch.cuda.is_available() and self.engine_config.device.startswith("cuda")
         sync = torch.cuda.synchronize if cuda else (lambda: None)
+
+        # points in time on the device's own clock: with steps launched ahead of the host's
+        # knowledge of their tokens, the host's clock would date a token by when it was read
+        def mark():
+            if not cuda:
+                return time.perf_counter()
+            ev = torch.cuda.Event(enable_timing=True)
+            ev.record()
+            return ev
+
+        def seconds(a, b) -> float:
+            return (b - a) if not cuda else a.elapsed_time(b) * 1e-3
+
         sync()
         t0 = time.perf_counter()
-        first_token_at: Dict[int, float] = {}
+        m0 = mark()
+        first_token_at: Dict[int, object] = {}
         decode_steps = 0
-        decode_time = 0.0
+        decode_spans = []  # (mark before, mark after, steps)
+        steps_ahead = 0
         while sched.has_work():
-            t_step = time.perf_counter()
+            before = mark()
             plan = sched.schedule()
             if not plan:
                 raise RuntimeError("the scheduler made no progress (pool too small for any request?)")
             logits = self.runner.step(sched.entries(plan))
             sampling = [s.request for s in plan if s.samples]
-            toks = self.sampler.sample(logits, [r.params for r in sampling], [len(r.output) for r in sampling])
+            prepared = self.sampler.prepare([r.params for r in sampling], [len(r.output) for r in sampling])
+            toks = self.sampler.sample_prepared(logits, prepared, 0) if sampling else None
+            after = mark()
+            for r in sampling:
+                first_token_at.setdefault(r.rid, after)
+            if all(s.n_tokens == 1 and s.samples for s in plan):
+                decode_spans.append((before, after, 1))
             if get_logits:
                 for r, row in zip(sampling, logits):
                     r.logits.append(row.clone())
-            sched.update(plan, toks)
-            now = time.perf_counter()
-            for r in sampling:
-                first_token_at.setdefault(r.rid, now)
-            if all(s.n_tokens == 1 and s.samples for s in plan):
-                decode_steps += 1
-                decode_time += now - t_step
+            # Steps that need no decision (the same requests, one token each) are launched
+            # without waiting for the tokens of the step before: each feeds on them where
+            # they are, on the device, and the host reads all of them afterwards.
+            ahead = 0 if get_logits else sched.run_ahead_steps(plan, limit=64)
+            if ahead > 0:
+                single = [Scheduled(s.request, 1, True) for s in plan]
+                entries = [StepEntry(s.request.rid, [0], [0]) for s in plan]
+                run = [toks]
+                for j in range(ahead):
+                    logits = self.runner.step(entries, token_source=run[-1])
+                    run.append(self.sampler.sample_prepared(logits, prepared, j + 1))
+                decode_spans.append((after, mark(), ahead))
+                steps_ahead += ahead
+                host = torch.stack([t.view(-1) for t in run]).tolist()
+                sched.update(plan, host[0])
+                for row in host[1:]:
+                    sched.update(single, row)
+                continue
+            sched.update(plan, toks.tolist() if toks is not None else [])
         sync()
         total = time.perf_counter() - t0
+        decode_steps = sum(n for _, _, n in decode_spans)
+        decode_time = sum(seconds(a, b) for a, b, _ in decode_spans)
 
         n = max(len(r.output) for r in reqs)
         pad = self.eos_token_ids[0] if self.eos_token_ids else 0
@@ -167,12 +203,13 @@ class LLMEngine:
             "PromptLength": max(len(p) for p in ids),
             "DecodeLength": n,
             "Throughput": sum(len(r.output) for r in reqs) / total if total > 0 else 0.0,
-            "TTFT": 1e3 * (max(first_token_at.values()) - t0) if first_token_at else 0.0,
+            "TTFT": 1e3 * max(seconds(m0, m) for m in first_token_at.values()) if first_token_at else 0.0,
             "TBT": 1e3 * decode_time / decode_steps if decode_steps else 0.0,
             "E2E": 1e3 * total,
             "TokenizationTime": tokenize_ms,
             "FinishedReason": "EOS" if reasons == {"EOS"} else "Max Token Length",
             "Preemptions": sched.n_preemptions,
+            "StepsLaunchedAhead": steps_ahead,
         }
         if report_throughput:
             # the line of yalis/engine.py:558-568

@@ -175,10 +175,19 @@ class ModelRunner:
 
     # --------------------------------------------------------------------- step
     @torch.inference_mode()
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], token_source: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Run the entries as one batch.  Pages for the new tokens must have been
         reserved.  Returns float32 logits [sum of wanted places, vocab], in the
-        order of the entries and of their ``want``."""
+        order of the entries and of their ``want``.
+
+        ``token_source``: for a step of single tokens, an int32 tensor on the engine's device
+        with one token per entry that replaces the entries' own (the tokens an earlier step
+        sampled, not yet copied to the host: the step can be launched without waiting)."""
+        if token_source is not None:
+            if any(len(e.tokens) != 1 for e in entries):
+                raise ValueError("tokens from the device are for steps of single tokens")
+            if token_source.dtype != torch.int32 or token_source.numel() != len(entries):
+                raise ValueError("token_source must hold one int32 token per entry")
         spans = []
         seen = set()
         for e in entries:
@@ -207,11 +216,14 @@ class ModelRunner:
             )
         decode_only = all(len(s.tokens) == 1 and len(s.want) == 1 for s in spans)
         if self.use_graphs and decode_only and len(spans) <= GRAPH_MAX_SEQS:
-            logits = self._graph_step(spans)
+            logits = self._graph_step(spans, token_source)
         else:
             hb = build_host_batch(spans, len(self.group_shapes), self.page_size)
             buf, layout = pack(named_arrays(hb, self.builders))
             dev = self._uploader.upload(buf)
+            if token_source is not None:
+                off = layout["token_ids"][0]
+                dev[off : off + len(spans)].copy_(token_source.view(-1))
             ctx = StepContext(hb, self._views(dev, layout), self.sites, self.rt)
             self.last_host_batch = hb
             logits = self.model.forward(ctx)
@@ -227,7 +239,7 @@ class ModelRunner:
             for name, (off, shape) in layout.items()
         }
 
-    def _graph_step(self, spans) -> torch.Tensor:
+    def _graph_step(self, spans, token_source: Optional[torch.Tensor] = None) -> torch.Tensor:
         """A step of single tokens through a captured graph.  The graph is keyed by what
         fixes its launches: the number of requests and the power-of-two bucket of the
         longest context (it decides how far attention splits the keys).  Block tables
@@ -244,6 +256,9 @@ class ModelRunner:
         if entry is None:
             ints = torch.empty(buf.size, dtype=torch.int32, device=self.config.device)
             ints.copy_(self._uploader.upload(buf))
+            if token_source is not None:
+                off = layout["token_ids"][0]
+                ints[off : off + len(spans)].copy_(token_source.view(-1))
             ctx = StepContext(hb, self._views(ints, layout), self.sites, self.rt)
             ops = self.rt.ops
             ops.reserve_workspaces(hb.n_seqs)
@@ -257,6 +272,9 @@ class ModelRunner:
             if layout != entry.layout:
                 raise RuntimeError("a decode step's integer arrays changed shape under a captured graph")
             entry.ints.copy_(self._uploader.upload(buf), non_blocking=True)
+            if token_source is not None:
+                off = layout["token_ids"][0]
+                entry.ints[off : off + len(spans)].copy_(token_source.view(-1))
         entry.graph.replay()
         self.graph_replays += 1
         return entry.logits

@@ -52,29 +52,30 @@ class Sampler:
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], draws: Sequence[int]) -> List[int]:
         """logits: float32 [rows, vocab]; one SamplingParams and one draw number (how
         many tokens the request has sampled so far) per row.  Returns token ids."""
-        rows = logits.shape[0]
-        if rows != len(params) or rows != len(draws):
-            raise ValueError("one SamplingParams and one draw number per row of logits")
-        if rows == 0:
+        if logits.shape[0] == 0:
             return []
+        return self.sample_prepared(logits, self.prepare(params, draws), 0).tolist()
+
+    def prepare(self, params: Sequence[SamplingParams], draws: Sequence[int]):
+        """What ``sample_prepared`` needs on the device for these rows: None when every row is
+        greedy, else (temperature, top_k, top_p, seeds, draws) tensors.  Made once for a run
+        of steps over the same requests."""
+        if len(params) != len(draws):
+            raise ValueError("one SamplingParams and one draw number per row of logits")
         if all(p.greedy for p in params):
-            return self.ops.argmax(logits).tolist()
-        host = torch.tensor(
-            [
-                [p.temperature for p in params],
-                [p.top_p for p in params],
-            ],
-            dtype=torch.float32,
-        )
+            return None
+        floats = torch.tensor([[p.temperature for p in params], [p.top_p for p in params]], dtype=torch.float32).to(self.device)
         ints = torch.tensor(
-            [
-                [p.top_k or 0 for p in params],
-                [p.seed & 0x7FFFFFFF for p in params],
-                list(draws),
-            ],
-            dtype=torch.int32,
-        )
-        host = host.to(self.device)
-        ints = ints.to(self.device)
-        out = self.ops.sample(logits, host[0].contiguous(), ints[0].contiguous(), host[1].contiguous(), ints[1].contiguous(), ints[2].contiguous())
-        return out.tolist()
+            [[p.top_k or 0 for p in params], [p.seed & 0x7FFFFFFF for p in params], list(draws)], dtype=torch.int32
+        ).to(self.device)
+        return floats[0].contiguous(), ints[0].contiguous(), floats[1].contiguous(), ints[1].contiguous(), ints[2].contiguous()
+
+    def sample_prepared(self, logits: torch.Tensor, prepared, step: int) -> torch.Tensor:
+        """Token ids (int32, on the device) for rows prepared with ``prepare``; ``step`` is
+        added to every row's draw number (the step within a run that shares one preparation)."""
+        if prepared is None:
+            return self.ops.argmax(logits)
+        temperature, top_k, top_p, seeds, draws = prepared
+        if logits.shape[0] != draws.numel():
+            raise ValueError("one SamplingParams and one draw number per row of logits")
+        return self.ops.sample(logits, temperature, top_k, top_p, seeds, draws + step if step else draws)
