@@ -56,6 +56,7 @@ def main() -> int:
     ap.add_argument("--prefill-len", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--only-prefill", action="store_true", help="measure the prefill only (for profiling)")
+    ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel (for hardware counters)")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="8b", help="layer sizes (default: the 8B shape of the headline)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -86,6 +87,7 @@ def main() -> int:
         max_model_len=min(cfg["max_position_embeddings"], pages_per_req * page),
         max_num_batched_tokens=8192,
         dtype="bfloat16",
+        decode_graphs=not args.no_graphs,
     )
     runner = random_runner(cfg, engine, seed=0)
     ops = runner.rt.ops
