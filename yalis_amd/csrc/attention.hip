@@ -270,19 +270,20 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
       for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          if (whole) {
-            s[u][sb][i] *= scale_log2;
-          } else {
+          if (!whole) {
             const int key = kb * 64 + 32 * u + 8 * gq + 4 * sb + i;
             const bool ok = col_ok && key <= pos_c && key >= lo_c;
-            s[u][sb][i] = ok ? s[u][sb][i] * scale_log2 : -INFINITY;
+            if (!ok) s[u][sb][i] = -INFINITY;
           }
           tmax = fmaxf(tmax, s[u][sb][i]);
         }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float m_new = fmaxf(m, tmax);
+    // the maximum was taken over the raw scores (the scale is positive); the scale joins the
+    // subtraction of the maximum in one fused multiply-add
+    const float m_new = fmaxf(m, tmax * scale_log2);
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const bool grew = __any(m_new > m);  // only then the running sums need rescaling
     const float alpha = fast_exp2(m - m_safe);
     float psum = 0.f;
     AFrag8 pf[2];
@@ -292,7 +293,7 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
       for (int sb = 0; sb < 2; ++sb) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          s[u][sb][i] = fast_exp2(s[u][sb][i] - m_safe);
+          s[u][sb][i] = fast_exp2(fmaf(s[u][sb][i], scale_log2, -m_safe));
           psum += s[u][sb][i];
         }
         pf[u].u[2 * sb] = pack_bf16x2(s[u][sb][0], s[u][sb][1]);
@@ -301,8 +302,10 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
     }
     l = l * alpha + psum;
     m = m_new;
+    if (grew) {
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) acc[dt] *= alpha;
+      for (int dt = 0; dt < DT; ++dt) acc[dt] *= alpha;
+    }
     // values of keys that do not exist yet may be anything: zero them (last block only)
     if (kb * 64 + 64 > hi) {
 #pragma unroll
@@ -565,8 +568,11 @@ __global__ __launch_bounds__(256, 3) void attn_mfma_prefill_kernel(
     const bool whole = kb * 64 + 63 <= (tile_pos0 + wave_tok0) && (window == 0 || kb * 64 >= max(0, wave_hi - window));
     AFrag8 pf[CT][2];
     float alpha[CT];
+    bool grew = false;  // some column's maximum rose: only then the running sums need rescaling
 #pragma unroll
     for (int c = 0; c < CT; ++c) {
+      // the maximum is taken over the raw scores (the scale is positive), and the scale
+      // joins the subtraction of the maximum in one fused multiply-add
       float tmax = -INFINITY;
 #pragma unroll
       for (int u = 0; u < 2; ++u)
@@ -574,19 +580,18 @@ __global__ __launch_bounds__(256, 3) void attn_mfma_prefill_kernel(
         for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            if (whole) {
-              s[c][u][sb][i] *= scale_log2;
-            } else {
+            if (!whole) {
               const int key = kb * 64 + 32 * u + 8 * gq + 4 * sb + i;
               const bool ok = col_ok[c] && key <= pos_c[c] && key >= lo_c[c];
-              s[c][u][sb][i] = ok ? s[c][u][sb][i] * scale_log2 : -INFINITY;
+              if (!ok) s[c][u][sb][i] = -INFINITY;
             }
             tmax = fmaxf(tmax, s[c][u][sb][i]);
           }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      const float m_new = fmaxf(m[c], tmax);
+      const float m_new = fmaxf(m[c], tmax * scale_log2);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      grew = grew || m_new > m[c];
       alpha[c] = fast_exp2(m[c] - m_safe);
       float psum = 0.f;
 #pragma unroll
@@ -595,7 +600,7 @@ __global__ __launch_bounds__(256, 3) void attn_mfma_prefill_kernel(
         for (int sb = 0; sb < 2; ++sb) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            s[c][u][sb][i] = fast_exp2(s[c][u][sb][i] - m_safe);
+            s[c][u][sb][i] = fast_exp2(fmaf(s[c][u][sb][i], scale_log2, -m_safe));
             psum += s[c][u][sb][i];
           }
           pf[c][u].u[2 * sb] = pack_bf16x2(s[c][u][sb][0], s[c][u][sb][1]);
@@ -604,10 +609,13 @@ __global__ __launch_bounds__(256, 3) void attn_mfma_prefill_kernel(
       l[c] = l[c] * alpha[c] + psum;
       m[c] = m_new;
     }
+    grew = __any(grew);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
+      if (grew) {
 #pragma unroll
-      for (int c = 0; c < CT; ++c) acc[c][dt] *= alpha[c];
+        for (int c = 0; c < CT; ++c) acc[c][dt] *= alpha[c];
+      }
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         AFrag8 a;
@@ -714,6 +722,7 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
   YK_REQUIRE(reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0,
              "attn_mfma_prefill: cache must be 16-byte aligned");
   YK_REQUIRE(window >= 0 && table_width > 0, "attn_mfma_prefill: bad window or table");
+  YK_REQUIRE(scale > 0.f, "attn_mfma_prefill: the score scale must be positive");
   if (n_tiles == 0) return 0;
   const int hpt = yk_attn_heads_per_tile(n_heads, n_kv);
   const int chunks = (n_heads / n_kv + hpt - 1) / hpt;
@@ -751,6 +760,7 @@ extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* 
              "attn_mfma: cache must be 16-byte aligned");
   YK_REQUIRE(n_splits >= 1 && n_splits <= 65535, "attn_mfma: bad split count");
   YK_REQUIRE(window >= 0 && table_width > 0, "attn_mfma: bad window or table");
+  YK_REQUIRE(scale > 0.f, "attn_mfma: the score scale must be positive");
   if (n_tiles == 0) return 0;
   const int hpt = yk_attn_heads_per_tile(n_heads, n_kv);
   const int chunks = (n_heads / n_kv + hpt - 1) / hpt;
