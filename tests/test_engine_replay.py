@@ -19,8 +19,9 @@ BACKENDS = [
 ]
 
 # prompt lengths of the brief's two tiny configurations, and own ones for C and D
-LENGTHS = {"A": [5, 17, 32, 61, 77, 40], "B": [1, 40, 130, 66, 25, 90], "C": [50, 3, 97, 140, 64, 31], "D": [33, 129, 70, 2, 65]}
-PAGE = {"A": 16, "B": 32, "C": 16, "D": 64}
+LENGTHS = {"A": [5, 17, 32, 61, 77, 40], "B": [1, 40, 130, 66, 25, 90], "C": [50, 3, 97, 140, 64, 31], "D": [33, 129, 70, 2, 65],
+           "E": [44, 9, 120, 71, 36]}
+PAGE = {"A": 16, "B": 32, "C": 16, "D": 64, "E": 48}
 
 _ops_cache = {}
 
@@ -40,7 +41,7 @@ _plain_cache = {}
 
 def setup(name, dtype):
     cfg = ALL[name]
-    weights = P.random_weights(cfg, seed={"A": 0, "B": 1, "C": 2, "D": 3}[name])
+    weights = P.random_weights(cfg, seed={"A": 0, "B": 1, "C": 2, "D": 3, "E": 4}[name])
     reqs = C.make_requests(cfg, LENGTHS[name], seed=10)
     key = (name, dtype == "bfloat16")
     if key not in _plain_cache:
@@ -49,7 +50,7 @@ def setup(name, dtype):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 @pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
 def test_replay_modes(backend, name, mode):
     device, dtype = backend

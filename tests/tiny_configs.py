@@ -86,4 +86,31 @@ TINY_D = {
     "tie_word_embeddings": True,
 }
 
-ALL = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+# Sizes that meet none of the fast paths: a head size the matrix-core attention does not take
+# (48), three query heads on one kv head, a hidden size that differs from heads x head size,
+# widths that are no multiples of 8 (no 16-byte rows: the few-row matrix-core product and the
+# packed gate/up layout do not apply), one layer, an odd vocabulary.
+TINY_E = {
+    "architectures": ["LlamaForCausalLM"],
+    "model_type": "llama",
+    "hidden_size": 100,
+    "num_hidden_layers": 1,
+    "num_attention_heads": 3,
+    "num_key_value_heads": 1,
+    "head_dim": 48,
+    "intermediate_size": 90,
+    "vocab_size": 1001,
+    "rms_norm_eps": 3e-6,
+    "rope_theta": 25000.0,
+    "rope_scaling": {
+        "rope_type": "llama3",
+        "factor": 4.0,
+        "low_freq_factor": 1.0,
+        "high_freq_factor": 2.0,
+        "original_max_position_embeddings": 32,
+    },
+    "max_position_embeddings": 192,
+    "tie_word_embeddings": True,
+}
+
+ALL = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
