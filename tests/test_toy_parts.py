@@ -1,8 +1,9 @@
 """Generality of the framework, shown with toy parts defined here, without a change to
-the framework's files: a mixer with per-request state of its own, an architecture
-registered from outside, a run order that names a layer twice and lets an entry read
-another entry's cache, and layers with a window beside layers without (two cache groups,
-pages given back while the request is live).  The toy model is nobody's architecture.
+the framework's files: a mixer with per-request state of its own, a feed-forward that
+routes every token to one of several experts, a position encoding with angles of its own,
+an architecture registered from outside, a run order that names a layer twice and lets an
+entry read another entry's cache, and layers with a window beside layers without (two cache
+groups, pages given back while the request is live).  The toy model is nobody's architecture.
 """
 import math
 
@@ -18,7 +19,7 @@ from yalis_amd.config.runtime import EngineConfig
 from yalis_amd.config.specs import LayerSpec, ModelSpec, PartSpec, RunEntry
 from yalis_amd.engine.factory import build_model, tensor_specs_for
 from yalis_amd.engine.step import ModelRunner
-from yalis_amd.parts import Mixer, StateNeed, register_mixer
+from yalis_amd.parts import FeedForward, Mixer, Position, StateNeed, register_feed_forward, register_mixer, register_position
 from yalis_amd.weights.loader import TensorSpec
 from yalis_amd.weights.random_init import random_tensors
 
@@ -65,6 +66,62 @@ class RunningMean(Mixer):
         return self.rt.ops.linear(out.to(self.rt.act_dtype), self.w, self.rt.act_dtype)
 
 
+# ------------------------------------------------------- a feed-forward with routing
+@register_feed_forward("toy_routed")
+class RoutedFeedForward(FeedForward):
+    """Every token goes to the one expert its router scores highest (lowest index on ties);
+    the expert's output is weighted with the router's float32 softmax probability.  An
+    expert is down(gelu(up(h))).  Tokens are gathered per expert, so each expert runs one
+    product over its own rows."""
+
+    def __init__(self, params, rt):
+        super().__init__(params, rt)
+        self.prefix, self.hidden, self.inner, self.experts = params["prefix"], params["hidden_size"], params["inner_size"], params["experts"]
+        self.router = None
+        self.up, self.down = [], []
+
+    def tensor_specs(self):
+        specs = {f"{self.prefix}.router.weight": TensorSpec((self.experts, self.hidden), "float", ("normal", 0.5))}
+        for e in range(self.experts):
+            specs[f"{self.prefix}.expert{e}.up.weight"] = TensorSpec((self.inner, self.hidden), "float", ("normal", 0.05))
+            specs[f"{self.prefix}.expert{e}.down.weight"] = TensorSpec((self.hidden, self.inner), "float", ("normal", 0.05))
+        return specs
+
+    def load(self, tensors):
+        self.router = tensors[f"{self.prefix}.router.weight"]
+        self.up = [tensors[f"{self.prefix}.expert{e}.up.weight"] for e in range(self.experts)]
+        self.down = [tensors[f"{self.prefix}.expert{e}.down.weight"] for e in range(self.experts)]
+
+    def forward(self, h, ctx):
+        ops = self.rt.ops
+        probs = torch.softmax(ops.linear(h, self.router, torch.float32), dim=-1)  # router in float32
+        weight, choice = probs.max(dim=-1)
+        out = torch.zeros(h.shape, dtype=torch.float32, device=h.device)
+        for e in range(self.experts):
+            rows = torch.nonzero(choice == e).flatten()
+            if rows.numel() == 0:
+                continue
+            a = torch.nn.functional.gelu(ops.linear(h[rows].contiguous(), self.up[e], self.rt.act_dtype).float(), approximate="tanh")
+            y = ops.linear(a.to(self.rt.act_dtype), self.down[e], self.rt.act_dtype).float()
+            out[rows] = y * weight[rows, None]
+        return out.to(self.rt.act_dtype)
+
+
+# ------------------------------------------------------ a position encoding of its own
+@register_position("toy_sqrt_rotary")
+class SqrtRotary(Position):
+    """Rotation by angles sqrt(position) * theta^(-2i/d): offers what the attention part
+    reads of a position encoding (cos, sin, rotary_dim, interleaved)."""
+
+    def __init__(self, params, rt):
+        super().__init__(params, rt)
+        self.rotary_dim = params["rotary_dim"]
+        self.interleaved = False
+        inv = 1.0 / (params["theta"] ** (torch.arange(0, self.rotary_dim, 2, dtype=torch.float32) / self.rotary_dim))
+        angle = torch.outer(torch.sqrt(torch.arange(rt.max_positions, dtype=torch.float32)), inv)
+        self.cos, self.sin = torch.cos(angle).to(rt.device), torch.sin(angle).to(rt.device)
+
+
 # ----------------------------------------------------------------- a toy architecture
 class ToyConfig:
     def __init__(self, raw):
@@ -76,6 +133,7 @@ class ToyConfig:
         self.head_dim = r.integer("head_dim")
         self.inter = r.integer("inner_size")
         self.window = r.integer("window")
+        self.experts = r.integer("experts")
         self.eps = r.number("eps")
         self.theta = r.number("theta")
         self.max_positions = r.integer("max_positions")
@@ -99,14 +157,16 @@ def build_toy_spec(c: ToyConfig) -> ModelSpec:
     def ffn(prefix):
         return PartSpec("gated_mlp", {"prefix": prefix, "hidden_size": c.hidden, "intermediate_size": c.inter, "activation": "gelu_tanh"})
 
-    def layer(i, mixer):
+    def layer(i, mixer, feed_forward=None):
         p = f"toy.{i}"
-        return LayerSpec(p, "prenorm", mixer, ffn(p + ".ff"), norm(p + ".n1"), norm(p + ".n2"))
+        return LayerSpec(p, "prenorm", mixer, feed_forward or ffn(p + ".ff"), norm(p + ".n1"), norm(p + ".n2"))
 
+    routed = PartSpec("toy_routed", {"prefix": "toy.1.ff", "hidden_size": c.hidden, "inner_size": c.inter // 2, "experts": c.experts})
+    sqrt_rotary = PartSpec("toy_sqrt_rotary", {"rotary_dim": c.head_dim, "theta": c.theta})
     layers = (
         layer(0, attn("toy.0.att", None, rotary)),  # all keys, partial interleaved rotary
-        layer(1, PartSpec("toy_running_mean", {"prefix": "toy.1", "hidden_size": c.hidden})),
-        layer(2, attn("toy.2.att", c.window, rotary)),  # a window: its own cache group
+        layer(1, PartSpec("toy_running_mean", {"prefix": "toy.1", "hidden_size": c.hidden}), routed),
+        layer(2, attn("toy.2.att", c.window, sqrt_rotary)),  # a window: its own cache group; its own positions
         layer(3, attn("toy.3.att", None, None)),  # no position encoding; only ever borrows a cache
     )
     run_order = (
@@ -128,7 +188,7 @@ def build_toy_spec(c: ToyConfig) -> ModelSpec:
 register_architecture("ToyForCausalLM", ToyConfig, build_toy_spec)
 
 TOY = {"architectures": ["ToyForCausalLM"], "hidden_size": 96, "vocab_size": 131, "heads": 4, "kv_heads": 2, "head_dim": 32,
-       "inner_size": 136, "window": 24, "eps": 1e-5, "theta": 1000.0, "max_positions": 256}
+       "inner_size": 136, "window": 24, "experts": 3, "eps": 1e-5, "theta": 1000.0, "max_positions": 256}
 
 
 # ------------------------------------------------- the toy model, plainly and whole
@@ -152,6 +212,25 @@ def toy_plain(weights, tokens, rounder=P._identity):
         out[..., 1:rd:2] = b * cos[:, None, :] + a * sin[:, None, :]
         return out
 
+    sq_inv = 1.0 / (c.theta ** (torch.arange(0, c.head_dim, 2, dtype=torch.float32) / c.head_dim))
+    sq_angle = torch.outer(torch.sqrt(pos.float()), sq_inv)
+    sq_cos, sq_sin = torch.cos(sq_angle), torch.sin(sq_angle)
+
+    def rope_sqrt_half(v):
+        half = c.head_dim // 2
+        a, b = v[..., :half], v[..., half:]
+        return torch.cat([a * sq_cos[:, None, :] - b * sq_sin[:, None, :], b * sq_cos[:, None, :] + a * sq_sin[:, None, :]], dim=-1)
+
+    def routed(h, p):
+        probs = torch.softmax(h @ w(p + ".router.weight").T, dim=-1)
+        weight, choice = probs.max(dim=-1)
+        out = torch.zeros_like(h)
+        for tok in range(t):
+            e = int(choice[tok])
+            a = torch.nn.functional.gelu(rounder(h[tok] @ w(f"{p}.expert{e}.up.weight").T), approximate="tanh")
+            out[tok] = rounder(rounder(a) @ w(f"{p}.expert{e}.down.weight").T) * weight[tok]
+        return rounder(out)
+
     def ffn(h, p):
         g = rounder(h @ w(p + ".gate_proj.weight").T)
         u = rounder(h @ w(p + ".up_proj.weight").T)
@@ -164,10 +243,10 @@ def toy_plain(weights, tokens, rounder=P._identity):
             k = rounder(h @ w(p + ".k_proj.weight").T).view(t, c.kv_heads, c.head_dim)
             v = rounder(h @ w(p + ".v_proj.weight").T).view(t, c.kv_heads, c.head_dim)
             if rotate:
-                k = rounder(rope_interleaved_partial(k))
+                k = rounder(rotate(k))
             kv = (k, v)
         if rotate:
-            q = rounder(rope_interleaved_partial(q))
+            q = rounder(rotate(q))
         a = P.causal_attention(q, kv[0], kv[1], 1.0 / math.sqrt(c.head_dim), pos, pos, window, round_p=rounder)
         return rounder(rounder(a).reshape(t, -1) @ w(p + ".o_proj.weight").T), kv
 
@@ -182,13 +261,13 @@ def toy_plain(weights, tokens, rounder=P._identity):
         if layer == 1:
             a = running_mean(h, p)
         elif layer == 3:
-            a, _ = attention(h, p + ".att", None, False, kv=first_cache)
+            a, _ = attention(h, p + ".att", None, None, kv=first_cache)
         else:
-            a, kv = attention(h, p + ".att", c.window if layer == 2 else None, True)
+            a, kv = attention(h, p + ".att", c.window if layer == 2 else None, rope_sqrt_half if layer == 2 else rope_interleaved_partial)
             if first_cache is None:
                 first_cache = kv
         x = x + a
-        x = x + ffn(norm(x, p + ".n2"), p + ".ff")
+        x = x + (routed if layer == 1 else ffn)(norm(x, p + ".n2"), p + ".ff")
     return norm(x, "toy.final") @ w("toy.head").T
 
 
