@@ -228,3 +228,10 @@ def test_tensors_are_made_when_a_part_asks(tmp_path):
     write_dict(os.path.join(bad, "model.safetensors"), t)
     with pytest.raises(WeightsError, match="model.norm.weight"):
         load_runner(bad, eng, ops=RefOps())
+
+
+def test_graphs_switch_follows_the_reference(monkeypatch):
+    monkeypatch.delenv("YALIS_DISABLE_DECODE_CUDAGRAPHS", raising=False)
+    assert EngineConfig().decode_graphs
+    monkeypatch.setenv("YALIS_DISABLE_DECODE_CUDAGRAPHS", "1")
+    assert not EngineConfig().decode_graphs and EngineConfig(decode_graphs=True).decode_graphs

@@ -10,7 +10,7 @@ adds: page size, page count, the per-step token budget.
 from __future__ import annotations
 
 import os
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Optional, Tuple
 
 _PRECISIONS = {
@@ -144,7 +144,9 @@ class EngineConfig:
     max_num_batched_tokens: int = 2048
     dtype: str = "bfloat16"
     device: str = "cuda:0"
-    decode_graphs: bool = True  # capture steps of single tokens as HIP graphs
+    # capture steps of single tokens as HIP graphs; YALIS_DISABLE_DECODE_CUDAGRAPHS=1 turns the
+    # default off, as it does in the reference
+    decode_graphs: bool = field(default_factory=lambda: os.environ.get("YALIS_DISABLE_DECODE_CUDAGRAPHS", "0") != "1")
 
     def __post_init__(self) -> None:
         self.dtype = canonical_dtype(self.dtype)
