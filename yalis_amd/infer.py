@@ -32,6 +32,8 @@ def parse_args(argv=None):
     ap.add_argument("--prompt", action="append", default=[], help="a text prompt (repeatable; needs a tokenizer)")
     ap.add_argument("--prompt-ids", action="append", default=[], help="a prompt as comma-separated token ids (repeatable)")
     ap.add_argument("--random-prompts", default=None, metavar="N,LEN", help="N prompts of LEN seeded random token ids")
+    ap.add_argument("--chat", action="store_true", help="wrap text prompts in the tokenizer's chat template (examples/infer.py:50-62 of the reference does)")
+    ap.add_argument("--system-prompt", default=None, help="system message for --chat")
     ap.add_argument("--prompt-file", default=None, help="a file with one prompt a line: text, or comma-separated token ids")
     ap.add_argument("--tokens-to-generate", "--max-tokens", dest="tokens_to_generate", type=int, default=50)
     ap.add_argument("--max-batch-size", "--max-num-seqs", dest="max_batch_size", type=int, default=32)
@@ -94,6 +96,14 @@ def main(argv=None) -> int:
         prompts = list(args.prompt)
     else:
         prompts = DEFAULT_PROMPTS[: args.max_batch_size]
+    if args.chat and prompts and isinstance(prompts[0], str):
+        if engine.tokenizer is None or not getattr(engine.tokenizer, "chat_template", None):
+            raise SystemExit("--chat needs a tokenizer with a chat template in the model folder")
+        wrapped = []
+        for p in prompts:
+            conversation = ([{"role": "system", "content": args.system_prompt}] if args.system_prompt else []) + [{"role": "user", "content": p}]
+            wrapped.append(engine.tokenizer.apply_chat_template(conversation, add_generation_prompt=True, tokenize=False))
+        prompts = wrapped
     print_rank0(f"Number of prompts = {len(prompts)}")
 
     for _ in range(args.iters):
