@@ -220,3 +220,30 @@ def test_command_line(tmp_path):
         outs = [ast.literal_eval(ln.split("=", 1)[1].strip()) for ln in run.stdout.splitlines() if ln.startswith("output =")]
         assert outs == [P.greedy_generate(cfg, weights, p, 8) for p in prompts]
         assert "metrics = " in run.stdout and "Number of prompts = 2" in run.stdout
+
+
+def test_text_prompts_through_a_tokenizer(tmp_path):
+    """A folder with a tokenizer takes text prompts (the reference always tokenizes,
+    yalis/engine.py:306-341): a small word-level tokenizer made here, the CPU backend."""
+    tokenizers = pytest.importorskip("tokenizers")
+    pytest.importorskip("transformers")
+    cfg = ALL["A"]
+    words = ["<unk>", "<eos>"] + [f"w{i}" for i in range(200)]
+    tok = tokenizers.Tokenizer(tokenizers.models.WordLevel({w: i for i, w in enumerate(words)}, unk_token="<unk>"))
+    tok.pre_tokenizer = tokenizers.pre_tokenizers.Whitespace()
+    eng, cfg, weights = make_engine(tmp_path, "A", ("cpu", "fp32"), 2, temperature=0.0, page_size=16, num_pages=16)
+    folder = str(tmp_path / "A")
+    tok.save(os.path.join(folder, "tokenizer.json"))
+    with open(os.path.join(folder, "tokenizer_config.json"), "w") as f:
+        json.dump({"tokenizer_class": "PreTrainedTokenizerFast", "unk_token": "<unk>", "eos_token": "<eos>"}, f)
+    eng = LLMEngine(ModelConfig(model_path=folder, precision="fp32"),
+                    InferenceConfig(max_batch_size=2, max_length_of_generated_sequences=64, temperature=0.0),
+                    device="cpu", engine_config=eng.engine_config, ops=RefOps())
+    assert eng.tokenizer is not None
+    texts = ["w5 w17 w3 w150", "w9 nothing w44"]
+    ids = [[7, 19, 5, 152], [11, 0, 46]]
+    assert eng._tokenize_prompts(texts) == ids
+    out, metrics = eng.generate(texts, tokens_to_generate=5)
+    assert out.tolist() == [P.greedy_generate(cfg, weights, p, 5) for p in ids]
+    assert metrics["TokenizationTime"] >= 0.0 and metrics["PromptLength"] == 4
+    assert len(eng.tokenizer.batch_decode(out, skip_special_tokens=True)) == 2
