@@ -247,3 +247,26 @@ def test_text_prompts_through_a_tokenizer(tmp_path):
     assert out.tolist() == [P.greedy_generate(cfg, weights, p, 5) for p in ids]
     assert metrics["TokenizationTime"] >= 0.0 and metrics["PromptLength"] == 4
     assert len(eng.tokenizer.batch_decode(out, skip_special_tokens=True)) == 2
+
+
+@pytest.mark.parametrize("backend", BACKENDS[:2])
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_more_requests_than_slots_and_a_small_pool(tmp_path, backend, seed):
+    """Ten requests of random lengths through three slots and a pool that holds about one and a half of
+    them: requests wait, are admitted in portions and, with some seeds, preempted and
+    recomputed; every request's greedy tokens are the plain implementation's."""
+    g = torch.Generator().manual_seed(seed)
+    lengths = torch.randint(1, 70, (10,), generator=g).tolist()
+    eng, cfg, weights = make_engine(tmp_path, "A", backend, 10, temperature=0.0,
+                                    page_size=16, num_pages=8, max_num_batched_tokens=40)
+    eng.engine_config.max_num_seqs = 3
+    eng2 = LLMEngine(eng.model_config, eng.inference_config, device=backend[0],
+                     engine_config=EngineConfig(page_size=16, num_pages=8, max_num_seqs=3, max_model_len=cfg["max_position_embeddings"],
+                                                max_num_batched_tokens=40, dtype="float32", device=backend[0]),
+                     ops=RefOps() if backend[0] == "cpu" else None)
+    prompts = prompts_for(cfg, lengths, seed=seed)
+    out, metrics = eng2.generate(prompts, tokens_to_generate=12)
+    for p, row in zip(prompts, out.tolist()):
+        assert row == P.greedy_generate(cfg, weights, p, 12)
+    eng2.runner.pages.audit()
+    assert eng2.runner.pages.live_requests() == 0 and eng2.runner.pages.free_pages(0) == 8
