@@ -342,17 +342,33 @@ __global__ void rope_append_kernel(const TS* src, int n_splits, size_t split_str
   const float* cs = cos_t ? cos_t + static_cast<size_t>(pos) * half : nullptr;
   const float* sn = sin_t ? sin_t + static_cast<size_t>(pos) * half : nullptr;
   const TS* row = src + static_cast<size_t>(n) * src_stride;
-  auto value = [&](int idx) {
-    float a = 0.f;
-    for (int s0 = 0; s0 < n_splits; s0 += 4) {  // four slices in flight, see add_rmsnorm
-      float d[4];
+  // Two elements at once (a rotary pair, or two value elements): up to eight slices of both
+  // are in flight before the first is added; a slice index beyond the last is clamped and
+  // its value dropped, so that the loads carry no condition.  Slices are added in order.
+  auto value2 = [&](int idx_a, int idx_b, float& out_a, float& out_b) {
+    float a = 0.f, b = 0.f;
+    for (int s0 = 0; s0 < n_splits; s0 += 8) {
+      float da[8], db[8];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) d[j] = to_f32<TS>(row[static_cast<size_t>(min(s0 + j, n_splits - 1)) * split_stride + idx]);
+      for (int j = 0; j < 8; ++j) {
+        const size_t off = static_cast<size_t>(min(s0 + j, n_splits - 1)) * split_stride;
+        da[j] = to_f32<TS>(row[off + idx_a]);
+        db[j] = to_f32<TS>(row[off + idx_b]);
+      }
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (s0 + j < n_splits) a += d[j];
+      for (int j = 0; j < 8; ++j)
+        if (s0 + j < n_splits) {
+          a += da[j];
+          b += db[j];
+        }
     }
-    return as_output(a, round_sum);
+    out_a = as_output(a, round_sum);
+    out_b = as_output(b, round_sum);
+  };
+  auto value = [&](int idx) {
+    float a, b;
+    value2(idx, idx, a, b);
+    return a;
   };
   const bool is_q = h < n_heads;
   T* dst;
@@ -367,14 +383,20 @@ __global__ void rope_append_kernel(const TS* src, int n_splits, size_t split_str
     // the value head of the same group, transposed
     T* vdst = v_cache + (page * n_kv + g) * head_dim * page_size + off;
     const int vbase = (n_heads + n_kv + g) * head_dim;
-    for (int d = threadIdx.x; d < head_dim; d += blockDim.x)
-      vdst[static_cast<size_t>(d) * page_size] = from_f32<T>(value(vbase + d));
+    for (int d = threadIdx.x; d < head_dim; d += 2 * blockDim.x) {
+      const int d2 = d + blockDim.x;  // this thread's second element, when there is one
+      float va, vb;
+      value2(vbase + d, vbase + min(d2, head_dim - 1), va, vb);
+      vdst[static_cast<size_t>(d) * page_size] = from_f32<T>(va);
+      if (d2 < head_dim) vdst[static_cast<size_t>(d2) * page_size] = from_f32<T>(vb);
+    }
   }
   const int base = h * head_dim;
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
     const int ia = interleaved ? 2 * i : i;
     const int ib = interleaved ? 2 * i + 1 : i + half;
-    const float a = value(base + ia), b = value(base + ib);
+    float a, b;
+    value2(base + ia, base + ib, a, b);
     const float c = cs[i], s = sn[i];
     dst[ia] = from_f32<T>(rot_first(a, b, c, s));
     dst[ib] = from_f32<T>(rot_second(a, b, c, s));
