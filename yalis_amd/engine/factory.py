@@ -6,8 +6,7 @@ the registry, describe it as parts, build the parts, load their tensors by name.
 """
 from __future__ import annotations
 
-import sys
-from typing import Dict, Optional, Tuple
+from typing import Dict
 
 import torch
 

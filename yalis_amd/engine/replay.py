@@ -16,7 +16,6 @@ import os
 import sys
 from typing import Dict, Iterable, List, Optional
 
-import numpy as np
 import torch
 
 from .step import ModelRunner, StepEntry

@@ -18,7 +18,7 @@ import sys
 import tempfile
 import threading
 import time
-from typing import Dict, List, Optional, Sequence
+from typing import Dict, List, Sequence
 
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 
