@@ -99,12 +99,14 @@ def test_greedy_matches_plain(tmp_path, backend, engine_kw):
 
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("temperature,top_k,top_p", [(0.0, None, 1.0), (0.9, 12, 0.8)])
-def test_steps_launched_ahead_change_nothing(tmp_path, backend, temperature, top_k, top_p):
+@pytest.mark.parametrize("budget", [64, 16])
+def test_steps_launched_ahead_change_nothing(tmp_path, backend, temperature, top_k, top_p, budget):
     """Decode steps that need no decision are launched without waiting for the tokens of the
     step before; asking for the logits switches that off.  Both ways give the same tokens,
-    also when requests have different lengths to go and finish at different steps."""
+    also when requests start decoding at different steps (a small token budget cuts the
+    prompts into portions) and so drop out of the run one after the other."""
     eng, cfg, _ = make_engine(tmp_path, "C", backend, 3, temperature=temperature, top_k=top_k, top_p=top_p,
-                              page_size=16, num_pages=40, max_num_batched_tokens=64)
+                              page_size=16, num_pages=40, max_num_batched_tokens=budget)
     prompts = prompts_for(cfg, [7, 40, 21], seed=31)
     ahead, m1 = eng.generate(prompts, tokens_to_generate=20)
     plain, m2, _ = eng.generate(prompts, tokens_to_generate=20, get_logits=True)

@@ -135,12 +135,13 @@ def test_steps_that_need_no_decision():
     plan = sched.schedule()
     for s in plan:
         runner.cached[s.request.rid] += s.n_tokens
-    # both prompts whole, both sample: b needs 4 more tokens after this step's, a needs 8
+    # both prompts whole, both sample: b needs 4 more tokens after this step's, a needs 8;
+    # b drops out after its four steps, a goes on alone
     assert [s.samples for s in plan] == [True, True]
-    assert sched.run_ahead_steps(plan) == 4
     assert sched.run_ahead_steps(plan, limit=3) == 3
-    # pages for those steps are there: 10 + 4 and 30 + 4 tokens
-    assert runner.pages.reserve(a.rid, 14) and runner.pages.reserve(b.rid, 34)
+    assert sched.run_ahead_steps(plan) == 8
+    # pages for those steps are there: 10 + 8 and 30 + 4 tokens
+    assert runner.pages.reserve(a.rid, 18) and runner.pages.reserve(b.rid, 34)
     sched.update(plan, [1, 1])
     # a third request waits: the next step must admit it, nothing runs ahead
     sched.add([1, 2, 3], SamplingParams(temperature=0.0, max_tokens=4))

@@ -125,6 +125,8 @@ def named_arrays(hb: HostBatch, builders: Dict[str, Callable[[HostBatch], np.nda
         out[f"slots_g{g}"] = sl
     for name, fn in builders.items():
         out[name] = np.ascontiguousarray(fn(hb), dtype=np.int32)
+    for name, a in hb.extra.items():
+        out[name] = np.ascontiguousarray(a, dtype=np.int32)
     return out
 
 

@@ -173,18 +173,34 @@ class LLMEngine:
             # they are, on the device, and the host reads all of them afterwards.
             ahead = 0 if get_logits else sched.run_ahead_steps(plan, limit=64)
             if ahead > 0:
-                single = [Scheduled(s.request, 1, True) for s in plan]
-                entries = [StepEntry(s.request.rid, [0], [0]) for s in plan]
-                run = [toks]
+                # tokens each request has once this step is accounted for
+                have = {s.request.rid: len(s.request.output) + 1 for s in plan}
+                rows = [s.request for s in plan]  # the requests of the last launched step, in its order
+                run, plans = [toks], []
                 for j in range(ahead):
-                    logits = self.runner.step(entries, token_source=run[-1])
+                    cur = [r for r in rows if have[r.rid] < r.params.max_tokens]
+                    if not cur:
+                        break
+                    index = [rows.index(r) for r in cur]
+                    moved = index != list(range(len(rows)))
+                    logits = self.runner.step([StepEntry(r.rid, [0], [0]) for r in cur], token_source=run[-1],
+                                              token_index=index if moved else None)
+                    if moved and prepared is not None:
+                        where = torch.tensor(index, dtype=torch.int32).to(self.engine_config.device, non_blocking=True)
+                        prepared = self.sampler.narrow(prepared, where)
                     run.append(self.sampler.sample_prepared(logits, prepared, j + 1))
-                decode_spans.append((after, mark(), ahead))
-                steps_ahead += ahead
-                host = torch.stack([t.view(-1) for t in run]).tolist()
-                sched.update(plan, host[0])
-                for row in host[1:]:
-                    sched.update(single, row)
+                    plans.append([Scheduled(r, 1, True) for r in cur])
+                    for r in cur:
+                        have[r.rid] += 1
+                    rows = cur
+                decode_spans.append((after, mark(), len(plans)))
+                steps_ahead += len(plans)
+                flat = torch.cat([t.view(-1) for t in run]).tolist()
+                sched.update(plan, flat[: len(plan)])
+                at = len(plan)
+                for p in plans:
+                    sched.update(p, flat[at : at + len(p)])
+                    at += len(p)
                 continue
             sched.update(plan, toks.tolist() if toks is not None else [])
         sync()

@@ -166,17 +166,19 @@ class Scheduler:
     def run_ahead_steps(self, plan: Sequence[Scheduled], limit: int = 256) -> int:
         """How many further steps can follow ``plan`` (already launched, its tokens not yet
         known) without any decision of the scheduler: every running request is in the plan
-        and samples in it, nothing waits, no request stops at EOS, none reaches its length
-        before the last of these steps, and the pool gives every request its pages (they are
-        reserved here).  Such steps hold one token per request, the one the step before
-        sampled, so they can be launched without waiting for the tokens."""
+        and samples in it, nothing waits, and no request stops at EOS.  In such steps every
+        request that still has tokens to produce takes one token, the one the step before
+        sampled; a request that reaches its length simply drops out (that is known without
+        the tokens).  The pages for those steps are reserved here; fewer steps are returned
+        when the pool cannot give them all."""
         if self.waiting or not plan or len(plan) != len(self.running):
             return 0
         if any(not s.samples or not s.request.params.ignore_eos for s in plan):
             return 0
-        # a request has len(output) + 1 tokens once the plan's step is accounted for
-        k = min(limit, min(s.request.params.max_tokens - (len(s.request.output) + 1) for s in plan))
-        while k > 0 and not all(self.runner.reserve(s.request.rid, k) for s in plan):
+        # once the plan's step is accounted for, a request has len(output) + 1 tokens
+        left = {s.request.rid: s.request.params.max_tokens - (len(s.request.output) + 1) for s in plan}
+        k = min(limit, max(left.values()))
+        while k > 0 and not all(self.runner.reserve(rid, min(k, n)) for rid, n in left.items() if n > 0):
             k //= 2
         return max(k, 0)
 

@@ -175,19 +175,28 @@ class ModelRunner:
 
     # --------------------------------------------------------------------- step
     @torch.inference_mode()
-    def step(self, entries: Sequence[StepEntry], token_source: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], token_source: Optional[torch.Tensor] = None,
+             token_index: Optional[Sequence[int]] = None) -> torch.Tensor:
         """Run the entries as one batch.  Pages for the new tokens must have been
         reserved.  Returns float32 logits [sum of wanted places, vocab], in the
         order of the entries and of their ``want``.
 
         ``token_source``: for a step of single tokens, an int32 tensor on the engine's device
-        with one token per entry that replaces the entries' own (the tokens an earlier step
-        sampled, not yet copied to the host: the step can be launched without waiting)."""
+        whose tokens replace the entries' own (the tokens an earlier step sampled, not yet
+        copied to the host: the step can be launched without waiting).  Entry i takes element
+        ``token_index[i]`` of it, or element i when no index is given."""
         if token_source is not None:
             if any(len(e.tokens) != 1 for e in entries):
                 raise ValueError("tokens from the device are for steps of single tokens")
-            if token_source.dtype != torch.int32 or token_source.numel() != len(entries):
-                raise ValueError("token_source must hold one int32 token per entry")
+            if token_source.dtype != torch.int32:
+                raise ValueError("token_source must be int32")
+            if token_index is None:
+                if token_source.numel() != len(entries):
+                    raise ValueError("token_source must hold one token per entry")
+            elif len(token_index) != len(entries) or not all(0 <= int(i) < token_source.numel() for i in token_index):
+                raise ValueError("token_index must name one element of token_source per entry")
+        elif token_index is not None:
+            raise ValueError("token_index needs token_source")
         spans = []
         seen = set()
         for e in entries:
@@ -216,14 +225,14 @@ class ModelRunner:
             )
         decode_only = all(len(s.tokens) == 1 and len(s.want) == 1 for s in spans)
         if self.use_graphs and decode_only and len(spans) <= GRAPH_MAX_SEQS:
-            logits = self._graph_step(spans, token_source)
+            logits = self._graph_step(spans, token_source, token_index)
         else:
             hb = build_host_batch(spans, len(self.group_shapes), self.page_size)
+            if token_index is not None:
+                hb.extra["token_gather"] = np.asarray(token_index, dtype=np.int32)
             buf, layout = pack(named_arrays(hb, self.builders))
             dev = self._uploader.upload(buf)
-            if token_source is not None:
-                off = layout["token_ids"][0]
-                dev[off : off + len(spans)].copy_(token_source.view(-1))
+            self._feed_tokens(dev, layout, len(spans), token_source, token_index is not None)
             ctx = StepContext(hb, self._views(dev, layout), self.sites, self.rt)
             self.last_host_batch = hb
             logits = self.model.forward(ctx)
@@ -239,7 +248,20 @@ class ModelRunner:
             for name, (off, shape) in layout.items()
         }
 
-    def _graph_step(self, spans, token_source: Optional[torch.Tensor] = None) -> torch.Tensor:
+    @staticmethod
+    def _feed_tokens(ints: torch.Tensor, layout, n: int, token_source: Optional[torch.Tensor], gathered: bool) -> None:
+        """Put the tokens of ``token_source`` (chosen by the step's own "token_gather" array
+        when ``gathered``) where the step's kernels read their token ids; all on the device."""
+        if token_source is None:
+            return
+        src = token_source.view(-1)
+        if gathered:
+            goff = layout["token_gather"][0]
+            src = src.index_select(0, ints[goff : goff + n])
+        off = layout["token_ids"][0]
+        ints[off : off + n].copy_(src)
+
+    def _graph_step(self, spans, token_source: Optional[torch.Tensor] = None, token_index: Optional[Sequence[int]] = None) -> torch.Tensor:
         """A step of single tokens through a captured graph.  The graph is keyed by what
         fixes its launches: the number of requests and the power-of-two bucket of the
         longest context (it decides how far attention splits the keys).  Block tables
@@ -249,6 +271,8 @@ class ModelRunner:
         while bucket < hb.max_ctx:
             bucket *= 2
         hb.max_ctx = bucket
+        # always there, so that the integer buffer keeps one layout
+        hb.extra["token_gather"] = np.asarray(token_index if token_index is not None else range(hb.n_seqs), dtype=np.int32)
         buf, layout = pack(named_arrays(hb, self.builders))
         key = (hb.n_seqs, bucket)
         entry = self._graphs.get(key)
@@ -256,9 +280,7 @@ class ModelRunner:
         if entry is None:
             ints = torch.empty(buf.size, dtype=torch.int32, device=self.config.device)
             ints.copy_(self._uploader.upload(buf))
-            if token_source is not None:
-                off = layout["token_ids"][0]
-                ints[off : off + len(spans)].copy_(token_source.view(-1))
+            self._feed_tokens(ints, layout, len(spans), token_source, token_index is not None)
             ctx = StepContext(hb, self._views(ints, layout), self.sites, self.rt)
             ops = self.rt.ops
             ops.reserve_workspaces(hb.n_seqs)
@@ -272,9 +294,7 @@ class ModelRunner:
             if layout != entry.layout:
                 raise RuntimeError("a decode step's integer arrays changed shape under a captured graph")
             entry.ints.copy_(self._uploader.upload(buf), non_blocking=True)
-            if token_source is not None:
-                off = layout["token_ids"][0]
-                entry.ints[off : off + len(spans)].copy_(token_source.view(-1))
+            self._feed_tokens(entry.ints, layout, len(spans), token_source, token_index is not None)
         entry.graph.replay()
         self.graph_replays += 1
         return entry.logits

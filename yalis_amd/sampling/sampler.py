@@ -70,6 +70,14 @@ class Sampler:
         ).to(self.device)
         return floats[0].contiguous(), ints[0].contiguous(), floats[1].contiguous(), ints[1].contiguous(), ints[2].contiguous()
 
+    @staticmethod
+    def narrow(prepared, index: torch.Tensor):
+        """The preparation for the rows ``index`` (an int32 tensor on the device) of a
+        prepared set, in that order."""
+        if prepared is None:
+            return None
+        return tuple(t.index_select(0, index) for t in prepared)
+
     def sample_prepared(self, logits: torch.Tensor, prepared, step: int) -> torch.Tensor:
         """Token ids (int32, on the device) for rows prepared with ``prepare``; ``step`` is
         added to every row's draw number (the step within a run that shares one preparation)."""
