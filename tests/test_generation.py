@@ -112,9 +112,18 @@ def test_steps_launched_ahead_change_nothing(tmp_path, backend, temperature, top
     plain, m2, _ = eng.generate(prompts, tokens_to_generate=20, get_logits=True)
     assert m1["StepsLaunchedAhead"] >= 15 and m2["StepsLaunchedAhead"] == 0
     assert torch.equal(ahead, plain)
-    # a request that stops at EOS needs its tokens on the host: nothing is launched ahead
-    _, m3 = eng.generate(prompts, tokens_to_generate=6, ignore_eos=False)
-    assert m3["StepsLaunchedAhead"] == 0
+    # where a request may stop at EOS the steps ahead are a guess (a few at most) and what
+    # they computed for it after its EOS is thrown away: make a token that one request
+    # produces half way its EOS, and compare with the run that waits for every token
+    eng.eos_token_ids = (int(plain[1, 9]),)
+    eng.last_scheduler = None
+    guessed, m3 = eng.generate(prompts, tokens_to_generate=20, ignore_eos=False)
+    waited, m4, _ = eng.generate(prompts, tokens_to_generate=20, ignore_eos=False, get_logits=True)
+    assert m3["StepsLaunchedAhead"] > 0 and m4["StepsLaunchedAhead"] == 0
+    assert torch.equal(guessed, waited)
+    stop = plain[1].tolist().index(eng.eos_token_ids[0])
+    assert guessed[1, : stop + 1].tolist() == plain[1, : stop + 1].tolist()
+    assert all(t == eng.eos_token_ids[0] for t in guessed[1, stop:].tolist())
     eng.runner.pages.audit()
     assert eng.runner.pages.live_requests() == 0
 

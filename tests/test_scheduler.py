@@ -146,13 +146,18 @@ def test_steps_that_need_no_decision():
     # a third request waits: the next step must admit it, nothing runs ahead
     sched.add([1, 2, 3], SamplingParams(temperature=0.0, max_tokens=4))
     assert sched.run_ahead_steps(plan) == 0
-    # EOS may stop a request: its tokens are needed on the host
+    # EOS may stop a request: only a few guessed steps, and a finished request is skipped
     sched2, runner2 = make()
-    sched2.add([1, 2, 3], SamplingParams(temperature=0.0, max_tokens=9, ignore_eos=False))
+    r2 = sched2.add([1, 2, 3], SamplingParams(temperature=0.0, max_tokens=30, ignore_eos=False))
     plan2 = sched2.schedule()
     for s in plan2:
         runner2.cached[s.request.rid] += s.n_tokens
-    assert sched2.run_ahead_steps(plan2) == 0
+    assert sched2.run_ahead_steps(plan2) == 8 and sched2.run_ahead_steps(plan2, eos_limit=2) == 2
+    sched2.update(plan2, [5])
+    single = [type(plan2[0])(r2, 1, True)]
+    sched2.update(single, [7])  # 7 is the EOS of this scheduler
+    assert r2.state == FINISHED and r2.output == [5, 7] and r2.finish_reason == "EOS"
+    assert sched2.update(single, [9]) == [] and r2.output == [5, 7], "a step launched past the EOS changes nothing"
     # a portion of a prompt that does not sample yet: no
     sched3, runner3 = make(budget=8)
     sched3.add(list(range(1, 21)), SamplingParams(temperature=0.0, max_tokens=9))

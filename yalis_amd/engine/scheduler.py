@@ -163,18 +163,22 @@ class Scheduler:
             out.append(StepEntry(s.request.rid, toks, [s.n_tokens - 1] if s.samples else []))
         return out
 
-    def run_ahead_steps(self, plan: Sequence[Scheduled], limit: int = 256) -> int:
+    def run_ahead_steps(self, plan: Sequence[Scheduled], limit: int = 256, eos_limit: int = 8) -> int:
         """How many further steps can follow ``plan`` (already launched, its tokens not yet
         known) without any decision of the scheduler: every running request is in the plan
-        and samples in it, nothing waits, and no request stops at EOS.  In such steps every
-        request that still has tokens to produce takes one token, the one the step before
-        sampled; a request that reaches its length simply drops out (that is known without
-        the tokens).  The pages for those steps are reserved here; fewer steps are returned
+        and samples in it, and nothing waits.  In such steps every request that still has
+        tokens to produce takes one token, the one the step before sampled; a request that
+        reaches its length simply drops out (that is known without the tokens).  Where a
+        request may stop at EOS the steps are a guess: at most ``eos_limit`` of them, and what
+        they computed for a request after its EOS is thrown away (``update`` skips finished
+        requests).  The pages for those steps are reserved here; fewer steps are returned
         when the pool cannot give them all."""
         if self.waiting or not plan or len(plan) != len(self.running):
             return 0
-        if any(not s.samples or not s.request.params.ignore_eos for s in plan):
+        if any(not s.samples for s in plan):
             return 0
+        if any(not s.request.params.ignore_eos for s in plan):
+            limit = min(limit, eos_limit)
         # once the plan's step is accounted for, a request has len(output) + 1 tokens
         left = {s.request.rid: s.request.params.max_tokens - (len(s.request.output) + 1) for s in plan}
         k = min(limit, max(left.values()))
@@ -189,6 +193,11 @@ class Scheduler:
         it = iter(sampled)
         for s in plan:
             req = s.request
+            if req.state == FINISHED:
+                # a step launched ahead of the news that this request had met its EOS
+                if s.samples:
+                    next(it)
+                continue
             req.computed += s.n_tokens
             if not s.samples:
                 continue
