@@ -146,6 +146,16 @@ def test_steps_that_need_no_decision():
     # a third request waits: the next step must admit it, nothing runs ahead
     sched.add([1, 2, 3], SamplingParams(temperature=0.0, max_tokens=4))
     assert sched.run_ahead_steps(plan) == 0
+    # all slots taken and a request waiting: it cannot get in before the first running
+    # request reaches its length, so the steps up to there need no decision
+    sched5, runner5 = make(num_pages=16, max_seqs=2, budget=64)
+    sched5.add(list(range(1, 11)), SamplingParams(temperature=0.0, max_tokens=9))
+    sched5.add(list(range(1, 31)), SamplingParams(temperature=0.0, max_tokens=5))
+    sched5.add([1, 2, 3], SamplingParams(temperature=0.0, max_tokens=4))
+    plan5 = sched5.schedule()
+    for s in plan5:
+        runner5.cached[s.request.rid] += s.n_tokens
+    assert len(plan5) == 2 and len(sched5.waiting) == 1 and sched5.run_ahead_steps(plan5) == 4
     # EOS may stop a request: only a few guessed steps, and a finished request is skipped
     sched2, runner2 = make()
     r2 = sched2.add([1, 2, 3], SamplingParams(temperature=0.0, max_tokens=30, ignore_eos=False))

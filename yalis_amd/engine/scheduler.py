@@ -166,21 +166,25 @@ class Scheduler:
     def run_ahead_steps(self, plan: Sequence[Scheduled], limit: int = 256, eos_limit: int = 8) -> int:
         """How many further steps can follow ``plan`` (already launched, its tokens not yet
         known) without any decision of the scheduler: every running request is in the plan
-        and samples in it, and nothing waits.  In such steps every request that still has
+        and samples in it, and no waiting request can get in.  In such steps every request that still has
         tokens to produce takes one token, the one the step before sampled; a request that
         reaches its length simply drops out (that is known without the tokens).  Where a
         request may stop at EOS the steps are a guess: at most ``eos_limit`` of them, and what
         they computed for a request after its EOS is thrown away (``update`` skips finished
         requests).  The pages for those steps are reserved here; fewer steps are returned
         when the pool cannot give them all."""
-        if self.waiting or not plan or len(plan) != len(self.running):
-            return 0
-        if any(not s.samples for s in plan):
+        if not plan or len(plan) != len(self.running) or any(not s.samples for s in plan):
             return 0
         if any(not s.request.params.ignore_eos for s in plan):
             limit = min(limit, eos_limit)
         # once the plan's step is accounted for, a request has len(output) + 1 tokens
         left = {s.request.rid: s.request.params.max_tokens - (len(s.request.output) + 1) for s in plan}
+        if self.waiting:
+            # a waiting request gets in when a slot frees; until the first running request
+            # reaches its length none does (if a slot is free now, the next step admits)
+            if len(self.running) < self.cfg.max_num_seqs:
+                return 0
+            limit = min(limit, min(left.values()))
         k = min(limit, max(left.values()))
         while k > 0 and not all(self.runner.reserve(rid, min(k, n)) for rid, n in left.items() if n > 0):
             k //= 2
