@@ -281,3 +281,31 @@ def test_more_requests_than_slots_and_a_small_pool(tmp_path, backend, seed):
         assert row == P.greedy_generate(cfg, weights, p, 12)
     eng2.runner.pages.audit()
     assert eng2.runner.pages.live_requests() == 0 and eng2.runner.pages.free_pages(0) == 8
+
+
+def test_nested_timers():
+    from yalis_amd.utils import Timers
+
+    t = Timers("cpu")
+    t.start("outer")
+    for _ in range(3):
+        t.start("inner")
+        t.stop("inner")
+    with pytest.raises(RuntimeError, match="innermost"):
+        t.stop("other")
+    t.stop("outer")
+    t.start("inner")  # the same name under another stack is another timer
+    t.stop("inner")
+    times, counts = t.get_times()
+    assert counts == {("outer",): 1, ("outer", "inner"): 3, ("inner",): 1}
+    assert times[("outer",)] >= times[("outer", "inner")] >= 0.0
+    assert t.get_times() == ({}, {}), "asking for the times starts a new account"
+
+
+def test_generate_leaves_its_timers(tmp_path):
+    eng, cfg, _ = make_engine(tmp_path, "A", ("cpu", "fp32"), 2, temperature=0.0, page_size=16, num_pages=16)
+    eng.generate(prompts_for(cfg, [5, 9]), tokens_to_generate=6)
+    times, counts = eng.last_timers.get_times()
+    assert counts[("tokenize",)] == 1 and counts[("generate",)] == 1
+    assert counts[("generate", "Prefill")] == 1 and counts[("generate", "DecodeAhead")] == 1
+    assert times[("generate",)] >= times[("generate", "DecodeAhead")]

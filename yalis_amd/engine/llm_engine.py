@@ -16,6 +16,7 @@ from ..config.reader import read_config_json
 from ..config.runtime import EngineConfig, InferenceConfig, ModelConfig
 from ..sampling.sampler import Sampler, SamplingParams
 from .factory import load_runner, random_runner
+from ..utils.timers import Timers
 from .scheduler import Request, Scheduled, Scheduler
 from .step import StepEntry
 
@@ -64,6 +65,7 @@ class LLMEngine:
         self.eos_token_ids = tuple(self.model.spec.eos_token_ids)
         self.tokenizer = self._load_tokenizer(model_config.model_path)
         self.last_scheduler: Optional[Scheduler] = None
+        self.last_timers: Optional[Timers] = None
 
     # --------------------------------------------------------------- tokenizer
     @staticmethod
@@ -106,10 +108,15 @@ class LLMEngine:
         Returns ``(tokens [batch, n] int64, metrics)`` and, with ``get_logits``, a
         list of n float32 tensors [batch, vocab] as well (yalis/engine.py:371-409,
         570-573).  Rows that stop early at EOS are padded with EOS, as the reference
-        keeps finished rows at EOS (:515-516).  ``enable_nvtx`` is accepted and
-        ignored (no range markers here)."""
+        keeps finished rows at EOS (:515-516).  ``enable_nvtx`` opens named ranges
+        (Prefill, Decode, DecodeAhead) for profilers; the same spans are always timed on the
+        device's clock and left in ``last_timers``."""
+        timers = Timers(self.engine_config.device)
+        self.last_timers = timers
         t_tok = time.perf_counter()
+        timers.start("tokenize")
         ids = self._tokenize_prompts(prompts)
+        timers.stop("tokenize")
         tokenize_ms = (time.perf_counter() - t_tok) * 1e3
         ic = self.inference_config
         if len(ids) > ic.max_batch_size:
@@ -144,9 +151,20 @@ class LLMEngine:
         def seconds(a, b) -> float:
             return (b - a) if not cuda else a.elapsed_time(b) * 1e-3
 
+        def open_range(name):  # a named range for profilers (the reference's NVTX ranges, yalis/utils.py:34-51)
+            timers.start(name)
+            if enable_nvtx and cuda:
+                torch.cuda.nvtx.range_push(name)
+
+        def close_range(name):
+            if enable_nvtx and cuda:
+                torch.cuda.nvtx.range_pop()
+            timers.stop(name)
+
         sync()
         t0 = time.perf_counter()
         m0 = mark()
+        timers.start("generate")
         first_token_at: Dict[int, object] = {}
         decode_steps = 0
         decode_spans = []  # (mark before, mark after, steps)
@@ -156,10 +174,13 @@ class LLMEngine:
             plan = sched.schedule()
             if not plan:
                 raise RuntimeError("the scheduler made no progress (pool too small for any request?)")
+            kind = "Decode" if all(s.n_tokens == 1 for s in plan) else "Prefill"
+            open_range(kind)
             logits = self.runner.step(sched.entries(plan))
             sampling = [s.request for s in plan if s.samples]
             prepared = self.sampler.prepare([r.params for r in sampling], [len(r.output) for r in sampling])
             toks = self.sampler.sample_prepared(logits, prepared, 0) if sampling else None
+            close_range(kind)
             after = mark()
             for r in sampling:
                 first_token_at.setdefault(r.rid, after)
@@ -177,6 +198,7 @@ class LLMEngine:
                 have = {s.request.rid: len(s.request.output) + 1 for s in plan}
                 rows = [s.request for s in plan]  # the requests of the last launched step, in its order
                 run, plans = [toks], []
+                open_range("DecodeAhead")
                 for j in range(ahead):
                     cur = [r for r in rows if have[r.rid] < r.params.max_tokens]
                     if not cur:
@@ -193,6 +215,7 @@ class LLMEngine:
                     for r in cur:
                         have[r.rid] += 1
                     rows = cur
+                close_range("DecodeAhead")
                 decode_spans.append((after, mark(), len(plans)))
                 steps_ahead += len(plans)
                 flat = torch.cat([t.view(-1) for t in run]).tolist()
@@ -203,6 +226,7 @@ class LLMEngine:
                     at += len(p)
                 continue
             sched.update(plan, toks.tolist() if toks is not None else [])
+        timers.stop("generate")
         sync()
         total = time.perf_counter() - t0
         decode_steps = sum(n for _, _, n in decode_spans)
