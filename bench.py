@@ -56,6 +56,7 @@ def main() -> int:
     ap.add_argument("--prefill-len", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--only-prefill", action="store_true", help="measure the prefill only (for profiling)")
+    ap.add_argument("--mixed", action="store_true", help="measure mixed steps instead: 32 decode streams beside 512-token portions of 4,096-token prompts")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel (for hardware counters)")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="8b", help="layer sizes (default: the 8B shape of the headline)")
     args = ap.parse_args()
@@ -79,6 +80,8 @@ def main() -> int:
     max_batch = max(args.batch, 1 if args.no_points else 64)
     total_steps = args.steps + args.warmup + 8
     ctx_cap = max(args.prompt_len + total_steps + 1, args.prefill_len)
+    if args.mixed:
+        max_batch, ctx_cap = 34, 4096 + 64
     pages_per_req = -(-ctx_cap // page)
     engine = EngineConfig(
         page_size=page,
@@ -142,6 +145,52 @@ def main() -> int:
     def step_bytes(batch, mean_ctx_tokens):
         kv = mean_ctx_tokens * layers * 2 * g * d * 2
         return weight_bytes + batch * c * 2 + kv
+
+    if args.mixed:
+        # 32 requests decode while 4,096-token prompts arrive in portions of 512 tokens: every
+        # step holds 32 single tokens and one portion (the last portion's row is sampled too)
+        n_dec, portion, plen = 32, 512, 4096
+        toks = []
+        for r in range(n_dec):
+            assert runner.admit(r)
+            prompt = torch.randint(0, vocab, (args.prompt_len,), generator=gen).tolist()
+            assert runner.reserve(r, len(prompt))
+            toks.append(ops.argmax(runner.step([StepEntry(r, prompt, [len(prompt) - 1])])).tolist()[0])
+        prompt = torch.randint(0, vocab, (plen,), generator=gen).tolist()
+        times, kv_tokens = [], []
+        for rid in (100, 101, 102):  # the first prompt warms up
+            assert runner.admit(rid)
+            for c0 in range(0, plen, portion):
+                for r in range(n_dec):
+                    assert runner.reserve(r, 1)
+                assert runner.reserve(rid, portion)
+                last = c0 + portion == plen
+                entries = [StepEntry(r, [toks[r]], [0]) for r in range(n_dec)]
+                entries.append(StepEntry(rid, prompt[c0 : c0 + portion], [portion - 1] if last else []))
+                ctx_tokens = sum(runner.cached[r] + 1 for r in range(n_dec)) + c0 + portion
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                out = ops.argmax(runner.step(entries)).tolist()
+                torch.cuda.synchronize()
+                if rid != 100:
+                    times.append(time.perf_counter() - t0)
+                    kv_tokens.append(ctx_tokens)
+                toks = out[:n_dec]
+            runner.release(rid)
+        ms = 1e3 * sum(times) / len(times)
+        n_tok = n_dec + portion
+        mean_kv = sum(kv_tokens) / len(kv_tokens)
+        step_b = weight_bytes + mean_kv * layers * 2 * g * d * 2
+        # products over all tokens of the step; attention of the portion against the prompt so far
+        step_f = layers * (2 * n_tok * layer_params + 4 * h * d * portion * (plen / 2)) + 2 * (n_dec + 1 / 8) * vocab * c
+        bound_ms = 1e3 * max(step_b / (HBM_GBPS * 1e9), step_f / BF16_FLOPS)
+        print(json.dumps({
+            "metric": f"mixed steps ({shape_name} shape): {n_dec} decode streams beside {portion}-token portions of {plen:,}-token prompts",
+            "ms_per_step": round(ms, 3), "decode_tokens_per_s": round(n_dec / ms * 1e3, 1), "prefill_tokens_per_s": round(portion / ms * 1e3, 1),
+            "steps": len(times), "dtype": "bf16", "n_gpus": 1,
+            "roofline": {"bound": "max(hbm, mfma)", "bound_ms": round(bound_ms, 3), "frac": round(bound_ms / ms, 4)},
+        }))
+        return 0
 
     if args.only_prefill:
         t = args.prefill_len

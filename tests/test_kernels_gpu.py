@@ -313,7 +313,7 @@ def test_rope_append_prompt_portions(ops, h, g, d, rd, page):
 
 
 # ------------------------------------------------------------------------- attention
-def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True, n_pages=64, plan=None):
+def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True, n_pages=64, plan=None, long_plan=None):
     """spans: list of (cached tokens before the step, new tokens).  Builds pages in a
     shuffled order, fills cache for the earlier tokens, runs rope-free attention."""
     gen = torch.Generator().manual_seed(seed)
@@ -349,7 +349,7 @@ def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True,
     n = hb.n_tokens
     q = (torch.randn((n, h * d), generator=gen) * 1.5).to(dtype)
     scale = 1.0 / math.sqrt(d)
-    got = ops.attention(q.to(DEV), h, g, d, kc.to(DEV), vc.to(DEV), page, scale, window, ctx, 0, ctx.arrays["tiles"], ctx.arrays["long_tiles"], plan=plan)
+    got = ops.attention(q.to(DEV), h, g, d, kc.to(DEV), vc.to(DEV), page, scale, window, ctx, 0, ctx.arrays["tiles"], ctx.arrays["long_tiles"], plan=plan, long_plan=long_plan)
     want = R.attention(q.float(), h, g, d, kc.float(), vc.float(), page, scale, window, ctx_cpu, 0, None)
     return got, want
 
@@ -398,6 +398,27 @@ def test_attention_mfma_every_way_of_dividing_keys(ops, plan, d):
     for window in (0, 700, 33):
         got, want = _attention_case(ops, torch.bfloat16, 8, 2, d, 32, spans, window, seed=16, n_pages=96, plan=plan)
         close(got, want, 2e-2, 2**-6)
+
+
+@pytest.mark.parametrize("splits", [1, 2, 5, 16])
+@pytest.mark.parametrize("h,g,d,page", [(8, 2, 128, 64), (6, 3, 64, 16), (32, 1, 128, 32)])
+def test_attention_long_spans_with_split_keys(ops, splits, h, g, d, page):
+    """Portions of prompts against a long cached context, the keys split across workgroups
+    and merged: spans that end a tile early, a window, more splits than some tiles have key
+    blocks (empty parts)."""
+    spans = [(900, 70), (0, 130), (1500, 33), (40, 100)]
+    for window in (0, 300):
+        got, want = _attention_case(ops, torch.bfloat16, h, g, d, page, spans, window, seed=18, n_pages=3000 // page + 8, long_plan=splits)
+        close(got, want, 2e-2, 2**-6)
+
+
+def test_attention_long_splits_policy():
+    from yalis_amd.ops.hip import HipOps
+
+    assert HipOps.attention_long_splits(1024, 32) == 1  # a whole prompt: tiles fill the GPU
+    assert HipOps.attention_long_splits(256, 64) == 3  # a 512-token portion against 4,096 keys
+    assert HipOps.attention_long_splits(8, 400) == 16 and HipOps.attention_long_splits(8, 20) == 2
+    assert HipOps.attention_long_splits(8, 4) == 1
 
 
 def test_attention_plan_covers_the_launch():

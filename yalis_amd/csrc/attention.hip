@@ -401,7 +401,8 @@ __global__ __launch_bounds__(256, 3) void attn_mfma_prefill_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ block_table, int table_width,
-    int page_size, int n_heads, int n_kv, int hpt, int chunks, float scale_log2, int window) {
+    int page_size, int n_heads, int n_kv, int hpt, int chunks, float scale_log2, int window,
+    int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml) {
   constexpr int KS = D / 32, DT = D / 16, CT = PF_CT;
   constexpr int KROW = D + 8;   // bf16 elements per parked key row
   constexpr int VROW = 64 + 8;  // bf16 elements per parked value row
@@ -435,14 +436,18 @@ __global__ __launch_bounds__(256, 3) void attn_mfma_prefill_kernel(
   const int hi = tile_pos0 + tile_ntok;  // keys the workgroup may need
   const int lo = window > 0 ? max(0, tile_pos0 - window + 1) : 0;
   const int wave_hi = min(hi, tile_pos0 + wave_tok0 + CT * tpt);  // keys this wave may need
-  const int kb_lo = lo / 64, kb_hi = (hi + 63) / 64;
+  // the workgroup's share of the key blocks when a launch splits them (blockIdx.y): few long
+  // tiles against a long context would otherwise leave most of the GPU idle
+  const int all_lo = lo / 64, all_hi = (hi + 63) / 64;
+  const int per_split = (all_hi - all_lo + n_splits - 1) / n_splits;
+  const int kb_lo = all_lo + blockIdx.y * per_split, kb_hi = min(all_hi, kb_lo + per_split);
   const int32_t* bt = block_table + static_cast<size_t>(seq) * table_width;
   const int last_page_col = min(table_width - 1, (hi - 1) / page_size);
   // page ids of the keys this workgroup walks, once, into LDS (a lookup per fetched piece
   // would put a dependent memory round trip before every load)
   constexpr int PAGES_LDS = 2048;
   __shared__ int32_t pages_s[PAGES_LDS];
-  const int first_col = min(last_page_col, kb_lo * 64 / page_size);
+  const int first_col = min(last_page_col, max(0, kb_lo) * 64 / page_size);
   const bool pages_in_lds = last_page_col - first_col < PAGES_LDS;
   if (pages_in_lds)
     for (int c = first_col + threadIdx.x; c <= last_page_col; c += 256) pages_s[c - first_col] = max(0, bt[c]);
@@ -632,6 +637,19 @@ __global__ __launch_bounds__(256, 3) void attn_mfma_prefill_kernel(
     float lc = l[c];
     lc += __shfl_xor(lc, 16, 64);
     lc += __shfl_xor(lc, 32, 64);
+    if (n_splits > 1) {
+      // partial result of this split, a group of 16 columns per wave (and column tile)
+      const size_t group = (static_cast<size_t>(t) * 4 * CT + wave * CT + c) * n_y + by;
+      const size_t widx = group * n_splits + blockIdx.y;
+      float* wo = ws_o + (widx * 16 + r) * D + 4 * gq;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4_t*>(wo + 16 * dt) = acc[c][dt];
+      if (gq == 0) {
+        ws_ml[(widx * 16 + r) * 2] = m[c];
+        ws_ml[(widx * 16 + r) * 2 + 1] = lc;
+      }
+      continue;
+    }
     if (col_ok[c]) {
       const float inv = 1.f / lc;
       bf16_t* op = out + (static_cast<size_t>(tile_tok0 + tok_c[c]) * n_heads + h_base + hh) * D + 4 * gq;
@@ -648,17 +666,20 @@ __global__ __launch_bounds__(256, 3) void attn_mfma_prefill_kernel(
 
 // Merge the splits of every column: weights exp2(m_s - max m), in the order of s.
 // A thread owns four consecutive output elements of one column.
+// blockIdx.x names a group of 16 columns: a tile of the short-span kernel (parts == 1), or one
+// wave's share of a long tile (parts == 4: group x is wave x % 4 of tile x / 4).
 template <int D>
 __global__ __launch_bounds__(256) void attn_combine_kernel(
     bf16_t* __restrict__ out, const int32_t* __restrict__ tiles, int n_heads, int n_kv, int hpt,
-    int chunks, int n_splits, const float* __restrict__ ws_o, const float* __restrict__ ws_ml) {
-  const int t = blockIdx.x;
-  const int tok0 = tiles[4 * t + 1], ntok = tiles[4 * t + 2];
+    int chunks, int n_splits, const float* __restrict__ ws_o, const float* __restrict__ ws_ml, int parts) {
+  const int t = blockIdx.x / parts, part = blockIdx.x % parts;
+  const int tpt_ = 16 / hpt;
+  const int tok0 = tiles[4 * t + 1] + part * tpt_, ntok = tiles[4 * t + 2] - part * tpt_;
   const int g = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
   const int qpk = n_heads / n_kv;
   const int h_base = g * qpk + chunk * hpt;
   const int heads_here = min(hpt, qpk - chunk * hpt);
-  const size_t w0 = (static_cast<size_t>(t) * gridDim.y + blockIdx.y) * n_splits;
+  const size_t w0 = (static_cast<size_t>(blockIdx.x) * gridDim.y + blockIdx.y) * n_splits;
   for (int e = threadIdx.x; e < 16 * (D / 4); e += blockDim.x) {
     const int c = e / (D / 4), d = (e % (D / 4)) * 4;
     const int tt = c / hpt, hh = c % hpt;
@@ -713,6 +734,7 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
                                     const void* v_cache, const int32_t* tiles, int n_tiles,
                                     const int32_t* block_table, int table_width, int page_size,
                                     int head_dim, int n_heads, int n_kv, float scale, int window,
+                                    int n_splits, float* workspace, size_t workspace_floats,
                                     hipStream_t stream) {
   YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_mfma_prefill: bad head counts");
   YK_REQUIRE(yk_attn_mfma_supported(head_dim), "attn_mfma_prefill: head_dim must be 64 or 128");
@@ -727,13 +749,19 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
   const int hpt = yk_attn_heads_per_tile(n_heads, n_kv);
   const int chunks = (n_heads / n_kv + hpt - 1) / hpt;
   YK_REQUIRE(static_cast<long long>(n_tiles) * n_kv * chunks <= 0x7fffffffLL, "attn_mfma_prefill: too many tiles for one launch");
+  YK_REQUIRE(n_splits >= 1 && n_splits <= 65535, "attn_mfma_prefill: bad split count");
+  static_assert(PF_CT == 1, "the merge of split long tiles takes one column tile per wave");
+  const size_t need = yk_attn_mfma_workspace(4 * n_tiles, n_heads, n_kv, head_dim, n_splits);
+  YK_REQUIRE(workspace_floats >= need, "attn_mfma_prefill: workspace too small");
+  float* ws_o = workspace;
+  float* ws_ml = workspace ? workspace + (need / (head_dim + 2)) * head_dim : nullptr;
   const float scale_log2 = scale * 1.4426950408889634f;
-  dim3 grid(n_tiles * n_kv * chunks), block(256);
+  dim3 grid(n_tiles * n_kv * chunks, n_splits), block(256);
 #define YK_PF(DD, BIP)                                                                                       \
   attn_mfma_prefill_kernel<DD, BIP><<<grid, block, 0, stream>>>(                                                 \
       static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),   \
       static_cast<const bf16_t*>(v_cache), tiles, block_table, table_width, page_size, n_heads, n_kv, hpt, chunks, \
-      scale_log2, window)
+      scale_log2, window, n_splits, ws_o, ws_ml)
   const bool bip = page_size % 64 == 0;
   if (head_dim == 64) {
     if (bip) YK_PF(64, true); else YK_PF(64, false);
@@ -741,7 +769,16 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
     if (bip) YK_PF(128, true); else YK_PF(128, false);
   }
 #undef YK_PF
-  return yk_check_launch("attn_mfma_prefill");
+  if (yk_check_launch("attn_mfma_prefill")) return -1;
+  if (n_splits > 1) {
+    dim3 cgrid(4 * n_tiles, n_kv * chunks);
+    if (head_dim == 64)
+      attn_combine_kernel<64><<<cgrid, 256, 0, stream>>>(static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 4);
+    else
+      attn_combine_kernel<128><<<cgrid, 256, 0, stream>>>(static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 4);
+    return yk_check_launch("attn_combine");
+  }
+  return 0;
 }
 
 extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* k_cache,
@@ -781,7 +818,7 @@ extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* 
   if (yk_check_launch("attn_mfma")) return -1;                                                     \
   if (n_splits > 1) {                                                                              \
     attn_combine_kernel<DD><<<dim3(n_tiles, n_kv * chunks), 256, 0, stream>>>(                     \
-        static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml);      \
+        static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 1);   \
     if (yk_check_launch("attn_combine")) return -1;                                                \
   }
   if (head_dim == 64) {

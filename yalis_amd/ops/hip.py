@@ -72,7 +72,7 @@ _SIGNATURES = {
     "yk_attn_tokens_per_tile": ([_c_int, _c_int], _c_int),
     "yk_attn_mfma_workspace": ([_c_int, _c_int, _c_int, _c_int, _c_int], _c_size_t),
     "yk_attn_mfma_prefill": (
-        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp],
+        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _vp, _c_size_t, _vp],
         _c_int,
     ),
     "yk_attn_mfma": (
@@ -378,11 +378,21 @@ class HipOps:
             return 1, 1
         return 4, max(1, min(-(-par // 4), 256))
 
+    @staticmethod
+    def attention_long_splits(workgroups: int, key_blocks: int) -> int:
+        """Splits of the keys for the long-span kernel: one where the tiles alone fill the GPU
+        (a prompt of a few thousand tokens); more where few tiles meet a long context (a
+        portion of a prompt whose earlier portions are cached), at least 8 key blocks a split."""
+        if workgroups >= 512:
+            return 1
+        return max(1, min(-(-768 // workgroups), key_blocks // 8, 16))
+
     def attention(self, qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size,
-                  scale, window, ctx, group, tiles, long_tiles=None, plan=None) -> torch.Tensor:
+                  scale, window, ctx, group, tiles, long_tiles=None, plan=None, long_plan=None) -> torch.Tensor:
         """Queries are the first n_heads heads of each row of ``qkv`` (whatever follows
         them in the row is skipped); keys and values come from the cache through the
-        block table of ``group``.  ``plan`` overrides ``attention_plan`` (tests, measurements)."""
+        block table of ``group``.  ``plan`` overrides ``attention_plan`` and ``long_plan``
+        ``attention_long_splits`` (tests, measurements)."""
         self._rows(qkv, "qkv")
         n = qkv.shape[0]
         bt = ctx.arrays[f"block_table_g{group}"]
@@ -398,11 +408,18 @@ class HipOps:
             and qkv.data_ptr() % 16 == 0
         )
         if use_mfma and long_tiles is not None and long_tiles.shape[0] > 0:
+            n_long = long_tiles.shape[0]
+            hpt = self.lib.yk_attn_heads_per_tile(n_heads, n_kv)
+            groups = n_long * n_kv * (-(-(n_heads // n_kv) // hpt))
+            long_splits = long_plan if long_plan is not None else self.attention_long_splits(groups, max(1, -(-ctx.max_ctx // 64)))
+            ws_floats = self.lib.yk_attn_mfma_workspace(4 * n_long, n_heads, n_kv, head_dim, long_splits)
+            ws = self._ws(ws_floats) if ws_floats else None
             self._check(
                 self.lib.yk_attn_mfma_prefill(
                     qkv.data_ptr(), qkv.stride(0), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-                    long_tiles.data_ptr(), long_tiles.shape[0], bt.data_ptr(), bt.shape[1], page_size, head_dim,
-                    n_heads, n_kv, float(scale), int(window), self._stream(),
+                    long_tiles.data_ptr(), n_long, bt.data_ptr(), bt.shape[1], page_size, head_dim,
+                    n_heads, n_kv, float(scale), int(window), long_splits, _ptr(ws), 0 if ws is None else ws.numel(),
+                    self._stream(),
                 )
             )
         if use_mfma and tiles.shape[0] == 0:
