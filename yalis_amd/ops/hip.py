@@ -132,11 +132,18 @@ class HipOps:
             fn.restype = res
         if self.lib.yk_abi_version() != 4:
             raise KernelError("kernel library and bindings disagree; rebuild (python -c 'import __graft_entry__ as g; g.build()')")
+        self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
+        # the quick way to the current stream's handle, where this torch has it
+        self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
         self._workspace: Optional[torch.Tensor] = None  # attention splits, argmax parts
         self._gemm_workspace: Optional[torch.Tensor] = None  # K slices of products
 
     # ------------------------------------------------------------------ helpers
     def _stream(self) -> int:
+        """The raw handle of torch's current stream on this device (asked for at every
+        launch: a graph capture switches streams)."""
+        if self._raw_stream is not None:
+            return self._raw_stream(self._device_index)
         return torch.cuda.current_stream(self.device).cuda_stream
 
     def _check(self, rc: int) -> None:
