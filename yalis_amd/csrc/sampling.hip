@@ -145,7 +145,23 @@ template <typename F>
 __device__ __forceinline__ void for_each_logit(const float* __restrict__ row, int vocab, F f) {
   if (reinterpret_cast<uintptr_t>(row) % 16 == 0) {
     const int n4 = vocab / 4;
-    for (int j = threadIdx.x; j < n4; j += blockDim.x) {
+    // four loads in flight per thread: a pass over a row is one workgroup's work and would
+    // otherwise wait for memory once per load (elements still reach f in ascending order)
+    int j = threadIdx.x;
+    for (; j + 3 * static_cast<int>(blockDim.x) < n4; j += 4 * blockDim.x) {
+      float4 v[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v[q] = reinterpret_cast<const float4*>(row)[j + q * blockDim.x];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int i = 4 * (j + q * blockDim.x);
+        f(v[q].x, i);
+        f(v[q].y, i + 1);
+        f(v[q].z, i + 2);
+        f(v[q].w, i + 3);
+      }
+    }
+    for (; j < n4; j += blockDim.x) {
       const float4 v = reinterpret_cast<const float4*>(row)[j];
       f(v.x, 4 * j);
       f(v.y, 4 * j + 1);
