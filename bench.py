@@ -45,6 +45,64 @@ LLAMA31_70B = dict(LLAMA3_8B, hidden_size=8192, num_hidden_layers=80, num_attent
 SHAPES = {"8b": ("Llama-3-8B", LLAMA3_8B), "3b": ("Llama-3.2-3B", LLAMA32_3B), "70b": ("Llama-3.1-70B", LLAMA31_70B)}
 
 
+def machine_probe(cfg: dict) -> int:
+    """What the card gives a kernel that does nothing but read, at the sizes of the shape's
+    weight matrices, and a kernel that does nothing but issue bfloat16 matrix-core
+    instructions.  The decode products stream their weights once, so the first is their
+    practical bound; the second is the bound of any bfloat16 product."""
+    import torch
+
+    from yalis_amd.ops.hip import HipOps
+
+    ops = HipOps("cuda:0")
+    c, h, g, d = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    inter, vocab = cfg["intermediate_size"], cfg["vocab_size"]
+    sizes = {
+        "o_proj": h * d * c * 2,
+        "qkv_proj": (h + 2 * g) * d * c * 2,
+        "down_proj": c * inter * 2,
+        "gate_up_proj": 2 * inter * c * 2,
+        "head": vocab * c * 2,
+    }
+    arena = torch.empty(6 << 30, dtype=torch.uint8, device="cuda")
+    arena.view(torch.int32).random_(0, 1 << 20)  # small positive floats: no NaN, nothing cached from a memset
+    sink = torch.zeros(1, dtype=torch.float32, device="cuda")
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    out = {}
+    print("streaming read of one weight matrix (a fresh piece of a 6 GiB arena each time, mean of 20):")
+    for name, nbytes in sizes.items():
+        best = None
+        for wgs, nt in ((512, False), (2048, False), (16384, False), (512, True), (2048, True), (16384, True)):
+            offset, total = 0, 0.0
+            for rep in range(23):
+                if offset + nbytes > arena.numel():
+                    offset = 0
+                piece = arena[offset : offset + nbytes]
+                offset += -(-nbytes // 4096) * 4096
+                start.record()
+                ops.probe_stream_read(piece, wgs, sink, nontemporal=nt)
+                stop.record()
+                stop.synchronize()
+                if rep >= 3:
+                    total += start.elapsed_time(stop)
+            us = total / 20 * 1e3
+            if best is None or us < best[0]:
+                best = (us, wgs, nt)
+        tbs = nbytes / (best[0] * 1e-6) / 1e12
+        out[name] = {"MB": round(nbytes / 1e6, 1), "us": round(best[0], 1), "TB/s": round(tbs, 2), "workgroups": best[1], "nontemporal": best[2]}
+        print(f"  {name:13s} {nbytes / 1e6:8.1f} MB  {best[0]:7.1f} us  {tbs:5.2f} TB/s  ({best[1]} workgroups{', nontemporal loads' if best[2] else ''})")
+    wgs, iters = 256 * 8, 20000
+    for rep in range(3):
+        start.record()
+        flops = ops.probe_mfma_bf16(wgs, iters, sink)
+        stop.record()
+        stop.synchronize()
+    pf = flops / (start.elapsed_time(stop) * 1e-3) / 1e15
+    print(f"bfloat16 matrix-core loop from registers ({wgs} workgroups of 4 waves, 4 accumulators each): {pf:.2f} PFLOP/s")
+    print(json.dumps({"probe": "machine", "stream_read": out, "mfma_bf16_pflops": round(pf, 3)}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -59,12 +117,16 @@ def main() -> int:
     ap.add_argument("--mixed", action="store_true", help="measure mixed steps instead: 32 decode streams beside 512-token portions of 4,096-token prompts")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel (for hardware counters)")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="8b", help="layer sizes (default: the 8B shape of the headline)")
+    ap.add_argument("--probe", action="store_true", help="measure instead what a plain streaming read and a plain matrix-core loop reach on this card")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
         return 2
 
     import torch
+
+    if args.probe:
+        return machine_probe(SHAPES[args.shape][1])
 
     from yalis_amd.config.runtime import EngineConfig
     from yalis_amd.engine.factory import random_runner

@@ -567,3 +567,22 @@ def test_sample_frequencies(ops):
     p = torch.softmax(logits[0].cpu().double() / temperature, dim=0)
     chi2 = ((counts - draws * p) ** 2 / (draws * p)).sum().item()
     assert chi2 < 40.0, chi2  # 11 degrees of freedom: 40 is beyond the 99.99th percentile
+
+
+def test_machine_probes_run_and_refuse_bad_sizes(ops):
+    """The benchmark's two probes: they leave their input and (for ordinary data) their sink
+    alone, count their flops, and refuse sizes their kernels do not take."""
+    from yalis_amd.ops.hip import KernelError
+
+    data = rnd((1 << 16,), torch.float32, 0)
+    before = data.clone()
+    sink = torch.zeros(1, dtype=torch.float32, device=DEV)
+    for workgroups in (1, 7, 300):
+        ops.probe_stream_read(data, workgroups, sink, nontemporal=workgroups == 7)
+    assert ops.probe_mfma_bf16(3, 32, sink) == 3 * 4 * 32 * 4 * 16384
+    torch.cuda.synchronize()
+    assert torch.equal(data, before) and sink.item() == 0.0
+    with pytest.raises(KernelError):
+        ops.probe_stream_read(data[1:4], 4, sink)  # neither aligned nor whole 16-byte pieces
+    with pytest.raises(KernelError):
+        ops.probe_mfma_bf16(3, 10, sink)

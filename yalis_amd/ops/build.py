@@ -28,6 +28,7 @@ KERNEL_SOURCES = [
     "gemm.hip",
     "attention.hip",
     "sampling.hip",
+    "probe.hip",
 ]
 HEADERS = ["common.h"]
 

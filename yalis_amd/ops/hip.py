@@ -81,6 +81,8 @@ _SIGNATURES = {
     ),
     "yk_argmax": ([_vp, _vp, _c_int, _c_int, _vp, _c_size_t, _vp], _c_int),
     "yk_sample": ([_vp, _vp, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _vp], _c_int),
+    "yk_probe_stream_read": ([_vp, _c_size_t, _c_int, _c_int, _vp, _vp], _c_int),
+    "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
 }
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
@@ -130,7 +132,7 @@ class HipOps:
             fn = getattr(self.lib, name)
             fn.argtypes = args
             fn.restype = res
-        if self.lib.yk_abi_version() != 4:
+        if self.lib.yk_abi_version() != 5:
             raise KernelError("kernel library and bindings disagree; rebuild (python -c 'import __graft_entry__ as g; g.build()')")
         self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
         # the quick way to the current stream's handle, where this torch has it
@@ -515,3 +517,15 @@ class HipOps:
             )
         )
         return out
+
+    # ------------------------------------------------------------------ machine probes
+    def probe_stream_read(self, data: torch.Tensor, workgroups: int, sink: torch.Tensor, nontemporal: bool = False) -> None:
+        """Reads every byte of ``data`` once with a plain streaming kernel (for timing);
+        ``nontemporal`` marks the loads as not to be kept in the caches."""
+        self._check(self.lib.yk_probe_stream_read(data.data_ptr(), data.numel() * data.element_size(), int(workgroups),
+                                                  int(bool(nontemporal)), sink.data_ptr(), self._stream()))
+
+    def probe_mfma_bf16(self, workgroups: int, iterations: int, sink: torch.Tensor) -> int:
+        """Issues a loop of bfloat16 matrix-core instructions from registers; returns its flop count."""
+        self._check(self.lib.yk_probe_mfma_bf16(int(workgroups), int(iterations), sink.data_ptr(), self._stream()))
+        return int(workgroups) * 4 * int(iterations) * 4 * 16384
