@@ -175,3 +175,45 @@ class RefOps:
                 sample_token(logits[i].cpu(), float(temperature[i]), k if k > 0 else None, float(top_p[i]), int(seeds[i]), int(draws[i]))
             )
         return torch.tensor(out, dtype=torch.int32, device=logits.device)
+
+
+# ------------------------------------------------------------------ tiled cache pages
+# The matrix-core attention keeps bfloat16 pages of a multiple of 64 tokens (head sizes 64 and
+# 128) in the order its loads take them.  Written out here once more, from the layout's
+# description (yalis_amd/csrc/common.h), so that tests can fill pages and read them back:
+#   keys:   within a block of 64 slots, piece (((u*2 + sb) * D/32 + ks) * 4 + g) * 16 + r holds
+#           dims 32ks + 8g .. +7 of slot 32u + 8(r/4) + 4sb + r%4;
+#   values: piece ((u * D/16 + dt) * 4 + g) * 16 + r holds slots 32u + 8g .. +7 of dim 16dt + r.
+def _tiled_indices(page, d):
+    import numpy as np
+
+    slot = np.arange(page)[:, None]
+    dim = np.arange(d)[None, :]
+    j = slot % 64
+    u, a, sb, b = j // 32, (j % 32) // 8, (j % 8) // 4, j % 4
+    piece_k = (((u * 2 + sb) * (d // 32) + dim // 32) * 4 + (dim % 32) // 8) * 16 + 4 * a + b
+    k_at = (slot // 64) * 64 * d + piece_k * 8 + dim % 8            # [slot, dim] -> offset in the slab
+    piece_v = ((u * (d // 16) + dim // 16) * 4 + (j % 32) // 8) * 16 + dim % 16
+    v_at = (slot // 64) * 64 * d + piece_v * 8 + j % 8              # [slot, dim] -> offset in the slab
+    assert sorted(k_at.ravel()) == list(range(page * d)) and sorted(v_at.ravel()) == list(range(page * d))
+    return torch.from_numpy(k_at.ravel()), torch.from_numpy(v_at.T.copy().ravel())  # in the plain slabs' element order
+
+
+def tile_cache(k_plain, v_plain):
+    """Plain pages ([pages, kv, page, D] keys, [pages, kv, D, page] values) -> the same shapes
+    holding the tiled order."""
+    n, g, page, d = k_plain.shape
+    k_at, v_at = _tiled_indices(page, d)
+    k = torch.empty_like(k_plain).view(n, g, page * d)
+    v = torch.empty_like(v_plain).view(n, g, page * d)
+    k[:, :, k_at] = k_plain.reshape(n, g, page * d)
+    v[:, :, v_at] = v_plain.reshape(n, g, page * d)
+    return k.view(n, g, page, d), v.view(n, g, d, page)
+
+
+def untile_cache(k_tiled, v_tiled):
+    n, g, page, d = k_tiled.shape
+    k_at, v_at = _tiled_indices(page, d)
+    k = k_tiled.reshape(n, g, page * d)[:, :, k_at]
+    v = v_tiled.reshape(n, g, page * d)[:, :, v_at]
+    return k.reshape(n, g, page, d), v.reshape(n, g, d, page)

@@ -28,6 +28,20 @@ def rnd(shape, dtype, seed, scale=1.0):
     return (torch.randn(shape, generator=g) * scale).to(dtype).to(DEV)
 
 
+def device_cache(ops, kc, vc):
+    """Pages written in the plain order -> what the kernels expect, on the GPU."""
+    if ops.cache_tiled(kc.dtype, kc.shape[3], kc.shape[2]):
+        kc, vc = R.tile_cache(kc.cpu(), vc.cpu())
+    return kc.to(DEV), vc.to(DEV)
+
+
+def plain_cache(ops, kc, vc):
+    """Pages as the kernels keep them -> the plain order, on the CPU."""
+    if ops.cache_tiled(kc.dtype, kc.shape[3], kc.shape[2]):
+        return R.untile_cache(kc.cpu(), vc.cpu())
+    return kc.cpu(), vc.cpu()
+
+
 def close(got, want, atol, rtol=0.0):
     got = got.float().cpu()
     want = want.float().cpu()
@@ -275,7 +289,7 @@ def test_rope_append(ops, dtype, h, g, d, rd, inter):
         assert torch.equal(vc.cpu(), vc_r), "values are copied, not changed"
 
 
-@pytest.mark.parametrize("h,g,d,rd,page", [(8, 2, 128, 128, 64), (6, 3, 64, 32, 16), (4, 4, 48, 48, 32), (5, 1, 80, 16, 16)])
+@pytest.mark.parametrize("h,g,d,rd,page", [(8, 2, 128, 128, 64), (6, 3, 64, 32, 16), (4, 4, 48, 48, 32), (5, 1, 80, 16, 16), (6, 3, 64, 32, 128)])
 def test_rope_append_prompt_portions(ops, h, g, d, rd, page):
     """Many bfloat16 tokens: portions whose slots run on from a multiple of 8 (values stored
     as 16-byte pieces), portions that start anywhere, scattered single tokens, a token count
@@ -296,17 +310,18 @@ def test_rope_append_prompt_portions(ops, h, g, d, rd, page):
     cos, sin = _tables(rd, 200)
     positions = torch.tensor(positions, dtype=torch.int32, device=DEV)
     slots = torch.tensor(slots, dtype=torch.int32, device=DEV)
-    kc = rnd((n_pages, g, page, d), torch.bfloat16, 41)
-    vc = rnd((n_pages, g, d, page), torch.bfloat16, 42)
-    kc_r, vc_r, qkv_r = kc.cpu().clone(), vc.cpu().clone(), qkv.cpu().clone()
+    kc_r, vc_r = rnd((n_pages, g, page, d), torch.bfloat16, 41).cpu(), rnd((n_pages, g, d, page), torch.bfloat16, 42).cpu()
+    kc, vc = device_cache(ops, kc_r.clone(), vc_r.clone())
+    qkv_r = qkv.cpu().clone()
     ops.rope_append(qkv, h, g, d, positions, cos, sin, rd, False, kc, vc, slots, page)
     R.rope_append(qkv_r, h, g, d, positions.cpu(), cos.cpu(), sin.cpu(), rd, False, kc_r, vc_r, slots.cpu(), page)
     close(qkv.view(n, -1, d)[:, :h], qkv_r.view(n, -1, d)[:, :h], 2**-7, 2**-7)
-    close(kc, kc_r, 2**-7, 2**-7)
-    assert torch.equal(vc.cpu(), vc_r), "values are copied, not changed"
+    kc_p, vc_p = plain_cache(ops, kc, vc)
+    close(kc_p, kc_r, 2**-7, 2**-7)
+    assert torch.equal(vc_p, vc_r), "values are copied, not changed"
     # the same rows one token at a time (the scalar kernel) give the same bits
     qkv1 = rnd((n, (h + 2 * g) * d), torch.bfloat16, 40)
-    kc1, vc1 = rnd((n_pages, g, page, d), torch.bfloat16, 41), rnd((n_pages, g, d, page), torch.bfloat16, 42)
+    kc1, vc1 = device_cache(ops, rnd((n_pages, g, page, d), torch.bfloat16, 41), rnd((n_pages, g, d, page), torch.bfloat16, 42))
     for i in range(n):
         ops.rope_append(qkv1[i : i + 1], h, g, d, positions[i : i + 1], cos, sin, rd, False, kc1, vc1, slots[i : i + 1], page)
     assert torch.equal(qkv1.view(n, -1, d)[:, :h], qkv.view(n, -1, d)[:, :h]) and torch.equal(kc1, kc) and torch.equal(vc1, vc)
@@ -349,7 +364,8 @@ def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True,
     n = hb.n_tokens
     q = (torch.randn((n, h * d), generator=gen) * 1.5).to(dtype)
     scale = 1.0 / math.sqrt(d)
-    got = ops.attention(q.to(DEV), h, g, d, kc.to(DEV), vc.to(DEV), page, scale, window, ctx, 0, ctx.arrays["tiles"], ctx.arrays["long_tiles"], plan=plan, long_plan=long_plan)
+    kc_d, vc_d = device_cache(ops, kc, vc)
+    got = ops.attention(q.to(DEV), h, g, d, kc_d, vc_d, page, scale, window, ctx, 0, ctx.arrays["tiles"], ctx.arrays["long_tiles"], plan=plan, long_plan=long_plan)
     want = R.attention(q.float(), h, g, d, kc.float(), vc.float(), page, scale, window, ctx_cpu, 0, None)
     return got, want
 
@@ -372,6 +388,7 @@ def test_attention_generic_bf16(ops, h, g, d, page):
 
 @pytest.mark.parametrize("h,g,d,page", [
     (8, 2, 128, 64), (6, 3, 64, 16), (4, 4, 64, 32), (32, 1, 128, 16), (5, 1, 64, 48), (24, 8, 128, 64), (40, 2, 64, 16),
+    (4, 4, 64, 128), (12, 3, 128, 192),
 ])
 @pytest.mark.parametrize("window", [0, 40])
 def test_attention_mfma(ops, h, g, d, page, window):
@@ -389,19 +406,20 @@ def test_attention_mfma_long_context_splits(ops):
 
 
 @pytest.mark.parametrize("plan", [(1, 1), (4, 1), (1, 5), (4, 3), (4, 7)])
-@pytest.mark.parametrize("d", [64, 128])
-def test_attention_mfma_every_way_of_dividing_keys(ops, plan, d):
+@pytest.mark.parametrize("d,page", [(64, 32), (128, 32), (64, 64), (128, 128)])
+def test_attention_mfma_every_way_of_dividing_keys(ops, plan, d, page):
     """Keys divided among the waves of a workgroup, among workgroups, or both, give the
     same result; spans include ones with fewer key blocks than waves (idle waves hold
-    an empty part) and windows that cut the first block."""
+    an empty part) and windows that cut the first block.  Pages of 32 tokens are plain,
+    those of 64 and 128 tiled."""
     spans = [(1500, 1), (900, 3), (0, 2), (63, 1), (64, 1), (200, 2)]
     for window in (0, 700, 33):
-        got, want = _attention_case(ops, torch.bfloat16, 8, 2, d, 32, spans, window, seed=16, n_pages=96, plan=plan)
+        got, want = _attention_case(ops, torch.bfloat16, 8, 2, d, page, spans, window, seed=16, n_pages=3072 // page + 6, plan=plan)
         close(got, want, 2e-2, 2**-6)
 
 
 @pytest.mark.parametrize("splits", [1, 2, 5, 16])
-@pytest.mark.parametrize("h,g,d,page", [(8, 2, 128, 64), (6, 3, 64, 16), (32, 1, 128, 32)])
+@pytest.mark.parametrize("h,g,d,page", [(8, 2, 128, 64), (6, 3, 64, 16), (32, 1, 128, 32), (6, 2, 64, 128)])
 def test_attention_long_spans_with_split_keys(ops, splits, h, g, d, page):
     """Portions of prompts against a long cached context, the keys split across workgroups
     and merged: spans that end a tile early, a window, more splits than some tiles have key
@@ -460,7 +478,8 @@ def test_attention_far_key_stands_out(ops):
             arrays={kk: torch.from_numpy(np.ascontiguousarray(vv)).to(DEV) for kk, vv in arrays.items()},
             max_ctx=hb.max_ctx,
         )
-        got = ops.attention(q.to(dtype).to(DEV), h, g, d, kc.to(DEV), vc.to(DEV), page, 1.0 / math.sqrt(d), 0, ctx, 0, ctx.arrays["tiles"])
+        kc_d, vc_d = device_cache(ops, kc, vc)
+        got = ops.attention(q.to(dtype).to(DEV), h, g, d, kc_d, vc_d, page, 1.0 / math.sqrt(d), 0, ctx, 0, ctx.arrays["tiles"])
         head1 = got.view(h, d)[1].float().cpu()
         close(head1, v[far, 0].to(dtype).float(), 2e-2, 2**-6)
 
@@ -567,6 +586,26 @@ def test_sample_frequencies(ops):
     p = torch.softmax(logits[0].cpu().double() / temperature, dim=0)
     chi2 = ((counts - draws * p) ** 2 / (draws * p)).sum().item()
     assert chi2 < 40.0, chi2  # 11 degrees of freedom: 40 is beyond the 99.99th percentile
+
+
+def test_tiled_pages_layout(ops):
+    """Which pages are tiled, and that the description of the order which the tests work
+    from is the one the kernels write: a token's key and value land where it says."""
+    assert ops.cache_tiled(torch.bfloat16, 128, 64) and ops.cache_tiled(torch.bfloat16, 64, 192)
+    assert not ops.cache_tiled(torch.float32, 128, 64) and not ops.cache_tiled(torch.bfloat16, 128, 32)
+    assert not ops.cache_tiled(torch.bfloat16, 48, 64) and not ops.cache_tiled(torch.bfloat16, 256, 64)
+    h, g, d, page = 2, 1, 64, 128
+    cos, sin = _tables(d, 4)
+    for slot in (0, 5, 37, 64, 127, 128 + 70):
+        qkv = rnd((1, (h + 2 * g) * d), torch.bfloat16, slot)
+        kc = torch.zeros((2, g, page, d), dtype=torch.bfloat16, device=DEV)
+        vc = torch.zeros((2, g, d, page), dtype=torch.bfloat16, device=DEV)
+        want_k, want_v = qkv[0, h * d : (h + 1) * d].clone(), qkv[0, (h + 1) * d :].clone()
+        ops.rope_append(qkv, h, g, d, torch.zeros(1, dtype=torch.int32, device=DEV), cos, sin, d, False, kc, vc,
+                        torch.tensor([slot], dtype=torch.int32, device=DEV), page)  # position 0: no rotation
+        kp, vp = R.untile_cache(kc.cpu(), vc.cpu())
+        assert torch.equal(kp[slot // page, 0, slot % page], want_k.cpu()) and kp.ne(0).sum() == want_k.ne(0).sum()
+        assert torch.equal(vp[slot // page, 0, :, slot % page], want_v.cpu()) and vp.ne(0).sum() == want_v.ne(0).sum()
 
 
 def test_machine_probes_run_and_refuse_bad_sizes(ops):

@@ -62,6 +62,36 @@ __device__ __forceinline__ bf16_t from_f32<bf16_t>(float x) {
 
 constexpr int kWave = 64;
 
+// ------------------------------------------------------------------ layout of a cache page
+// A page holds, for every kv head, a slab of page_size x head_dim keys and one of values.
+// Plain slabs: keys [slot][dim], values transposed [dim][slot].
+// Tiled slabs (bfloat16, a head size the matrix-core attention takes, pages of a multiple of
+// 64 tokens): the slab is cut into blocks of 64 slots, and a block is stored as the 16-byte
+// pieces that the matrix-core attention loads, in the order of the lanes that load them, so
+// that one wave-wide load reads 1 KiB of consecutive memory:
+//   keys:   piece (((u*2 + sb) * head_dim/32 + ks) * 4 + g) * 16 + r holds dims 32ks + 8g .. 8g+7
+//           of slot 32u + 8(r/4) + 4sb + r%4 (the row order of the two score products of a
+//           group of 32 keys),
+//   values: piece ((u * head_dim/16 + dt) * 4 + g) * 16 + r holds slots 32u + 8g .. 8g+7 of dim
+//           16dt + r.
+// Writers (rotary + append) and readers (the attention kernels) go through these functions.
+__host__ __device__ inline bool cache_is_tiled(int dtype, int head_dim, int page_size) {
+  return dtype == YK_BF16 && (head_dim == 64 || head_dim == 128) && page_size % 64 == 0;
+}
+// element offsets within a slab
+__host__ __device__ inline size_t cache_k_offset(bool tiled, int page_size, int head_dim, int slot, int d) {
+  if (!tiled) return static_cast<size_t>(slot) * head_dim + d;
+  const int j = slot % 64, u = j / 32, r = 4 * ((j % 32) / 8) + j % 4, sb = (j % 8) / 4;
+  const int piece = (((u * 2 + sb) * (head_dim / 32) + d / 32) * 4 + (d % 32) / 8) * 16 + r;
+  return static_cast<size_t>(slot / 64) * 64 * head_dim + piece * 8 + d % 8;
+}
+__host__ __device__ inline size_t cache_v_offset(bool tiled, int page_size, int head_dim, int slot, int d) {
+  if (!tiled) return static_cast<size_t>(d) * page_size + slot;
+  const int j = slot % 64, u = j / 32, g = (j % 32) / 8;
+  const int piece = ((u * (head_dim / 16) + d / 16) * 4 + g) * 16 + d % 16;
+  return static_cast<size_t>(slot / 64) * 64 * head_dim + piece * 8 + j % 8;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);

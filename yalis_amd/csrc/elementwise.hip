@@ -25,7 +25,10 @@ int yk_check_launch(const char* what) {
   return 0;
 }
 extern "C" const char* yk_last_error() { return yk_error_slot().c_str(); }
-extern "C" int yk_abi_version() { return 5; }
+extern "C" int yk_abi_version() { return 6; }
+
+// Whether the pages of such a cache are stored tiled (cache_is_tiled).
+extern "C" int yk_cache_tiled(int dtype, int head_dim, int page_size) { return cache_is_tiled(dtype, head_dim, page_size) ? 1 : 0; }
 
 // ------------------------------------------------------------------------- embedding
 // out[n, :] = float(table[ids[n], :])
@@ -316,8 +319,9 @@ extern "C" int yk_add_rmsnorm(float* residual, const void* delta, int delta_dtyp
 // then n_kv key heads, then n_kv value heads, each of head_dim elements; with n_splits > 1
 // `src` holds the unreduced float32 K slices of the projection and they are summed here.
 // Query heads are rotated into `q_out` (which may be `src` itself); key heads are rotated
-// and stored at the token's slot of the key pages [page][kv_head][page_size][head_dim];
-// value heads are stored transposed in the value pages [page][kv_head][head_dim][page_size].
+// and stored at the token's slot of the key pages [page][kv_head][page_size x head_dim];
+// value heads are stored in the value pages [page][kv_head][head_dim x page_size] (within a
+// slab plain or tiled: cache_k_offset, cache_v_offset).
 // n_kv may be 0 (rotate queries only).  Rotation of a pair (a, b) by the angle of
 // (position, pair index i): a' = a cos - b sin, b' = b cos + a sin; pairs are
 // (i, i + rotary_dim/2) ("half") or (2i, 2i + 1) ("interleaved"); elements beyond
@@ -371,26 +375,32 @@ __global__ void rope_append_kernel(const TS* src, int n_splits, size_t split_str
     return a;
   };
   const bool is_q = h < n_heads;
-  T* dst;
+  const bool tiled = cache_is_tiled(sizeof(T) == 2 ? YK_BF16 : YK_F32, head_dim, page_size);
+  const size_t slab = static_cast<size_t>(page_size) * head_dim;
+  T* dst;   // the query row, or the key slab of the token's page
+  int off = 0;  // the token's slot within its page
   if (is_q) {
     dst = q_out + static_cast<size_t>(n) * q_stride + static_cast<size_t>(h) * head_dim;
   } else {
     const int slot = slots[n];
     const size_t page = static_cast<size_t>(slot / page_size);
-    const int off = slot % page_size;
+    off = slot % page_size;
     const int g = h - n_heads;
-    dst = k_cache + ((page * n_kv + g) * page_size + off) * head_dim;
-    // the value head of the same group, transposed
-    T* vdst = v_cache + (page * n_kv + g) * head_dim * page_size + off;
+    dst = k_cache + (page * n_kv + g) * slab;
+    // the value head of the same group
+    T* vdst = v_cache + (page * n_kv + g) * slab;
     const int vbase = (n_heads + n_kv + g) * head_dim;
     for (int d = threadIdx.x; d < head_dim; d += 2 * blockDim.x) {
       const int d2 = d + blockDim.x;  // this thread's second element, when there is one
       float va, vb;
       value2(vbase + d, vbase + min(d2, head_dim - 1), va, vb);
-      vdst[static_cast<size_t>(d) * page_size] = from_f32<T>(va);
-      if (d2 < head_dim) vdst[static_cast<size_t>(d2) * page_size] = from_f32<T>(vb);
+      vdst[cache_v_offset(tiled, page_size, head_dim, off, d)] = from_f32<T>(va);
+      if (d2 < head_dim) vdst[cache_v_offset(tiled, page_size, head_dim, off, d2)] = from_f32<T>(vb);
     }
   }
+  auto put = [&](int d, float v) {
+    dst[is_q ? static_cast<size_t>(d) : cache_k_offset(tiled, page_size, head_dim, off, d)] = from_f32<T>(v);
+  };
   const int base = h * head_dim;
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
     const int ia = interleaved ? 2 * i : i;
@@ -398,10 +408,10 @@ __global__ void rope_append_kernel(const TS* src, int n_splits, size_t split_str
     float a, b;
     value2(base + ia, base + ib, a, b);
     const float c = cs[i], s = sn[i];
-    dst[ia] = from_f32<T>(rot_first(a, b, c, s));
-    dst[ib] = from_f32<T>(rot_second(a, b, c, s));
+    put(ia, rot_first(a, b, c, s));
+    put(ib, rot_second(a, b, c, s));
   }
-  for (int d = rotary_dim + threadIdx.x; d < head_dim; d += blockDim.x) dst[d] = from_f32<T>(value(base + d));
+  for (int d = rotary_dim + threadIdx.x; d < head_dim; d += blockDim.x) put(d, value(base + d));
 }
 
 // The same for many tokens of plain bfloat16 rows with "half" pairs: a workgroup takes
@@ -438,6 +448,8 @@ __global__ __launch_bounds__(64) void rope_append_vec_kernel(
   const int n0 = blockIdx.x * ROPE_TOK, h = blockIdx.y;
   const int n_here = min(ROPE_TOK, n_tokens - n0);
   const int half = rotary_dim / 2;
+  const bool tiled = cache_is_tiled(YK_BF16, head_dim, page_size);
+  const size_t slab = static_cast<size_t>(page_size) * head_dim;
   if (h >= n_heads + n_kv) {
     // value head g of these tokens, transposed into the pages
     const int g = h - n_heads - n_kv;
@@ -452,7 +464,7 @@ __global__ __launch_bounds__(64) void rope_append_vec_kernel(
         v[t] = src[static_cast<size_t>(n0 + min(t, n_here - 1)) * src_stride + vbase + d];
       if (together) {
         const size_t page = static_cast<size_t>(slot0 / page_size);
-        bf16_t* vdst = v_cache + ((page * n_kv + g) * head_dim + d) * page_size + slot0 % page_size;
+        bf16_t* vdst = v_cache + (page * n_kv + g) * slab + cache_v_offset(tiled, page_size, head_dim, slot0 % page_size, d);
         uint4 w;
         w.x = v[0] | (static_cast<uint32_t>(v[1]) << 16);
         w.y = v[2] | (static_cast<uint32_t>(v[3]) << 16);
@@ -463,7 +475,7 @@ __global__ __launch_bounds__(64) void rope_append_vec_kernel(
         for (int t = 0; t < n_here; ++t) {
           const int slot = slots[n0 + t];
           const size_t page = static_cast<size_t>(slot / page_size);
-          v_cache[((page * n_kv + g) * head_dim + d) * page_size + slot % page_size] = v[t];
+          v_cache[(page * n_kv + g) * slab + cache_v_offset(tiled, page_size, head_dim, slot % page_size, d)] = v[t];
         }
       }
     }
@@ -477,14 +489,18 @@ __global__ __launch_bounds__(64) void rope_append_vec_kernel(
     const int t = item / per_tok, pc = item % per_tok;
     const int n = n0 + t;
     const bf16_t* row = src + static_cast<size_t>(n) * src_stride + static_cast<size_t>(h) * head_dim;
-    bf16_t* dst;
+    bf16_t* dst;  // the query row, or the key slab of the token's page
+    int off = 0;
     if (is_q) {
       dst = q_out + static_cast<size_t>(n) * q_stride + static_cast<size_t>(h) * head_dim;
     } else {
       const int slot = slots[n];
       const size_t page = static_cast<size_t>(slot / page_size);
-      dst = k_cache + ((page * n_kv + (h - n_heads)) * page_size + slot % page_size) * head_dim;
+      off = slot % page_size;
+      dst = k_cache + (page * n_kv + (h - n_heads)) * slab;
     }
+    // where the 8 elements from d on go (they stay together in either layout)
+    auto at = [&](int d) { return dst + (is_q ? static_cast<size_t>(d) : cache_k_offset(tiled, page_size, head_dim, off, d)); };
     if (pc < pieces) {
       int pos = positions[n];
       pos = pos < 0 ? 0 : (pos >= max_positions ? max_positions - 1 : pos);
@@ -500,11 +516,11 @@ __global__ __launch_bounds__(64) void rope_append_vec_kernel(
       }
       uint4 oa, ob;
       rope_rotate8(a, b, c, s_, oa, ob);
-      *reinterpret_cast<uint4*>(dst + 8 * pc) = oa;
-      *reinterpret_cast<uint4*>(dst + half + 8 * pc) = ob;
+      *reinterpret_cast<uint4*>(at(8 * pc)) = oa;
+      *reinterpret_cast<uint4*>(at(half + 8 * pc)) = ob;
     } else {
       const int d = rotary_dim + 8 * (pc - pieces);
-      *reinterpret_cast<uint4*>(dst + d) = *reinterpret_cast<const uint4*>(row + d);
+      *reinterpret_cast<uint4*>(at(d)) = *reinterpret_cast<const uint4*>(row + d);
     }
   }
 }

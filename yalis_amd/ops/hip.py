@@ -42,6 +42,7 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 _SIGNATURES = {
     "yk_abi_version": ([], _c_int),
+    "yk_cache_tiled": ([_c_int, _c_int, _c_int], _c_int),
     "yk_embed": ([_vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_add_rmsnorm": (
         [_vp, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp],
@@ -132,7 +133,7 @@ class HipOps:
             fn = getattr(self.lib, name)
             fn.argtypes = args
             fn.restype = res
-        if self.lib.yk_abi_version() != 5:
+        if self.lib.yk_abi_version() != 6:
             raise KernelError("kernel library and bindings disagree; rebuild (python -c 'import __graft_entry__ as g; g.build()')")
         self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
         # the quick way to the current stream's handle, where this torch has it
@@ -517,6 +518,13 @@ class HipOps:
             )
         )
         return out
+
+    def cache_tiled(self, dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
+        """Whether pages of this kind are kept in the order the matrix-core attention loads
+        them rather than as plain [slot, dim] keys and [dim, slot] values.  The kernels that
+        write and read pages decide alike from the same three numbers; code that fills or
+        inspects pages by hand (tests) has to ask."""
+        return bool(self.lib.yk_cache_tiled(_code(dtype), int(head_dim), int(page_size)))
 
     # ------------------------------------------------------------------ machine probes
     def probe_stream_read(self, data: torch.Tensor, workgroups: int, sink: torch.Tensor, nontemporal: bool = False) -> None:
