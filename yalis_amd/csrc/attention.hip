@@ -182,7 +182,7 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // 1 KiB of consecutive memory instead of 16 rows x 64 bytes (measured at 64 requests of 1,024
 // tokens: 46 us a layer against 58).
 template <int D, int W, bool TILED>
-__global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
+__global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ block_table, int table_width,
@@ -207,9 +207,17 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
   const int per_split = (kb_hi - kb_lo + n_splits - 1) / n_splits;
   const int wg_lo = kb_lo + blockIdx.z * per_split;
   const int wg_hi = min(kb_hi, wg_lo + per_split);
-  const int per_wave = (max(0, wg_hi - wg_lo) + W - 1) / W;
-  const int my_lo = wg_lo + wave * per_wave;
-  const int my_hi = min(wg_hi, my_lo + per_wave);
+  // the waves divide the workgroup's keys in halves of a block (32 keys: one group of the two
+  // score products), so that the longest share is at most half a block above the mean; a half
+  // beyond the last key is nobody's.  A half that is not the wave's own is not loaded: its keys
+  // and values stand as zeros in the products and its scores are masked.
+  const int h_lo = wg_lo * 2, h_hi = min(wg_hi * 2, (hi + 31) / 32);
+  const int per_wave = (max(0, h_hi - h_lo) + W - 1) / W;
+  const int my_hlo = h_lo + wave * per_wave;
+  const int my_hhi = min(h_hi, my_hlo + per_wave);
+  const int my_lo = my_hlo / 2;
+  const int my_hi = my_hlo < my_hhi ? (my_hhi + 1) / 2 : my_lo;
+  auto mine = [&](int kb, int u) { return 2 * kb + u >= my_hlo && 2 * kb + u < my_hhi; };
   const int32_t* bt = block_table + static_cast<size_t>(seq) * table_width;
   const int last_page_col = min(table_width - 1, (hi - 1) / page_size);
 
@@ -236,19 +244,35 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
 
   AFrag8 kf[2][2][KS];
 #define ATT_LOAD_K(KB)                                                                            \
+  {                                                                                                \
   if (TILED) {                                                                                     \
     const int key0 = (KB) * 64;                                                                    \
     const bf16_t* kp = k_cache + (static_cast<size_t>(page_of(key0)) * n_kv + g) * page_size * D + \
                        static_cast<size_t>(key0 % page_size) * D + 8 * lane;                       \
-    _Pragma("unroll") for (int u = 0; u < 2; ++u) _Pragma("unroll") for (int sb = 0; sb < 2; ++sb) \
-    _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                              \
-        kf[u][sb][ks].u = *reinterpret_cast<const u32x4_t*>(kp + ((u * 2 + sb) * KS + ks) * 512);  \
+    _Pragma("unroll") for (int u = 0; u < 2; ++u) {                                                \
+      if (mine((KB), u)) {                                                                         \
+        _Pragma("unroll") for (int sb = 0; sb < 2; ++sb)                                           \
+        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                          \
+            kf[u][sb][ks].u = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(kp + ((u * 2 + sb) * KS + ks) * 512)); \
+      } else {                                                                                     \
+        _Pragma("unroll") for (int sb = 0; sb < 2; ++sb)                                           \
+        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) kf[u][sb][ks].u = zero4;                 \
+      }                                                                                            \
+    }                                                                                              \
   } else {                                                                                         \
-  _Pragma("unroll") for (int u = 0; u < 2; ++u) _Pragma("unroll") for (int sb = 0; sb < 2; ++sb) { \
-    const int key = (KB) * 64 + 32 * u + krow + 4 * sb;                                           \
-    const bf16_t* kp = k_cache + ((static_cast<size_t>(page_of(key)) * n_kv + g) * page_size + key % page_size) * D + 8 * gq; \
-    _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                             \
-        kf[u][sb][ks].u = *reinterpret_cast<const u32x4_t*>(kp + 32 * ks);                        \
+    _Pragma("unroll") for (int u = 0; u < 2; ++u) {                                                \
+      if (mine((KB), u)) {                                                                         \
+        _Pragma("unroll") for (int sb = 0; sb < 2; ++sb) {                                         \
+          const int key = (KB) * 64 + 32 * u + krow + 4 * sb;                                     \
+          const bf16_t* kp = k_cache + ((static_cast<size_t>(page_of(key)) * n_kv + g) * page_size + key % page_size) * D + 8 * gq; \
+          _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                       \
+              kf[u][sb][ks].u = *reinterpret_cast<const u32x4_t*>(kp + 32 * ks);                  \
+        }                                                                                          \
+      } else {                                                                                     \
+        _Pragma("unroll") for (int sb = 0; sb < 2; ++sb)                                           \
+        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) kf[u][sb][ks].u = zero4;                 \
+      }                                                                                            \
+    }                                                                                              \
   }                                                                                                \
   }
 
@@ -256,23 +280,35 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
   for (int kb = my_lo; kb < my_hi; ++kb) {
     // values of this block: lane (r, gq) holds 8 consecutive keys of value row 16*dt + r
     AFrag8 vf[2][DT];
+    const bool mine0 = mine(kb, 0), mine1 = mine(kb, 1);
     if (TILED) {
       const int key0 = kb * 64;
       const bf16_t* vp = v_cache + (static_cast<size_t>(page_of(key0)) * n_kv + g) * D * page_size +
                          static_cast<size_t>(key0 % page_size) * D + 8 * lane;
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
+      for (int u = 0; u < 2; ++u) {
+        if (u == 0 ? mine0 : mine1) {
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-          vf[u][dt].u = *reinterpret_cast<const u32x4_t*>(vp + (u * DT + dt) * 512);
+          for (int dt = 0; dt < DT; ++dt)
+            vf[u][dt].u = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(vp + (u * DT + dt) * 512));
+        } else {
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) vf[u][dt].u = zero4;
+        }
+      }
     } else {
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        const int key = kb * 64 + 32 * u + 8 * gq;
-        const bf16_t* vp = v_cache + (static_cast<size_t>(page_of(key)) * n_kv + g) * D * page_size + key % page_size;
+        if (u == 0 ? mine0 : mine1) {
+          const int key = kb * 64 + 32 * u + 8 * gq;
+          const bf16_t* vp = v_cache + (static_cast<size_t>(page_of(key)) * n_kv + g) * D * page_size + key % page_size;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-          vf[u][dt].u = *reinterpret_cast<const u32x4_t*>(vp + static_cast<size_t>(16 * dt + r) * page_size);
+          for (int dt = 0; dt < DT; ++dt)
+            vf[u][dt].u = *reinterpret_cast<const u32x4_t*>(vp + static_cast<size_t>(16 * dt + r) * page_size);
+        } else {
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) vf[u][dt].u = zero4;
+        }
       }
     }
     // scores
@@ -290,7 +326,7 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
     float tmax = -INFINITY;
     // a block that every column sees whole needs no mask (columns that stand for nothing
     // compute on zeros and are never stored)
-    const bool whole = kb * 64 + 63 <= pos0 && (window == 0 || kb * 64 >= max(0, pos0 + ntok - window));
+    const bool whole = mine0 && mine1 && kb * 64 + 63 <= pos0 && (window == 0 || kb * 64 >= max(0, pos0 + ntok - window));
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -299,7 +335,7 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
         for (int i = 0; i < 4; ++i) {
           if (!whole) {
             const int key = kb * 64 + 32 * u + 8 * gq + 4 * sb + i;
-            const bool ok = col_ok && key <= pos_c && key >= lo_c;
+            const bool ok = col_ok && key <= pos_c && key >= lo_c && (u == 0 ? mine0 : mine1);
             if (!ok) s[u][sb][i] = -INFINITY;
           }
           tmax = fmaxf(tmax, s[u][sb][i]);
