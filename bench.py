@@ -114,7 +114,8 @@ def main() -> int:
     ap.add_argument("--prefill-len", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--only-prefill", action="store_true", help="measure the prefill only (for profiling)")
-    ap.add_argument("--mixed", action="store_true", help="measure mixed steps instead: 32 decode streams beside 512-token portions of 4,096-token prompts")
+    ap.add_argument("--mixed", action="store_true", help="measure mixed steps instead: 32 decode streams beside portions of 4,096-token prompts")
+    ap.add_argument("--portion", type=int, default=480, help="tokens of a prompt portion in --mixed steps (with the 32 decoded tokens: 512 rows, as the scheduler cuts under a budget of 512)")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel (for hardware counters)")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="8b", help="layer sizes (default: the 8B shape of the headline)")
     ap.add_argument("--probe", action="store_true", help="measure instead what a plain streaming read and a plain matrix-core loop reach on this card")
@@ -209,9 +210,11 @@ def main() -> int:
         return weight_bytes + batch * c * 2 + kv
 
     if args.mixed:
-        # 32 requests decode while 4,096-token prompts arrive in portions of 512 tokens: every
-        # step holds 32 single tokens and one portion (the last portion's row is sampled too)
-        n_dec, portion, plen = 32, 512, 4096
+        # 32 requests decode while 4,096-token prompts arrive in portions: every step holds 32
+        # single tokens and one portion (the last portion's row is sampled too).  The rows of a
+        # step's products are the step's tokens: 480 + 32 = 512 rows fill the vendor library's
+        # tiles, 512 + 32 = 544 rows cost a fifth tile row for a quarter of its work.
+        n_dec, portion, plen = 32, args.portion, 4096
         toks = []
         for r in range(n_dec):
             assert runner.admit(r)
@@ -222,11 +225,11 @@ def main() -> int:
         times, kv_tokens = [], []
         for rid in (100, 101, 102):  # the first prompt warms up
             assert runner.admit(rid)
-            for c0 in range(0, plen, portion):
+            for c0 in range(0, plen - portion + 1, portion):
                 for r in range(n_dec):
                     assert runner.reserve(r, 1)
                 assert runner.reserve(rid, portion)
-                last = c0 + portion == plen
+                last = c0 + 2 * portion > plen
                 entries = [StepEntry(r, [toks[r]], [0]) for r in range(n_dec)]
                 entries.append(StepEntry(rid, prompt[c0 : c0 + portion], [portion - 1] if last else []))
                 ctx_tokens = sum(runner.cached[r] + 1 for r in range(n_dec)) + c0 + portion
