@@ -10,23 +10,6 @@
 
 #include "common.h"
 
-// ------------------------------------------------------------------ error reporting
-std::string& yk_error_slot() {
-  static thread_local std::string s;
-  return s;
-}
-int yk_fail(const std::string& msg) {
-  yk_error_slot() = msg;
-  return -1;
-}
-int yk_check_launch(const char* what) {
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return yk_fail(std::string(what) + ": " + hipGetErrorString(e));
-  return 0;
-}
-extern "C" const char* yk_last_error() { return yk_error_slot().c_str(); }
-extern "C" int yk_abi_version() { return 6; }
-
 // Whether the pages of such a cache are stored tiled (cache_is_tiled).
 extern "C" int yk_cache_tiled(int dtype, int head_dim, int page_size) { return cache_is_tiled(dtype, head_dim, page_size) ? 1 : 0; }
 

@@ -1,8 +1,9 @@
 """Compiling and loading the native libraries.
 
-Two shared libraries are built from ``yalis_amd/csrc``: the host-side cache manager
-(C++, g++) and the HIP kernels for gfx950 (hipcc).  Both expose a plain C interface
-and are loaded with ctypes.  Built files go into ``yalis_amd/csrc/_build`` when that
+Shared libraries are built from ``yalis_amd/csrc``: the host-side cache manager (C++, g++)
+and the HIP kernels for gfx950 (hipcc) in three libraries, each built when first needed: the
+kernels of a model step, those that choose tokens, and the benchmark's probes.  All expose a
+plain C interface and are loaded with ctypes.  Built files go into ``yalis_amd/csrc/_build`` when that
 is writable, else into a per-user folder under the system's temporary directory.
 ``load_*`` builds on first use when no library matching the sources is there, and
 prints a line now and then while the compiler runs.
@@ -23,13 +24,14 @@ from typing import Dict, List, Sequence
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 
 HOST_SOURCES = ["cache_manager.cpp"]
-KERNEL_SOURCES = [
-    "elementwise.hip",
-    "gemm.hip",
-    "attention.hip",
-    "sampling.hip",
-    "probe.hip",
-]
+# Libraries of HIP kernels, each built and loaded when first needed: a model step needs
+# "kernels" only (so that is all a trace replay compiles), choosing tokens "sampling", the
+# benchmark's machine probes "probe".  Every library carries runtime.hip (its error slot).
+KERNEL_LIBS = {
+    "kernels": ["runtime.hip", "elementwise.hip", "gemm.hip", "attention.hip"],
+    "sampling": ["runtime.hip", "sampling.hip"],
+    "probe": ["runtime.hip", "probe.hip"],
+}
 HEADERS = ["common.h"]
 
 HIPCC_FLAGS = [
@@ -147,15 +149,16 @@ def build_host(force: bool = False) -> str:
     return lib
 
 
-def build_kernels(force: bool = False) -> str:
-    """The HIP kernels for gfx950: one object per source, compiled side by side."""
-    digest = _digest(KERNEL_SOURCES, HIPCC_FLAGS)
+def build_kernels(name: str = "kernels", force: bool = False) -> str:
+    """One library of HIP kernels for gfx950: one object per source, compiled side by side."""
+    sources = KERNEL_LIBS[name]
+    digest = _digest(sources, HIPCC_FLAGS)
     bdir = build_dir()
-    lib = os.path.join(bdir, "libyalis_kernels.so")
+    lib = os.path.join(bdir, f"libyalis_{name}.so")
     if not force and _is_current(lib, digest):
         return lib
     hipcc = _find("hipcc", ["/opt/rocm/bin/hipcc"])
-    _say(f"compiling {len(KERNEL_SOURCES)} HIP sources for gfx950 (about a minute)")
+    _say(f"compiling {len(sources)} HIP sources for gfx950 (library '{name}'; the largest takes about a minute)")
     objs: List[str] = []
     errors: List[BaseException] = []
 
@@ -167,8 +170,8 @@ def build_kernels(force: bool = False) -> str:
             errors.append(e)
 
     threads = []
-    for src in KERNEL_SOURCES:
-        obj = os.path.join(bdir, f"{os.path.splitext(src)[0]}.{os.getpid()}.o")
+    for src in sources:
+        obj = os.path.join(bdir, f"{name}_{os.path.splitext(src)[0]}.{os.getpid()}.o")
         objs.append(obj)
         th = threading.Thread(target=one, args=(src, obj))
         th.start()
@@ -186,13 +189,14 @@ def build_kernels(force: bool = False) -> str:
         os.remove(o)
     os.replace(tmp, lib)
     _write_stamp(lib, digest)
-    _say("kernels built")
+    _say(f"library '{name}' built")
     return lib
 
 
 def build_all(force: bool = True) -> None:
     build_host(force=force)
-    build_kernels(force=force)
+    for name in KERNEL_LIBS:
+        build_kernels(name, force=force)
 
 
 def load_host() -> ctypes.CDLL:
@@ -202,8 +206,8 @@ def load_host() -> ctypes.CDLL:
         return _loaded["host"]
 
 
-def load_kernels() -> ctypes.CDLL:
+def load_kernels(name: str = "kernels") -> ctypes.CDLL:
     with _lock:
-        if "kernels" not in _loaded:
-            _loaded["kernels"] = ctypes.CDLL(build_kernels())
-        return _loaded["kernels"]
+        if name not in _loaded:
+            _loaded[name] = ctypes.CDLL(build_kernels(name))
+        return _loaded[name]

@@ -80,11 +80,21 @@ _SIGNATURES = {
         [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _vp],
         _c_int,
     ),
-    "yk_argmax": ([_vp, _vp, _c_int, _c_int, _vp, _c_size_t, _vp], _c_int),
-    "yk_sample": ([_vp, _vp, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _vp], _c_int),
-    "yk_probe_stream_read": ([_vp, _c_size_t, _c_int, _c_int, _vp, _vp], _c_int),
-    "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
 }
+# the libraries that are built and loaded when first used (choosing tokens; the benchmark's probes)
+_LATER_SIGNATURES = {
+    "sampling": {
+        "yk_abi_version": ([], _c_int),
+        "yk_argmax": ([_vp, _vp, _c_int, _c_int, _vp, _c_size_t, _vp], _c_int),
+        "yk_sample": ([_vp, _vp, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _vp], _c_int),
+    },
+    "probe": {
+        "yk_abi_version": ([], _c_int),
+        "yk_probe_stream_read": ([_vp, _c_size_t, _c_int, _c_int, _vp, _vp], _c_int),
+        "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
+    },
+}
+_ABI = 6
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
 # above it the vendor library does.
@@ -127,14 +137,8 @@ class HipOps:
         if not torch.cuda.is_available():
             raise KernelError("HipOps needs a GPU: torch.cuda.is_available() is False")
         self.device = torch.device(device)
-        self.lib = load_kernels()
-        self.lib.yk_last_error.restype = ctypes.c_char_p
-        for name, (args, res) in _SIGNATURES.items():
-            fn = getattr(self.lib, name)
-            fn.argtypes = args
-            fn.restype = res
-        if self.lib.yk_abi_version() != 6:
-            raise KernelError("kernel library and bindings disagree; rebuild (python -c 'import __graft_entry__ as g; g.build()')")
+        self.lib = self._bind(load_kernels(), _SIGNATURES)
+        self._later: dict = {}
         self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
         # the quick way to the current stream's handle, where this torch has it
         self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -142,6 +146,23 @@ class HipOps:
         self._gemm_workspace: Optional[torch.Tensor] = None  # K slices of products
 
     # ------------------------------------------------------------------ helpers
+    @staticmethod
+    def _bind(lib, signatures):
+        lib.yk_last_error.restype = ctypes.c_char_p
+        for name, (args, res) in signatures.items():
+            fn = getattr(lib, name)
+            fn.argtypes = args
+            fn.restype = res
+        if lib.yk_abi_version() != _ABI:
+            raise KernelError("kernel library and bindings disagree; rebuild (python -c 'import __graft_entry__ as g; g.build()')")
+        return lib
+
+    def _library(self, name: str):
+        """A library beside the step's kernels, built and loaded at its first use."""
+        if name not in self._later:
+            self._later[name] = self._bind(load_kernels(name), _LATER_SIGNATURES[name])
+        return self._later[name]
+
     def _stream(self) -> int:
         """The raw handle of torch's current stream on this device (asked for at every
         launch: a graph capture switches streams)."""
@@ -149,9 +170,9 @@ class HipOps:
             return self._raw_stream(self._device_index)
         return torch.cuda.current_stream(self.device).cuda_stream
 
-    def _check(self, rc: int) -> None:
+    def _check(self, rc: int, lib=None) -> None:
         if rc != 0:
-            raise KernelError(self.lib.yk_last_error().decode())
+            raise KernelError((lib or self.lib).yk_last_error().decode())
 
     def _ws(self, floats: int) -> torch.Tensor:
         """Float32 scratch that grows and is reused (stream order keeps uses apart)."""
@@ -495,8 +516,9 @@ class HipOps:
             raise KernelError("argmax takes contiguous float32 logits [rows, vocab]")
         out = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device)
         ws = self._ws(64 * logits.shape[0])
-        self._check(self.lib.yk_argmax(logits.data_ptr(), out.data_ptr(), logits.shape[0], logits.shape[1],
-                                       ws.data_ptr(), ws.numel(), self._stream()))
+        lib = self._library("sampling")
+        self._check(lib.yk_argmax(logits.data_ptr(), out.data_ptr(), logits.shape[0], logits.shape[1],
+                                  ws.data_ptr(), ws.numel(), self._stream()), lib)
         return out
 
     def sample(self, logits, temperature, top_k, top_p, seeds, draws, whole_row: bool = False) -> torch.Tensor:
@@ -511,11 +533,13 @@ class HipOps:
             if t.dtype != dt or t.numel() != rows or not t.is_contiguous():
                 raise KernelError(f"sample: {name} must be {dt} with one entry per row")
         out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+        lib = self._library("sampling")
         self._check(
-            self.lib.yk_sample(
+            lib.yk_sample(
                 logits.data_ptr(), out.data_ptr(), rows, logits.shape[1], temperature.data_ptr(), top_k.data_ptr(),
                 top_p.data_ptr(), seeds.data_ptr(), draws.data_ptr(), int(bool(whole_row)), self._stream(),
-            )
+            ),
+            lib,
         )
         return out
 
@@ -530,10 +554,12 @@ class HipOps:
     def probe_stream_read(self, data: torch.Tensor, workgroups: int, sink: torch.Tensor, nontemporal: bool = False) -> None:
         """Reads every byte of ``data`` once with a plain streaming kernel (for timing);
         ``nontemporal`` marks the loads as not to be kept in the caches."""
-        self._check(self.lib.yk_probe_stream_read(data.data_ptr(), data.numel() * data.element_size(), int(workgroups),
-                                                  int(bool(nontemporal)), sink.data_ptr(), self._stream()))
+        lib = self._library("probe")
+        self._check(lib.yk_probe_stream_read(data.data_ptr(), data.numel() * data.element_size(), int(workgroups),
+                                             int(bool(nontemporal)), sink.data_ptr(), self._stream()), lib)
 
     def probe_mfma_bf16(self, workgroups: int, iterations: int, sink: torch.Tensor) -> int:
         """Issues a loop of bfloat16 matrix-core instructions from registers; returns its flop count."""
-        self._check(self.lib.yk_probe_mfma_bf16(int(workgroups), int(iterations), sink.data_ptr(), self._stream()))
+        lib = self._library("probe")
+        self._check(lib.yk_probe_mfma_bf16(int(workgroups), int(iterations), sink.data_ptr(), self._stream()), lib)
         return int(workgroups) * 4 * int(iterations) * 4 * 16384
