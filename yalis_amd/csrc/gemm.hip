@@ -210,17 +210,32 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
       SK_LOAD_X(kc + SK_KC)
     }
     __syncthreads();
+    // The operands of the steps are read from LDS ahead of the products that take them (all
+    // of the chunk's at once where the registers allow, else two steps ahead): written the
+    // plain way, one read then its product, the compiler reuses one register set and every
+    // product waits for an LDS round trip.
+    constexpr int AHEAD = MT >= 4 ? 2 : (MT == 2 ? 3 : SK_STEPS);
+    Frag8 a[SK_STEPS], b[SK_STEPS][MT];
+#define SK_READ(U)                                                                          \
+  {                                                                                          \
+    a[U].u = *reinterpret_cast<const u32x4_t*>(&wl[r][32 * (U) + 8 * g]);                    \
+    _Pragma("unroll") for (int t = 0; t < MT; ++t)                                           \
+        b[U][t].u = *reinterpret_cast<const u32x4_t*>(&xs[16 * t + r][32 * (U) + 8 * g]);    \
+  }
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) SK_READ(u)
+    __builtin_amdgcn_sched_barrier(0);  // (the scheduler would otherwise move the reads back to their products)
 #pragma unroll
     for (int u = 0; u < SK_STEPS; ++u) {
-      Frag8 a;
-      a.u = *reinterpret_cast<const u32x4_t*>(&wl[r][32 * u + 8 * g]);
-#pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        Frag8 b;
-        b.u = *reinterpret_cast<const u32x4_t*>(&xs[16 * t + r][32 * u + 8 * g]);
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[t], 0, 0, 0);
+      if (u + AHEAD < SK_STEPS) {
+        SK_READ(u + AHEAD)
+        __builtin_amdgcn_sched_barrier(0);
       }
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u].v, b[u][t].v, acc[t], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
+#undef SK_READ
   }
 #undef SK_LOAD_W
 #undef SK_LOAD_X
