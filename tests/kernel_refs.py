@@ -104,7 +104,7 @@ def attention_paged(q, k_cache, v_cache, positions, token_seq, block_table, page
 
 
 def attention(qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size, scale,
-              window, ctx, group, tiles, long_tiles=None, plan=None, long_plan=None):
+              window, ctx, group, tiles, long_tiles=None, plan=None, long_plan=None, long_col_tiles=1):
     n = qkv.shape[0]
     q = qkv.view(n, -1, head_dim)[:, :n_heads]
     out = attention_paged(
@@ -145,8 +145,12 @@ class RefOps:
     def attention_tokens_per_tile(self, n_heads, n_kv):
         return 16 // min(n_heads // n_kv, 16)
 
-    def attention_long_span_tile(self, n_heads, n_kv):
-        return 4 * self.attention_tokens_per_tile(n_heads, n_kv)
+    def attention_long_span_tile(self, n_heads, n_kv, col_tiles=1):
+        return 4 * col_tiles * self.attention_tokens_per_tile(n_heads, n_kv)
+
+    @staticmethod
+    def attention_long_col_tiles(workgroups, fewest_keys):
+        return 1
 
     embed = staticmethod(embed)
     add_rmsnorm = staticmethod(add_rmsnorm)

@@ -328,7 +328,7 @@ def test_rope_append_prompt_portions(ops, h, g, d, rd, page):
 
 
 # ------------------------------------------------------------------------- attention
-def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True, n_pages=64, plan=None, long_plan=None):
+def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True, n_pages=64, plan=None, long_plan=None, col_tiles=1):
     """spans: list of (cached tokens before the step, new tokens).  Builds pages in a
     shuffled order, fills cache for the earlier tokens, runs rope-free attention."""
     gen = torch.Generator().manual_seed(seed)
@@ -355,7 +355,8 @@ def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True,
     hb = build_host_batch(seqs, 1, page)
     tpt = ops.attention_tokens_per_tile(h, g)
     big = ops.attention_long_span_tile(h, g)
-    arrays = named_arrays(hb, {"tiles": lambda b: attention_tiles(b, tpt, 1, big), "long_tiles": lambda b: attention_tiles(b, big, big + 1, longest_first=(seed % 2 == 0))})
+    big_c = ops.attention_long_span_tile(h, g, col_tiles)  # tokens of a long tile with col_tiles column tiles a wave
+    arrays = named_arrays(hb, {"tiles": lambda b: attention_tiles(b, tpt, 1, big), "long_tiles": lambda b: attention_tiles(b, big_c, big + 1, longest_first=(seed % 2 == 0))})
     ctx = types.SimpleNamespace(
         arrays={k: torch.from_numpy(np.ascontiguousarray(v)).to(DEV) for k, v in arrays.items()},
         max_ctx=hb.max_ctx,
@@ -365,7 +366,7 @@ def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True,
     q = (torch.randn((n, h * d), generator=gen) * 1.5).to(dtype)
     scale = 1.0 / math.sqrt(d)
     kc_d, vc_d = device_cache(ops, kc, vc)
-    got = ops.attention(q.to(DEV), h, g, d, kc_d, vc_d, page, scale, window, ctx, 0, ctx.arrays["tiles"], ctx.arrays["long_tiles"], plan=plan, long_plan=long_plan)
+    got = ops.attention(q.to(DEV), h, g, d, kc_d, vc_d, page, scale, window, ctx, 0, ctx.arrays["tiles"], ctx.arrays["long_tiles"], plan=plan, long_plan=long_plan, long_col_tiles=col_tiles)
     want = R.attention(q.float(), h, g, d, kc.float(), vc.float(), page, scale, window, ctx_cpu, 0, None)
     return got, want
 
@@ -418,16 +419,26 @@ def test_attention_mfma_every_way_of_dividing_keys(ops, plan, d, page):
         close(got, want, 2e-2, 2**-6)
 
 
+@pytest.mark.parametrize("col_tiles", [1, 2])
 @pytest.mark.parametrize("splits", [1, 2, 5, 16])
 @pytest.mark.parametrize("h,g,d,page", [(8, 2, 128, 64), (6, 3, 64, 16), (32, 1, 128, 32), (6, 2, 64, 128)])
-def test_attention_long_spans_with_split_keys(ops, splits, h, g, d, page):
+def test_attention_long_spans_with_split_keys(ops, splits, h, g, d, page, col_tiles):
     """Portions of prompts against a long cached context, the keys split across workgroups
     and merged: spans that end a tile early, a window, more splits than some tiles have key
-    blocks (empty parts)."""
+    blocks (empty parts); one and two column tiles per wave (tiles of twice the tokens)."""
     spans = [(900, 70), (0, 130), (1500, 33), (40, 100)]
     for window in (0, 300):
-        got, want = _attention_case(ops, torch.bfloat16, h, g, d, page, spans, window, seed=18, n_pages=3000 // page + 8, long_plan=splits)
+        got, want = _attention_case(ops, torch.bfloat16, h, g, d, page, spans, window, seed=18, n_pages=3000 // page + 8, long_plan=splits, col_tiles=col_tiles)
         close(got, want, 2e-2, 2**-6)
+
+
+def test_attention_long_col_tiles_policy():
+    from yalis_amd.ops.hip import HipOps
+
+    assert HipOps.attention_long_col_tiles(512, 0) == 1  # a 2,048-token prompt that starts from nothing
+    assert HipOps.attention_long_col_tiles(1024, 0) == 2  # a 4,096-token one: workgroups enough to balance
+    assert HipOps.attention_long_col_tiles(512, 6144) == 2  # 2,048 tokens against 6,144 cached, 8 kv heads
+    assert HipOps.attention_long_col_tiles(128, 3584) == 1  # one 512-token portion: too few workgroups
 
 
 def test_attention_long_splits_policy():

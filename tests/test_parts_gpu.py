@@ -85,7 +85,7 @@ def _context(spans, page, group_tables, builders):
     arrays = named_arrays(hb, builders)
     return types.SimpleNamespace(
         host=hb, arrays={k: torch.from_numpy(np.ascontiguousarray(v)).to(DEV) for k, v in arrays.items()},
-        n_tokens=hb.n_tokens, n_seqs=hb.n_seqs, max_ctx=hb.max_ctx, max_qlen=hb.max_qlen,
+        n_tokens=hb.n_tokens, n_seqs=hb.n_seqs, max_ctx=hb.max_ctx, max_qlen=hb.max_qlen, memo={},
     )
 
 

@@ -447,26 +447,26 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
 }
 
 // The same arithmetic for long spans (prompt portions): a workgroup of four waves owns one
-// long tile of a request; every wave has PF_CT column tiles of 16 (consecutive tokens), so
-// the workgroup walks the keys once for 64 * PF_CT columns and every key or value operand
-// read from LDS feeds PF_CT products.  Each block of 64 keys and values is fetched from the
-// pages with coalesced loads, parked in LDS (keys in the row order the score products read
-// them, so that the reads are free of bank conflicts) and read from there by the four
-// waves; the next block's loads are in flight meanwhile.  No split of the keys: long spans
-// bring enough workgroups.  Measured on 2,048-token prompts: one column tile per wave with
-// three workgroups resident per CU (the launch bound below keeps the registers to that) is
-// the fastest; more columns per wave save LDS reads but leave too few workgroups to balance
-// the triangle of a causal prompt.
-constexpr int PF_CT = 1;
-
-template <int D, bool TILED>
-__global__ __launch_bounds__(256, 3) void attn_mfma_prefill_kernel(
+// long tile of a request; every wave has CT column tiles of 16 (consecutive tokens), so the
+// workgroup walks the keys once for 64 * CT columns and every key or value operand read from
+// LDS feeds CT products.  Each block of 64 keys and values is fetched from the pages with
+// coalesced loads, parked in LDS (keys in the row order the score products read them, so
+// that the reads are free of bank conflicts) and read from there by the four waves; the next
+// block's loads are in flight meanwhile.  The keys are split across workgroups only where
+// few tiles meet a long context.
+// CT is the caller's choice, with the tiles it built: one column tile per wave (three
+// workgroups a CU) balances the triangle of a prompt that starts from nothing; two (224
+// registers, two workgroups a CU) stage every block through LDS for twice the columns and
+// win where many tiles each meet thousands of keys (measured on the 8B shape: 2,048 tokens
+// against 8,192 cached 383 us against 499, a whole 2,048-token prompt 99 us against 80).
+template <int D, bool TILED, int CT>
+__global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ block_table, int table_width,
     int page_size, int n_heads, int n_kv, int hpt, int chunks, float scale_log2, int window,
     int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml) {
-  constexpr int KS = D / 32, DT = D / 16, CT = PF_CT;
+  constexpr int KS = D / 32, DT = D / 16;
   constexpr int KROW = D + 8;   // bf16 elements per parked key row
   constexpr int VROW = 64 + 8;  // bf16 elements per parked value row
   constexpr int PP = D / 32;    // 16-byte pieces of keys (and of values) per thread and block
@@ -787,9 +787,10 @@ extern "C" int yk_attn_heads_per_tile(int n_heads, int n_kv) {
 extern "C" int yk_attn_tokens_per_tile(int n_heads, int n_kv) {
   return 16 / yk_attn_heads_per_tile(n_heads, n_kv);
 }
-// Tokens of one long tile (a workgroup of the long-span kernel): four waves of PF_CT column tiles.
-extern "C" int yk_attn_long_tile_tokens(int n_heads, int n_kv) {
-  return 4 * PF_CT * yk_attn_tokens_per_tile(n_heads, n_kv);
+// Tokens of one long tile (a workgroup of the long-span kernel): four waves of col_tiles (1 or 2)
+// column tiles.
+extern "C" int yk_attn_long_tile_tokens(int n_heads, int n_kv, int col_tiles) {
+  return 4 * col_tiles * yk_attn_tokens_per_tile(n_heads, n_kv);
 }
 
 // Floats of workspace for a launch with n_splits > 1: outputs, then (max, sum) pairs.
@@ -807,9 +808,10 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
                                     const void* v_cache, const int32_t* tiles, int n_tiles,
                                     const int32_t* block_table, int table_width, int page_size,
                                     int head_dim, int n_heads, int n_kv, float scale, int window,
-                                    int n_splits, float* workspace, size_t workspace_floats,
+                                    int n_splits, int col_tiles, float* workspace, size_t workspace_floats,
                                     hipStream_t stream) {
   YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_mfma_prefill: bad head counts");
+  YK_REQUIRE(col_tiles == 1 || col_tiles == 2, "attn_mfma_prefill: a wave has 1 or 2 column tiles");
   YK_REQUIRE(yk_attn_mfma_supported(head_dim), "attn_mfma_prefill: head_dim must be 64 or 128");
   YK_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_mfma_prefill: page_size must be a multiple of 16");
   YK_REQUIRE(q_stride % 8 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0,
@@ -823,32 +825,37 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
   const int chunks = (n_heads / n_kv + hpt - 1) / hpt;
   YK_REQUIRE(static_cast<long long>(n_tiles) * n_kv * chunks <= 0x7fffffffLL, "attn_mfma_prefill: too many tiles for one launch");
   YK_REQUIRE(n_splits >= 1 && n_splits <= 65535, "attn_mfma_prefill: bad split count");
-  static_assert(PF_CT == 1, "the merge of split long tiles takes one column tile per wave");
-  const size_t need = yk_attn_mfma_workspace(4 * n_tiles, n_heads, n_kv, head_dim, n_splits);
+  const size_t need = yk_attn_mfma_workspace(4 * col_tiles * n_tiles, n_heads, n_kv, head_dim, n_splits);
   YK_REQUIRE(workspace_floats >= need, "attn_mfma_prefill: workspace too small");
   float* ws_o = workspace;
   float* ws_ml = workspace ? workspace + (need / (head_dim + 2)) * head_dim : nullptr;
   const float scale_log2 = scale * 1.4426950408889634f;
   dim3 grid(n_tiles * n_kv * chunks, n_splits), block(256);
 #define YK_PF(DD, BIP)                                                                                       \
-  attn_mfma_prefill_kernel<DD, BIP><<<grid, block, 0, stream>>>(                                                 \
+  if (col_tiles == 1)                                                                                        \
+    attn_mfma_prefill_kernel<DD, BIP, 1><<<grid, block, 0, stream>>>(                                            \
+      static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),   \
+      static_cast<const bf16_t*>(v_cache), tiles, block_table, table_width, page_size, n_heads, n_kv, hpt, chunks, \
+      scale_log2, window, n_splits, ws_o, ws_ml);                                                                \
+  else                                                                                                       \
+    attn_mfma_prefill_kernel<DD, BIP, 2><<<grid, block, 0, stream>>>(                                            \
       static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),   \
       static_cast<const bf16_t*>(v_cache), tiles, block_table, table_width, page_size, n_heads, n_kv, hpt, chunks, \
       scale_log2, window, n_splits, ws_o, ws_ml)
   const bool bip = cache_is_tiled(YK_BF16, head_dim, page_size);
   if (head_dim == 64) {
-    if (bip) YK_PF(64, true); else YK_PF(64, false);
+    if (bip) { YK_PF(64, true); } else { YK_PF(64, false); }
   } else {
-    if (bip) YK_PF(128, true); else YK_PF(128, false);
+    if (bip) { YK_PF(128, true); } else { YK_PF(128, false); }
   }
 #undef YK_PF
   if (yk_check_launch("attn_mfma_prefill")) return -1;
   if (n_splits > 1) {
-    dim3 cgrid(4 * n_tiles, n_kv * chunks);
+    dim3 cgrid(4 * col_tiles * n_tiles, n_kv * chunks);
     if (head_dim == 64)
-      attn_combine_kernel<64><<<cgrid, 256, 0, stream>>>(static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 4);
+      attn_combine_kernel<64><<<cgrid, 256, 0, stream>>>(static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 4 * col_tiles);
     else
-      attn_combine_kernel<128><<<cgrid, 256, 0, stream>>>(static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 4);
+      attn_combine_kernel<128><<<cgrid, 256, 0, stream>>>(static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 4 * col_tiles);
     return yk_check_launch("attn_combine");
   }
   return 0;

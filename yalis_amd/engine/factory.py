@@ -33,6 +33,9 @@ class _ShapeOnlyOps:
     def attention_long_span_tile(self, *a):
         return 4
 
+    def attention_long_col_tiles(self, *a):
+        return 1
+
 
 def spec_from_config(config_dict: dict):
     arch = architecture_of(config_dict)

@@ -56,6 +56,7 @@ class StepContext:
         self.n_seqs = host.n_seqs
         self.max_qlen = host.max_qlen
         self.max_ctx = host.max_ctx
+        self.memo: Dict[str, object] = {}  # what a part worked out for this step, for the layers after it
 
     def site(self, entry: int) -> Site:
         return self._sites[entry]

@@ -69,11 +69,11 @@ _SIGNATURES = {
     ),
     "yk_attn_mfma_supported": ([_c_int], _c_int),
     "yk_attn_heads_per_tile": ([_c_int, _c_int], _c_int),
-    "yk_attn_long_tile_tokens": ([_c_int, _c_int], _c_int),
+    "yk_attn_long_tile_tokens": ([_c_int, _c_int, _c_int], _c_int),
     "yk_attn_tokens_per_tile": ([_c_int, _c_int], _c_int),
     "yk_attn_mfma_workspace": ([_c_int, _c_int, _c_int, _c_int, _c_int], _c_size_t),
     "yk_attn_mfma_prefill": (
-        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _vp, _c_size_t, _vp],
+        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _vp],
         _c_int,
     ),
     "yk_attn_mfma": (
@@ -212,9 +212,23 @@ class HipOps:
     def attention_tokens_per_tile(self, n_heads: int, n_kv: int) -> int:
         return self.lib.yk_attn_tokens_per_tile(n_heads, n_kv)
 
-    def attention_long_span_tile(self, n_heads: int, n_kv: int) -> int:
-        """Tokens per tile of the kernel for long spans (one workgroup a tile)."""
-        return self.lib.yk_attn_long_tile_tokens(n_heads, n_kv)
+    def attention_long_span_tile(self, n_heads: int, n_kv: int, col_tiles: int = 1) -> int:
+        """Tokens per tile of the kernel for long spans (one workgroup a tile) when a wave
+        has ``col_tiles`` (1 or 2) column tiles."""
+        return self.lib.yk_attn_long_tile_tokens(n_heads, n_kv, col_tiles)
+
+    @staticmethod
+    def attention_long_col_tiles(workgroups: int, fewest_keys: int) -> int:
+        """Column tiles per wave for a step's long spans.  ``workgroups``: how many the
+        larger tiles (two column tiles a wave) would make; ``fewest_keys``: the fewest keys
+        any of the spans has cached before it.  Two where those workgroups are enough to fill
+        the GPU twice over, or to fill it once when no span starts from nothing (a prompt from
+        nothing has tiles with a few keys and tiles with all of them: small tiles balance
+        that better); else one.  Measured on the 8B shape (us, one / two): a whole 2,048-token
+        prompt 81 / 99, a whole 4,096-token one 272 / 242, 2,048 tokens against 6,144 cached
+        461 / 341, four 512-token portions against 3,584 cached 247 / 189, one such portion
+        73 / 80."""
+        return 2 if workgroups >= 1024 or (workgroups >= 512 and fewest_keys >= 1024) else 1
 
     # ------------------------------------------------------------------ embedding
     def embed(self, token_ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
@@ -419,11 +433,14 @@ class HipOps:
         return max(1, min(-(-768 // workgroups), key_blocks // 8, 16))
 
     def attention(self, qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size,
-                  scale, window, ctx, group, tiles, long_tiles=None, plan=None, long_plan=None) -> torch.Tensor:
+                  scale, window, ctx, group, tiles, long_tiles=None, plan=None, long_plan=None,
+                  long_col_tiles: int = 1) -> torch.Tensor:
         """Queries are the first n_heads heads of each row of ``qkv`` (whatever follows
         them in the row is skipped); keys and values come from the cache through the
-        block table of ``group``.  ``plan`` overrides ``attention_plan`` and ``long_plan``
-        ``attention_long_splits`` (tests, measurements)."""
+        block table of ``group``.  ``long_tiles`` hold up to
+        ``attention_long_span_tile(n_heads, n_kv, long_col_tiles)`` tokens each.  ``plan``
+        overrides ``attention_plan`` and ``long_plan`` ``attention_long_splits`` (tests,
+        measurements)."""
         self._rows(qkv, "qkv")
         n = qkv.shape[0]
         bt = ctx.arrays[f"block_table_g{group}"]
@@ -443,13 +460,14 @@ class HipOps:
             hpt = self.lib.yk_attn_heads_per_tile(n_heads, n_kv)
             groups = n_long * n_kv * (-(-(n_heads // n_kv) // hpt))
             long_splits = long_plan if long_plan is not None else self.attention_long_splits(groups, max(1, -(-ctx.max_ctx // 64)))
-            ws_floats = self.lib.yk_attn_mfma_workspace(4 * n_long, n_heads, n_kv, head_dim, long_splits)
+            ws_floats = self.lib.yk_attn_mfma_workspace(4 * long_col_tiles * n_long, n_heads, n_kv, head_dim, long_splits)
             ws = self._ws(ws_floats) if ws_floats else None
             self._check(
                 self.lib.yk_attn_mfma_prefill(
                     qkv.data_ptr(), qkv.stride(0), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                     long_tiles.data_ptr(), n_long, bt.data_ptr(), bt.shape[1], page_size, head_dim,
-                    n_heads, n_kv, float(scale), int(window), long_splits, _ptr(ws), 0 if ws is None else ws.numel(),
+                    n_heads, n_kv, float(scale), int(window), long_splits, int(long_col_tiles), _ptr(ws),
+                    0 if ws is None else ws.numel(),
                     self._stream(),
                 )
             )

@@ -16,6 +16,7 @@ from __future__ import annotations
 
 from typing import Dict, Mapping
 
+import numpy as np
 import torch
 
 from ..config.specs import PartSpec
@@ -50,7 +51,10 @@ class Attention(Mixer):
             raise ValueError("rotary_dim exceeds head_dim")
         rt.ops.check_attention_sizes(self.n_heads, self.n_kv, self.head_dim, rt.page_size)
         self.tokens_per_tile = rt.ops.attention_tokens_per_tile(self.n_heads, self.n_kv)
+        # spans longer than `long_tile` go to the kernel for long spans, in tiles of that many
+        # tokens or twice as many (`long_tiles_of`: the step's choice)
         self.long_tile = rt.ops.attention_long_span_tile(self.n_heads, self.n_kv)
+        self.long_tile_2 = rt.ops.attention_long_span_tile(self.n_heads, self.n_kv, 2)
         self.group = None
         self.w_qkv = self.w_q = self.w_o = None
 
@@ -79,14 +83,32 @@ class Attention(Mixer):
     def kv_need(self) -> KVNeed:
         return KVNeed(self.n_kv, self.head_dim, self.window)
 
+    def long_col_tiles(self, hb) -> int:
+        """Column tiles per wave for this step's long spans (1 or 2), from what the host
+        knows of the batch: how many workgroups the larger tiles would make, and the fewest
+        keys any long span has cached before it."""
+        long_spans = hb.seq_qlen > self.long_tile
+        if not long_spans.any():
+            return 1
+        qlen = hb.seq_qlen[long_spans].astype(np.int64)
+        tiles = int((-(-qlen // self.long_tile_2)).sum())
+        heads_per_tile = min(self.n_heads // self.n_kv, 16)
+        chunks = -(-(self.n_heads // self.n_kv) // heads_per_tile)
+        fewest = int((hb.seq_ctx[long_spans] - hb.seq_qlen[long_spans]).min())
+        return self.rt.ops.attention_long_col_tiles(tiles * self.n_kv * chunks, fewest)
+
     def step_inputs(self):
         # spans of more than one large tile go to the kernel for long spans, the rest
         # (single decoded tokens, short portions) to the one that splits the keys
         tpt = self.tokens_per_tile
-        big = self.rt.ops.attention_long_span_tile(self.n_heads, self.n_kv)
+        big, big2 = self.long_tile, self.long_tile_2
+        none = np.zeros((0, 4), dtype=np.int32)
         return {
             f"attention_tiles_{tpt}_upto{big}": lambda hb: attention_tiles(hb, tpt, 1, big),
-            f"attention_long_tiles_{big}": lambda hb: attention_tiles(hb, big, big + 1, longest_first=True),
+            f"attention_long_tiles_{big}": lambda hb: attention_tiles(hb, big, big + 1, longest_first=True)
+            if self.long_col_tiles(hb) == 1 else none,
+            f"attention_long_tiles_{big2}": lambda hb: attention_tiles(hb, big2, big + 1, longest_first=True)
+            if self.long_col_tiles(hb) == 2 else none,
         }
 
     # ---- what it computes
@@ -101,6 +123,9 @@ class Attention(Mixer):
             qkv = ops.linear(h, self.w_q, self.rt.act_dtype, partial_ok=True)
             n_kv_rows = 0
         k_cache, v_cache = site.kv()
+        col_tiles = ctx.memo.get("attention_long_col_tiles")
+        if col_tiles is None:
+            col_tiles = ctx.memo["attention_long_col_tiles"] = self.long_col_tiles(ctx.host)
         pos = self.position
         q = ops.rope_append(
             qkv,
@@ -130,6 +155,7 @@ class Attention(Mixer):
             ctx,
             site.group,
             ctx.arrays[f"attention_tiles_{self.tokens_per_tile}_upto{self.long_tile}"],
-            ctx.arrays[f"attention_long_tiles_{self.long_tile}"],
+            ctx.arrays[f"attention_long_tiles_{self.long_tile_2 if col_tiles == 2 else self.long_tile}"],
+            long_col_tiles=col_tiles,
         )
         return ops.linear(out, self.w_o, self.rt.act_dtype, partial_ok=True)
