@@ -118,6 +118,24 @@ def test_full_width_replay(dtype):
         assert runner.pages.live_requests() == 0
 
 
+@pytest.mark.gpu
+def test_full_width_replay_with_large_long_tiles(monkeypatch):
+    """The attention part picks the size of its long tiles per step; at these sizes it never
+    picks the larger ones by itself, so the choice is forced: every long span then runs with
+    two column tiles a wave, and the logits are the same."""
+    from yalis_amd.ops.hip import HipOps
+
+    monkeypatch.setattr(HipOps, "attention_long_col_tiles", staticmethod(lambda workgroups, fewest_keys: 2))
+    weights, reqs, want = full_width_setup(True)
+    for mode, make in (("whole", C.trace_whole), ("portions", C.trace_portions), ("mixed", C.trace_mixed)):
+        steps = make(reqs)
+        runner = C.make_runner(FULL_WIDTH, weights, "bfloat16", "cuda:0", ops_for("cuda:0"), 64, C.pages_needed(steps, reqs, 64))
+        got, _ = C.run_trace(runner, steps)
+        C.assert_matches(got, want, True, f"full width, large long tiles/{mode}")
+        runner.pages.audit()
+        del runner
+
+
 @pytest.mark.parametrize("backend", BACKENDS)
 def test_readmission_reproduces(backend):
     """Release a request half way (as a preemption does) and replay it from the start:
