@@ -144,6 +144,7 @@ class HipOps:
         self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
         self._workspace: Optional[torch.Tensor] = None  # attention splits, argmax parts
         self._gemm_workspace: Optional[torch.Tensor] = None  # K slices of products
+        self._mm_f32: Optional[bool] = None  # see _library_f32_out
 
     # ------------------------------------------------------------------ helpers
     @staticmethod
@@ -289,10 +290,24 @@ class HipOps:
         bf = torch.bfloat16
         aligned = k % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
         if x.dtype == bf and w.dtype == bf and aligned:
-            if m <= SKINNY_MAX_ROWS or out_dtype != bf:
-                return self.gemm_mfma_skinny(x, w, out_dtype, partial_ok)
-            return torch.matmul(x, w.t())  # vendor library, bfloat16 in and out
+            if m > SKINNY_MAX_ROWS and out_dtype == bf:
+                return torch.matmul(x, w.t())  # vendor library, bfloat16 in and out
+            if m > SKINNY_MAX_ROWS and out_dtype == torch.float32 and self._library_f32_out():
+                # vendor library, float32 accumulators stored as they are (the output head for
+                # more than 64 wanted rows: the few-row kernel would stream the table once per 64)
+                return torch.mm(x, w.t(), out_dtype=torch.float32)
+            return self.gemm_mfma_skinny(x, w, out_dtype, partial_ok)
         return self.gemm_fma(x, w, out_dtype)
+
+    def _library_f32_out(self) -> bool:
+        """Whether this torch's matrix product takes bfloat16 operands and gives float32."""
+        if self._mm_f32 is None:
+            try:
+                a = torch.zeros((16, 16), dtype=torch.bfloat16, device=self.device)
+                self._mm_f32 = torch.mm(a, a, out_dtype=torch.float32).dtype == torch.float32
+            except (TypeError, RuntimeError):
+                self._mm_f32 = False
+        return self._mm_f32
 
     def gemm_fma(self, x, w, out_dtype):
         m, k = x.shape
