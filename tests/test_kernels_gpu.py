@@ -572,6 +572,35 @@ def test_sample_large_vocabulary_matches_plain(ops, vocab, kind):
             assert got == want and slow == want, (kind, temperature, top_k, top_p, draw, got, slow, want)
 
 
+@pytest.mark.parametrize("kind", ["peaked", "flat"])
+def test_sample_divided_rows(ops, kind):
+    """Rows of a large vocabulary are divided among workgroups: rows with different settings in
+    one launch give the plain implementation's tokens, and each goes the way its settings
+    say: greedy, a race over the row (plain temperature; top_p once its threshold is known),
+    settled among the candidates (top_k), or left to one workgroup (more candidates than fit)."""
+    import plain_llama as P
+
+    vocab = 128256
+    settings = [(0.0, 0, 1.0, 0), (1.0, 0, 1.0, 1), (1.0, 0, 0.8, 1), (1.0, 50, 1.0, 3), (0.7, 50, 0.8, 3),
+                (2.0, 0, 0.9, 1), (1.0, 6000, 1.0, 4), (0.5, 1, 1.0, 3), (1.3, 0, 0.0, 1), (0.9, 3000, 0.95, 3)]
+    gen = torch.Generator().manual_seed(77)
+    logits = torch.randn((len(settings), vocab), generator=gen) * (3.0 if kind == "peaked" else 0.3)
+    if kind == "peaked":
+        logits[:, 1000:1040] += 9.0
+    logits[1, 5] = float("-inf")  # a masked token: never drawn, and no part of the bins' extent
+    dev = logits.to(DEV)
+    col = lambda j, dt: torch.tensor([st[j] for st in settings], dtype=dt, device=DEV)
+    seeds = torch.arange(len(settings), dtype=torch.int32, device=DEV) + 11
+    for draw in range(3):
+        draws = torch.full((len(settings),), draw, dtype=torch.int32, device=DEV)
+        paths = torch.full((len(settings),), -1, dtype=torch.int32, device=DEV)
+        got = ops.sample(dev, col(0, torch.float32), col(1, torch.int32), col(2, torch.float32), seeds, draws, paths=paths).cpu()
+        assert paths.cpu().tolist() == [st[3] for st in settings]
+        for i, (temperature, top_k, top_p, _) in enumerate(settings):
+            want = P.sample_token(logits[i], temperature, top_k or None, top_p, 11 + i, draw)
+            assert got[i].item() == want, (kind, i, settings[i], draw, got[i].item(), want)
+
+
 def test_sample_rows_are_independent(ops):
     """Many rows with different settings in one launch give what each gives alone."""
     vocab = 50000

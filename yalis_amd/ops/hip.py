@@ -86,7 +86,8 @@ _LATER_SIGNATURES = {
     "sampling": {
         "yk_abi_version": ([], _c_int),
         "yk_argmax": ([_vp, _vp, _c_int, _c_int, _vp, _c_size_t, _vp], _c_int),
-        "yk_sample": ([_vp, _vp, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _vp], _c_int),
+        "yk_sample": ([_vp, _vp, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _vp, _c_size_t, _vp, _vp], _c_int),
+        "yk_sample_workspace_bytes": ([_c_int, _c_int], _c_size_t),
     },
     "probe": {
         "yk_abi_version": ([], _c_int),
@@ -94,7 +95,7 @@ _LATER_SIGNATURES = {
         "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
     },
 }
-_ABI = 6
+_ABI = 7
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
 # above it the vendor library does.
@@ -554,10 +555,13 @@ class HipOps:
                                   ws.data_ptr(), ws.numel(), self._stream()), lib)
         return out
 
-    def sample(self, logits, temperature, top_k, top_p, seeds, draws, whole_row: bool = False) -> torch.Tensor:
+    def sample(self, logits, temperature, top_k, top_p, seeds, draws, whole_row: bool = False, paths=None) -> torch.Tensor:
         """Per row: temperature (float32; 0 = greedy), top_k (int32; 0 = off), top_p
-        (float32), seed and draw number (int32).  Returns int32 token ids.  ``whole_row``
-        forces the path that never narrows the row down to candidates (for tests)."""
+        (float32), seed and draw number (int32).  Returns int32 token ids.  Rows of a large
+        vocabulary are divided among workgroups; ``whole_row`` forces one workgroup a row on
+        the path that never narrows the row down to candidates (for tests), and ``paths``
+        (int32, one per row) receives which way each divided row went: 0 greedy, 1 a race
+        over the row, 3 settled among candidates, 4 left to one workgroup after all."""
         if logits.dtype != torch.float32 or not logits.is_contiguous() or logits.dim() != 2:
             raise KernelError("sample takes contiguous float32 logits [rows, vocab]")
         rows = logits.shape[0]
@@ -565,12 +569,17 @@ class HipOps:
                             ("top_p", top_p, torch.float32), ("seeds", seeds, torch.int32), ("draws", draws, torch.int32)):
             if t.dtype != dt or t.numel() != rows or not t.is_contiguous():
                 raise KernelError(f"sample: {name} must be {dt} with one entry per row")
+        if paths is not None and (paths.dtype != torch.int32 or paths.numel() != rows or not paths.is_contiguous()):
+            raise KernelError("sample: paths must be int32 with one entry per row")
         out = torch.empty(rows, dtype=torch.int32, device=logits.device)
         lib = self._library("sampling")
+        need = 0 if whole_row else int(lib.yk_sample_workspace_bytes(rows, logits.shape[1]))
+        ws = self._ws((need + 3) // 4) if need else None
         self._check(
             lib.yk_sample(
                 logits.data_ptr(), out.data_ptr(), rows, logits.shape[1], temperature.data_ptr(), top_k.data_ptr(),
-                top_p.data_ptr(), seeds.data_ptr(), draws.data_ptr(), int(bool(whole_row)), self._stream(),
+                top_p.data_ptr(), seeds.data_ptr(), draws.data_ptr(), int(bool(whole_row)),
+                _ptr(ws), 0 if ws is None else ws.numel() * 4, _ptr(paths), self._stream(),
             ),
             lib,
         )
