@@ -103,6 +103,42 @@ def machine_probe(cfg: dict) -> int:
     return 0
 
 
+def sampling_times(vocab: int, batch: int) -> int:
+    """Times the choice of a token alone (no model) at this vocabulary for ``batch`` rows:
+    greedy and each sampling rule, on a nearly flat row (what random weights give) and on a
+    peaked one (a few dozen likely tokens, as a trained model gives)."""
+    import torch
+
+    from yalis_amd.ops.hip import HipOps
+
+    ops = HipOps("cuda:0")
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    flat = torch.randn(batch, vocab, device="cuda", generator=gen) * 0.3
+    peaked = torch.randn(batch, vocab, device="cuda", generator=gen) * 2.5
+    peaked[:, :50] += 12.0
+    full = lambda v, dt: torch.full((batch,), v, dtype=dt, device="cuda")
+    seeds, draws = torch.arange(batch, dtype=torch.int32, device="cuda"), full(0, torch.int32)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    out = {}
+    for rows_name, logits in (("flat", flat), ("peaked", peaked)):
+        for name, (t, k, p) in (("greedy", (0.0, 0, 1.0)), ("temperature", (1.0, 0, 1.0)), ("top_p 0.8", (1.0, 0, 0.8)),
+                                ("top_k 50", (1.0, 50, 1.0)), ("top_k 50, top_p 0.8, T 0.7", (0.7, 50, 0.8))):
+            temperature, top_k, top_p = full(t, torch.float32), full(k, torch.int32), full(p, torch.float32)
+            run = (lambda: ops.argmax(logits)) if t == 0.0 else (lambda: ops.sample(logits, temperature, top_k, top_p, seeds, draws))
+            for _ in range(3):
+                run()
+            start.record()
+            for _ in range(20):
+                run()
+            stop.record()
+            stop.synchronize()
+            us = start.elapsed_time(stop) / 20 * 1e3
+            out[f"{rows_name}: {name}"] = round(us, 1)
+            print(f"  {rows_name:7s} {name:28s} {us:7.1f} us")
+    print(json.dumps({"probe": "sampling", "vocab": vocab, "rows": batch, "us": out}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -118,6 +154,7 @@ def main() -> int:
     ap.add_argument("--portion", type=int, default=480, help="tokens of a prompt portion in --mixed steps (with the 32 decoded tokens: 512 rows, as the scheduler cuts under a budget of 512)")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel (for hardware counters)")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="8b", help="layer sizes (default: the 8B shape of the headline)")
+    ap.add_argument("--sample", action="store_true", help="time instead the choice of a token alone (greedy and each sampling rule) at the shape's vocabulary for --batch rows")
     ap.add_argument("--probe", action="store_true", help="measure instead what a plain streaming read and a plain matrix-core loop reach on this card")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -128,6 +165,8 @@ def main() -> int:
 
     if args.probe:
         return machine_probe(SHAPES[args.shape][1])
+    if args.sample:
+        return sampling_times(SHAPES[args.shape][1]["vocab_size"], args.batch)
 
     from yalis_amd.config.runtime import EngineConfig
     from yalis_amd.engine.factory import random_runner
