@@ -140,6 +140,7 @@ class HipOps:
         self.device = torch.device(device)
         self.lib = self._bind(load_kernels(), _SIGNATURES)
         self._later: dict = {}
+        self._answers: dict = {}
         self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
         # the quick way to the current stream's handle, where this torch has it
         self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -197,6 +198,15 @@ class HipOps:
         """The scratch buffers in use, for whoever must keep them alive (a captured graph)."""
         return (self._workspace, self._gemm_workspace)
 
+    def _ask(self, name: str, *args: int) -> int:
+        """A size question to the library (tile sizes, slices, workspace needs): the answers
+        depend on the arguments alone, so each is asked once."""
+        key = (name, args)
+        got = self._answers.get(key)
+        if got is None:
+            got = self._answers[key] = getattr(self.lib, name)(*args)
+        return got
+
     @staticmethod
     def _rows(t: torch.Tensor, what: str) -> None:
         if t.dim() != 2 or t.stride(1) != 1:
@@ -212,12 +222,12 @@ class HipOps:
             raise KernelError(f"attention: page_size must be a multiple of 16, got {page_size}")
 
     def attention_tokens_per_tile(self, n_heads: int, n_kv: int) -> int:
-        return self.lib.yk_attn_tokens_per_tile(n_heads, n_kv)
+        return self._ask("yk_attn_tokens_per_tile", n_heads, n_kv)
 
     def attention_long_span_tile(self, n_heads: int, n_kv: int, col_tiles: int = 1) -> int:
         """Tokens per tile of the kernel for long spans (one workgroup a tile) when a wave
         has ``col_tiles`` (1 or 2) column tiles."""
-        return self.lib.yk_attn_long_tile_tokens(n_heads, n_kv, col_tiles)
+        return self._ask("yk_attn_long_tile_tokens", n_heads, n_kv, col_tiles)
 
     @staticmethod
     def attention_long_col_tiles(workgroups: int, fewest_keys: int) -> int:
@@ -352,7 +362,7 @@ class HipOps:
             group == self.GATE_UP_GROUP and 0 < m <= SKINNY_MAX_ROWS and x.dtype == bf and w_gate_up.dtype == bf and out_dtype == bf
             and w_gate_up.shape[1] == k and k % 8 == 0 and x.stride(0) % 8 == 0 and w_gate_up.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0 and n % 16 == 0
-            and self.lib.yk_gemm_skinny_splits(m, n, k) == 1
+            and self._ask("yk_gemm_skinny_splits", m, n, k) == 1
         )
         if not fused:
             return self.gated_act(self.linear(x, w_gate_up, out_dtype, partial_ok=True), activation, out_dtype, group=group)
@@ -368,7 +378,7 @@ class HipOps:
     def gemm_mfma_skinny(self, x, w, out_dtype, partial_ok: bool = False):
         m, k = x.shape
         n = w.shape[0]
-        splits = self.lib.yk_gemm_skinny_splits(m, n, k)
+        splits = self._ask("yk_gemm_skinny_splits", m, n, k)
         keep = bool(partial_ok and splits > 1)
         ws = self._gemm_ws(splits * m * n) if splits > 1 else None
         y = None if keep else torch.empty((m, n), dtype=out_dtype, device=x.device)
@@ -467,16 +477,16 @@ class HipOps:
         out = torch.empty((n, n_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
         use_mfma = (
             qkv.dtype == torch.bfloat16
-            and self.lib.yk_attn_mfma_supported(head_dim)
+            and self._ask("yk_attn_mfma_supported", head_dim)
             and qkv.stride(0) % 8 == 0
             and qkv.data_ptr() % 16 == 0
         )
         if use_mfma and long_tiles is not None and long_tiles.shape[0] > 0:
             n_long = long_tiles.shape[0]
-            hpt = self.lib.yk_attn_heads_per_tile(n_heads, n_kv)
+            hpt = self._ask("yk_attn_heads_per_tile", n_heads, n_kv)
             groups = n_long * n_kv * (-(-(n_heads // n_kv) // hpt))
             long_splits = long_plan if long_plan is not None else self.attention_long_splits(groups, max(1, -(-ctx.max_ctx // 64)))
-            ws_floats = self.lib.yk_attn_mfma_workspace(4 * long_col_tiles * n_long, n_heads, n_kv, head_dim, long_splits)
+            ws_floats = self._ask("yk_attn_mfma_workspace", 4 * long_col_tiles * n_long, n_heads, n_kv, head_dim, long_splits)
             ws = self._ws(ws_floats) if ws_floats else None
             self._check(
                 self.lib.yk_attn_mfma_prefill(
@@ -491,11 +501,11 @@ class HipOps:
             return out
         if use_mfma:
             n_tiles = tiles.shape[0]
-            hpt = self.lib.yk_attn_heads_per_tile(n_heads, n_kv)
+            hpt = self._ask("yk_attn_heads_per_tile", n_heads, n_kv)
             chunks = -(-(n_heads // n_kv) // hpt)
             key_blocks = max(1, -(-ctx.max_ctx // 64))
             waves, splits = plan or self.attention_plan(n_tiles * n_kv * chunks, key_blocks)
-            ws_floats = self.lib.yk_attn_mfma_workspace(n_tiles, n_heads, n_kv, head_dim, splits)
+            ws_floats = self._ask("yk_attn_mfma_workspace", n_tiles, n_heads, n_kv, head_dim, splits)
             ws = self._ws(ws_floats) if ws_floats else None
             self._check(
                 self.lib.yk_attn_mfma(
