@@ -254,6 +254,12 @@ def test_linear_dispatch(ops):
     close(ops.linear(x, w, torch.bfloat16), want, 1e-2, 2**-7)
     close(ops.linear(x, w, torch.float32), want, 1e-4, 1e-5)
     close(ops.linear(x[:5], w, torch.bfloat16), want[:5], 1e-2, 2**-7)
+    # 65 to 192 rows where the vendor library would have few tiles: the few-row kernel, in row tiles of 64
+    assert ops.few_library_tiles(100, 515) and not ops.few_library_tiles(200, 515) and not ops.few_library_tiles(128, 28672)
+    for rows in (65, 100, 192):
+        close(ops.linear(x[:rows], w, torch.bfloat16), want[:rows], 1e-2, 2**-7)
+        part = ops.linear(x[:rows], w, torch.bfloat16, partial_ok=True)
+        close(part.reduce() if hasattr(part, "reduce") else part, want[:rows], 1e-2, 2**-7)
     wf = w.float()
     close(ops.linear(x, wf, torch.bfloat16), want, 1e-2, 2**-7)
 

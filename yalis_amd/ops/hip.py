@@ -301,7 +301,7 @@ class HipOps:
         bf = torch.bfloat16
         aligned = k % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
         if x.dtype == bf and w.dtype == bf and aligned:
-            if m > SKINNY_MAX_ROWS and out_dtype == bf:
+            if m > SKINNY_MAX_ROWS and out_dtype == bf and not self.few_library_tiles(m, n):
                 return torch.matmul(x, w.t())  # vendor library, bfloat16 in and out
             if m > SKINNY_MAX_ROWS and out_dtype == torch.float32 and self._library_f32_out():
                 # vendor library, float32 accumulators stored as they are (the output head for
@@ -309,6 +309,15 @@ class HipOps:
                 return torch.mm(x, w.t(), out_dtype=torch.float32)
             return self.gemm_mfma_skinny(x, w, out_dtype, partial_ok)
         return self.gemm_fma(x, w, out_dtype)
+
+    @staticmethod
+    def few_library_tiles(m: int, n: int) -> bool:
+        """Whether a product of 65 to 192 rows is still the few-row kernel's: where the vendor
+        library's tiles (about 128 x 256 of the output) would be too few to occupy the GPU's
+        256 compute units, while the few-row kernel divides K among workgroups.  Measured on
+        the 8B shapes at 128 rows (us, few-row kernel / library): o-proj 16 / 25, down-proj
+        48 / 76, qkv 24 / 26, but gate/up 102 / 57 (112 tiles of 256 columns: the library's)."""
+        return m <= 192 and -(-m // 128) * -(-n // 256) < 64
 
     def _library_f32_out(self) -> bool:
         """Whether this torch's matrix product takes bfloat16 operands and gives float32."""
