@@ -313,11 +313,12 @@ class HipOps:
     @staticmethod
     def few_library_tiles(m: int, n: int) -> bool:
         """Whether a product of 65 to 192 rows is still the few-row kernel's: where the vendor
-        library's tiles (about 128 x 256 of the output) would be too few to occupy the GPU's
-        256 compute units, while the few-row kernel divides K among workgroups.  Measured on
-        the 8B shapes at 128 rows (us, few-row kernel / library): o-proj 16 / 25, down-proj
-        48 / 76, qkv 24 / 26, but gate/up 102 / 57 (112 tiles of 256 columns: the library's)."""
-        return m <= 192 and -(-m // 128) * -(-n // 256) < 64
+        library's output tiles (256 columns wide, one or two tiles of rows) would be too few
+        to occupy the GPU's 256 compute units, while the few-row kernel divides K among
+        workgroups.  Measured at 128 rows (us, few-row kernel / library), 8B shapes: o-proj
+        16 / 25, down-proj 48 / 76, qkv 24 / 26, gate/up 102 / 57; 3B shapes: 13 / 21, 24 / 43,
+        17 / 21, 46 / 31; 70B shapes (8,192 columns and more): the library's everywhere."""
+        return m <= 192 and -(-n // 256) < 32
 
     def _library_f32_out(self) -> bool:
         """Whether this torch's matrix product takes bfloat16 operands and gives float32."""
