@@ -177,20 +177,23 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(
     }
   }
   if (del) {
-    // four slices at a time, all loads issued before the first sum; a slice index beyond
-    // the last is clamped and its value dropped, so that the loads carry no condition
+    // SL slices at a time (eight where a thread has one piece of the row: a product's eight
+    // slices then cost one wait for memory, not two), all loads issued before the first
+    // sum; a slice index beyond the last is clamped and its value dropped, so that the
+    // loads carry no condition
+    constexpr int SL = NORM_IT == 1 ? 8 : 4;
 #pragma unroll
     for (int it = 0; it < NORM_IT; ++it) ds[it] = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int s0 = 0; s0 < n_splits; s0 += 4) {
+    for (int s0 = 0; s0 < n_splits; s0 += SL) {
 #pragma unroll
       for (int it = 0; it < NORM_IT; ++it) {
         const int c = (threadIdx.x + it * blockDim.x) * 4;
         if (c < width) {
-          float4 d[4];
+          float4 d[SL];
 #pragma unroll
-          for (int j = 0; j < 4; ++j) d[j] = load4<TD>(del + static_cast<size_t>(min(s0 + j, n_splits - 1)) * split_stride + c);
+          for (int j = 0; j < SL; ++j) d[j] = load4<TD>(del + static_cast<size_t>(min(s0 + j, n_splits - 1)) * split_stride + c);
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
+          for (int j = 0; j < SL; ++j) {
             if (s0 + j < n_splits) {
               ds[it].x += d[j].x;
               ds[it].y += d[j].y;
