@@ -104,7 +104,7 @@ def attention_paged(q, k_cache, v_cache, positions, token_seq, block_table, page
 
 
 def attention(qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size, scale,
-              window, ctx, group, tiles, long_tiles=None, plan=None, long_plan=None, long_col_tiles=1):
+              window, ctx, group, tiles, long_tiles=None, plan=None, long_plan=None, long_col_tiles=1, token_cols=None):
     n = qkv.shape[0]
     q = qkv.view(n, -1, head_dim)[:, :n_heads]
     out = attention_paged(

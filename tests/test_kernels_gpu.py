@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import kernel_refs as R
-from yalis_amd.engine.batch import SeqSpan, attention_tiles, build_host_batch, named_arrays
+from yalis_amd.engine.batch import SeqSpan, attention_tiles, attention_token_columns, build_host_batch, named_arrays
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -334,7 +334,7 @@ def test_rope_append_prompt_portions(ops, h, g, d, rd, page):
 
 
 # ------------------------------------------------------------------------- attention
-def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True, n_pages=64, plan=None, long_plan=None, col_tiles=1):
+def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True, n_pages=64, plan=None, long_plan=None, col_tiles=1, with_cols=False):
     """spans: list of (cached tokens before the step, new tokens).  Builds pages in a
     shuffled order, fills cache for the earlier tokens, runs rope-free attention."""
     gen = torch.Generator().manual_seed(seed)
@@ -362,7 +362,8 @@ def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True,
     tpt = ops.attention_tokens_per_tile(h, g)
     big = ops.attention_long_span_tile(h, g)
     big_c = ops.attention_long_span_tile(h, g, col_tiles)  # tokens of a long tile with col_tiles column tiles a wave
-    arrays = named_arrays(hb, {"tiles": lambda b: attention_tiles(b, tpt, 1, big), "long_tiles": lambda b: attention_tiles(b, big_c, big + 1, longest_first=(seed % 2 == 0))})
+    arrays = named_arrays(hb, {"tiles": lambda b: attention_tiles(b, tpt, 1, big), "long_tiles": lambda b: attention_tiles(b, big_c, big + 1, longest_first=(seed % 2 == 0)),
+                               "cols": lambda b: attention_token_columns(b, tpt, 1, big)})
     ctx = types.SimpleNamespace(
         arrays={k: torch.from_numpy(np.ascontiguousarray(v)).to(DEV) for k, v in arrays.items()},
         max_ctx=hb.max_ctx,
@@ -372,7 +373,8 @@ def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True,
     q = (torch.randn((n, h * d), generator=gen) * 1.5).to(dtype)
     scale = 1.0 / math.sqrt(d)
     kc_d, vc_d = device_cache(ops, kc, vc)
-    got = ops.attention(q.to(DEV), h, g, d, kc_d, vc_d, page, scale, window, ctx, 0, ctx.arrays["tiles"], ctx.arrays["long_tiles"], plan=plan, long_plan=long_plan, long_col_tiles=col_tiles)
+    got = ops.attention(q.to(DEV), h, g, d, kc_d, vc_d, page, scale, window, ctx, 0, ctx.arrays["tiles"], ctx.arrays["long_tiles"], plan=plan, long_plan=long_plan, long_col_tiles=col_tiles,
+                        token_cols=ctx.arrays["cols"] if with_cols else None)
     want = R.attention(q.float(), h, g, d, kc.float(), vc.float(), page, scale, window, ctx_cpu, 0, None)
     return got, want
 
@@ -423,6 +425,42 @@ def test_attention_mfma_every_way_of_dividing_keys(ops, plan, d, page):
     for window in (0, 700, 33):
         got, want = _attention_case(ops, torch.bfloat16, 8, 2, d, page, spans, window, seed=16, n_pages=3072 // page + 6, plan=plan)
         close(got, want, 2e-2, 2**-6)
+
+
+@pytest.mark.parametrize("plan", [(4, 2), (4, 5), (1, 3)])
+@pytest.mark.parametrize("h,g,d,page", [(8, 2, 128, 64), (6, 3, 64, 32), (32, 8, 128, 64), (24, 8, 128, 64), (32, 1, 128, 32)])
+def test_attention_splits_merged_by_the_product(ops, plan, h, g, d, page, monkeypatch):
+    """A step of up to 16 tokens leaves its splits unmerged for the product that follows:
+    merged on their own they are the attention's output, and the product fed by the splits
+    gives the bits of the product fed by the merged tensor (tiles of 8, 4, 5 and 1 tokens;
+    heads that need two chunks; a product that keeps its K slices, one that does not, and
+    one whose K slices are too long, which merges first)."""
+    import yalis_amd.ops.hip as hip_ops
+    from yalis_amd.ops.hip import SplitAttention, SplitSum
+
+    monkeypatch.setattr(hip_ops, "MERGE_IN_PRODUCT_MAX_TOKENS", 16)  # as far as the kernel goes, not as far as it pays
+    spans = [(700, 1), (64, 2), (300, 1), (0, 3), (1500, 1), (63, 2)]
+    got, want = _attention_case(ops, torch.bfloat16, h, g, d, page, spans, 0, seed=21, n_pages=2700 // page + 8, plan=plan, with_cols=True)
+    assert isinstance(got, SplitAttention) and got.n_splits == plan[1] and got.shape == (10, h * d)
+    merged = got.merge()
+    close(merged, want, 2e-2, 2**-6)
+    plain, _ = _attention_case(ops, torch.bfloat16, h, g, d, page, spans, 0, seed=21, n_pages=2700 // page + 8, plan=plan)
+    assert torch.equal(plain, merged)
+    fed = 0
+    for n_out, out_dtype, partial_ok in ((h * d, torch.bfloat16, True), (515, torch.float32, False), (48, torch.bfloat16, True)):
+        w = rnd((n_out, h * d), torch.bfloat16, 22)
+        fed += bool(ops._ask("yk_gemm_skinny_from_attention_ok", 10, n_out, h * d))
+        y = ops.linear(got, w, out_dtype, partial_ok=partial_ok)
+        a = y.tensor.clone() if isinstance(y, SplitSum) else y.clone()
+        y = ops.linear(merged, w, out_dtype, partial_ok=partial_ok)
+        b = y.tensor if isinstance(y, SplitSum) else y
+        assert a.shape == b.shape and torch.equal(a, b), (n_out, out_dtype)
+        close(a.sum(0) if partial_ok and a.dim() == 3 else a, merged.double().cpu() @ w.double().cpu().T, 3e-2, 2**-6)
+    assert fed >= 1, "no product here took the splits itself"
+    # more than 16 tokens: merged by the attention itself
+    got, want = _attention_case(ops, torch.bfloat16, h, g, d, page, spans + [(5, 9)], 0, seed=21, n_pages=2700 // page + 8, plan=plan, with_cols=True)
+    assert isinstance(got, torch.Tensor)
+    close(got, want, 2e-2, 2**-6)
 
 
 @pytest.mark.parametrize("col_tiles", [1, 2])

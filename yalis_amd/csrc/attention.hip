@@ -139,18 +139,6 @@ union AFrag8 {
   bf16_t h[8];
 };
 
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef float f32x2_t __attribute__((ext_vector_type(2)));
-
-// two floats to two bfloat16 (round to nearest even) in one word: gfx950 converts in hardware
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  union {
-    bf16x2_t v;
-    uint32_t u;
-  } c;
-  c.v = __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t);
-  return c.u;
-}
 
 // 2^x for scores: -inf gives 0, no denormal handling needed
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -757,22 +745,11 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(
     // (a group of 16 columns holds tpt_ tokens; with a head count that does not divide 16 the
     // columns left over stand for nothing, not for the next part's first token)
     if (tt >= min(ntok, tpt_) || hh >= heads_here) continue;
-    const float* ml = ws_ml + (w0 * 16 + c) * 2;
-    float m_max = -INFINITY;
-#pragma unroll 4
-    for (int s = 0; s < n_splits; ++s) m_max = fmaxf(m_max, ml[static_cast<size_t>(s) * 32]);
-    f32x4_t num = {0.f, 0.f, 0.f, 0.f};
-    float den = 0.f;
-#pragma unroll 4
-    for (int s = 0; s < n_splits; ++s) {
-      const float w = exp2f(ml[static_cast<size_t>(s) * 32] - m_max);
-      num += w * *reinterpret_cast<const f32x4_t*>(ws_o + ((w0 + s) * 16 + c) * D + d);
-      den += w * ml[static_cast<size_t>(s) * 32 + 1];
-    }
-    const float inv = 1.f / den;
+    float merged[4];
+    attn_merge_splits(ws_o, ws_ml, w0 * 16 + c, n_splits, D, d, merged);
     u32x2_t o;
-    o[0] = pack_bf16x2(num[0] * inv, num[1] * inv);
-    o[1] = pack_bf16x2(num[2] * inv, num[3] * inv);
+    o[0] = pack_bf16x2(merged[0], merged[1]);
+    o[1] = pack_bf16x2(merged[2], merged[3]);
     *reinterpret_cast<u32x2_t*>(out + (static_cast<size_t>(tok0 + tt) * n_heads + h_base + hh) * D + d) = o;
   }
 }
@@ -780,10 +757,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(
 extern "C" int yk_attn_mfma_supported(int head_dim) { return head_dim == 64 || head_dim == 128; }
 
 // Heads of one kv head that share a wave, and tokens per tile, for a head layout.
-extern "C" int yk_attn_heads_per_tile(int n_heads, int n_kv) {
-  const int qpk = n_heads / n_kv;
-  return qpk < 16 ? qpk : 16;
-}
+extern "C" int yk_attn_heads_per_tile(int n_heads, int n_kv) { return attn_heads_per_tile(n_heads, n_kv); }
 extern "C" int yk_attn_tokens_per_tile(int n_heads, int n_kv) {
   return 16 / yk_attn_heads_per_tile(n_heads, n_kv);
 }
@@ -861,12 +835,15 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
   return 0;
 }
 
+// Short spans (single tokens, short portions): tiles of up to yk_attn_tokens_per_tile tokens.
+// leave_splits != 0 with n_splits > 1: the splits stay unmerged in the workspace (`out` is not
+// written) for a consumer that merges them itself or for yk_attn_combine.
 extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* k_cache,
                             const void* v_cache, const int32_t* tiles, int n_tiles,
                             const int32_t* block_table, int table_width, int page_size,
                             int head_dim, int n_heads, int n_kv, float scale, int window,
                             int n_waves, int n_splits, float* workspace, size_t workspace_floats,
-                            hipStream_t stream) {
+                            int leave_splits, hipStream_t stream) {
   YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_mfma: bad head counts");
   YK_REQUIRE(n_waves == 1 || n_waves == 4, "attn_mfma: a workgroup has 1 or 4 waves");
   YK_REQUIRE(yk_attn_mfma_supported(head_dim), "attn_mfma: head_dim must be 64 or 128");
@@ -902,7 +879,7 @@ extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* 
     else attn_mfma_kernel<DD, 4, false><<<grid, block, 0, stream>>>(YK_ARGS);                      \
   }                                                                                                \
   if (yk_check_launch("attn_mfma")) return -1;                                                     \
-  if (n_splits > 1) {                                                                              \
+  if (n_splits > 1 && !leave_splits) {                                                             \
     attn_combine_kernel<DD><<<dim3(n_tiles, n_kv * chunks), 256, 0, stream>>>(                     \
         static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 1);   \
     if (yk_check_launch("attn_combine")) return -1;                                                \
@@ -915,4 +892,27 @@ extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* 
 #undef YK_LAUNCH
 #undef YK_ARGS
   return 0;
+}
+
+// The second half of yk_attn_mfma for a launch that was told to leave its splits in the
+// workspace (leave_splits): merges them into `out`.  Same arguments as that launch had.
+extern "C" int yk_attn_combine(void* out, const int32_t* tiles, int n_tiles, int head_dim, int n_heads,
+                               int n_kv, int n_splits, const float* workspace, size_t workspace_floats,
+                               hipStream_t stream) {
+  YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_combine: bad head counts");
+  YK_REQUIRE(yk_attn_mfma_supported(head_dim), "attn_combine: head_dim must be 64 or 128");
+  YK_REQUIRE(n_splits > 1 && n_splits <= 65535, "attn_combine: nothing to merge");
+  if (n_tiles == 0) return 0;
+  const int hpt = attn_heads_per_tile(n_heads, n_kv);
+  const int chunks = (n_heads / n_kv + hpt - 1) / hpt;
+  const size_t need = yk_attn_mfma_workspace(n_tiles, n_heads, n_kv, head_dim, n_splits);
+  YK_REQUIRE(workspace && workspace_floats >= need, "attn_combine: workspace too small");
+  const float* ws_o = workspace;
+  const float* ws_ml = workspace + (need / (head_dim + 2)) * head_dim;
+  const dim3 grid(n_tiles, n_kv * chunks);
+  if (head_dim == 64)
+    attn_combine_kernel<64><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 1);
+  else
+    attn_combine_kernel<128><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 1);
+  return yk_check_launch("attn_combine");
 }

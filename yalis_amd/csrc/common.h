@@ -121,6 +121,57 @@ __device__ __forceinline__ float as_output(float v, int round_sum) {
   return round_sum ? to_f32<bf16_t>(from_f32<bf16_t>(v)) : v;
 }
 
+// ------------------------------------------------ attention whose keys were split across workgroups
+// Heads of one kv head that share a wave of the matrix-core attention (its 16 columns hold
+// 16 / heads_per_tile tokens of those heads); a kv group with more heads takes several
+// chunks of them.
+__host__ __device__ inline int attn_heads_per_tile(int n_heads, int n_kv) {
+  const int qpk = n_heads / n_kv;
+  return qpk < 16 ? qpk : 16;
+}
+
+// What the splits of a launch leave behind: for every group of 16 columns and split, the
+// unnormalised outputs [16][head_dim] in `o` and (running maximum, sum) pairs [16][2] in `ml`,
+// groups numbered (tile * groups_y + kv head * chunks + chunk) * n_splits + split.
+// Four consecutive output elements of one column, merged over its splits: weights
+// exp2(m_s - max m), in the order of s.  `col0` is the column's index in split 0
+// (group * 16 + column); split s lies 16 columns further each.
+__device__ __forceinline__ void attn_merge_splits(const float* __restrict__ o, const float* __restrict__ ml,
+                                                  size_t col0, int n_splits, int head_dim, int d,
+                                                  float out[4]) {
+  const float* mlc = ml + col0 * 2;
+  float m_max = -INFINITY;
+#pragma unroll 4
+  for (int s = 0; s < n_splits; ++s) m_max = fmaxf(m_max, mlc[static_cast<size_t>(s) * 32]);
+  float num[4] = {0.f, 0.f, 0.f, 0.f};
+  float den = 0.f;
+#pragma unroll 4
+  for (int s = 0; s < n_splits; ++s) {
+    const float w = exp2f(mlc[static_cast<size_t>(s) * 32] - m_max);
+    const float4 v = *reinterpret_cast<const float4*>(o + (col0 + static_cast<size_t>(s) * 16) * head_dim + d);
+    num[0] += w * v.x;
+    num[1] += w * v.y;
+    num[2] += w * v.z;
+    num[3] += w * v.w;
+    den += w * mlc[static_cast<size_t>(s) * 32 + 1];
+  }
+  const float inv = 1.f / den;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) out[e] = num[e] * inv;
+}
+
+// two floats to two bfloat16 (round to nearest even) in one word: gfx950 converts in hardware
+typedef __bf16 yk_bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float yk_f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  union {
+    yk_bf16x2_t v;
+    uint32_t u;
+  } c;
+  c.v = __builtin_convertvector(yk_f32x2_t{lo, hi}, yk_bf16x2_t);
+  return c.u;
+}
+
 __device__ __forceinline__ float block_sum(float v, float* scratch) {
   v = wave_sum(v);
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;

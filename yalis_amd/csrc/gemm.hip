@@ -138,15 +138,34 @@ static size_t skinny_lds_bytes(int mt, int waves) {
   return static_cast<size_t>(16 * mt * skinny_x_buffers(mt) + 16 * waves) * SK_ROW * sizeof(bf16_t);
 }
 
-template <int MT, int W, typename TO, int GATED>
+// Where the rows of x come from when they are the output of an attention whose keys were
+// split across workgroups and not yet merged (FROM_SPLITS): row m, column head * head_dim + d
+// is the merged value of column token_col[m] % 16 * heads_per_tile + (head's place in its
+// chunk) of tile token_col[m] / 16 (attn_merge_splits), rounded to bfloat16 as the merging
+// kernel would have stored it.
+struct AttnSplits {
+  const float* o;
+  const float* ml;
+  const int32_t* token_col;
+  int n_splits, n_heads, n_kv, head_dim, hpt, chunks;
+};
+constexpr int SK_SPLITS_MAX_K_BLOCK = 1024;  // a workgroup's whole slice of x then fits beside the weights
+
+template <int MT, int W, typename TO, int GATED, bool FROM_SPLITS>
 __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, float* __restrict__ part,
-    TO* __restrict__ y, int M, int N, int K, int ldx, int ldw, int ldy, int k_block) {
+    TO* __restrict__ y, int M, int N, int K, int ldx, int ldw, int ldy, int k_block, AttnSplits xa) {
+  static_assert(!FROM_SPLITS || (MT == 1 && GATED == 0), "unmerged attention feeds plain products of up to 16 rows");
   extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
   constexpr int XB = skinny_x_buffers(MT);
   bf16_t(*xs0)[SK_ROW] = reinterpret_cast<bf16_t(*)[SK_ROW]>(lds);  // XB x [16 * MT][SK_ROW]
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
-  bf16_t(*wl)[SK_ROW] = reinterpret_cast<bf16_t(*)[SK_ROW]>(lds + static_cast<size_t>(16 * MT * XB + 16 * wave) * SK_ROW);  // this wave's [16][SK_ROW]
+  // FROM_SPLITS: the workgroup's whole slice of x, [16][k_block + SK_PAD], merged once before the loop
+  const int x_all_row = k_block + SK_PAD;
+  bf16_t* x_all = lds;
+  bf16_t(*wl)[SK_ROW] = reinterpret_cast<bf16_t(*)[SK_ROW]>(
+      lds + (FROM_SPLITS ? static_cast<size_t>(16) * x_all_row : static_cast<size_t>(16 * MT * XB) * SK_ROW) +
+      static_cast<size_t>(16 * wave) * SK_ROW);  // this wave's [16][SK_ROW]
   const int r = lane % 16, g = lane / 16;
   const int n0 = (blockIdx.x * W + wave) * 16;
   const int m0 = blockIdx.y * (16 * MT);
@@ -186,7 +205,33 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
   }
 
   SK_LOAD_W(kb0)
-  SK_LOAD_X(kb0)
+  if (FROM_SPLITS) {
+    // (the first chunk of the weights is in flight meanwhile)
+    const int pieces = k_block / 4;
+    const int qpk = xa.n_heads / xa.n_kv;
+    // rows beyond M stand as zeros
+    for (int e = M * pieces + threadIdx.x; e < 16 * pieces; e += W * 64)
+      *reinterpret_cast<u32x2_t*>(x_all + static_cast<size_t>(e / pieces) * x_all_row + (e % pieces) * 4) = u32x2_t{0u, 0u};
+    // (unrolled: the loads of four pieces are in flight together)
+#pragma unroll 4
+    for (int e = threadIdx.x; e < M * pieces; e += W * 64) {
+      const int m = e / pieces, kk = (e % pieces) * 4, k = kb0 + kk;
+      u32x2_t piece = {0u, 0u};
+      if (k < K) {
+        const int tc = xa.token_col[m];
+        const int head = k / xa.head_dim, d = k % xa.head_dim;
+        const int hq = head % qpk;
+        const size_t group = static_cast<size_t>(tc / 16) * (xa.n_kv * xa.chunks) + (head / qpk) * xa.chunks + hq / xa.hpt;
+        float merged[4];
+        attn_merge_splits(xa.o, xa.ml, group * xa.n_splits * 16 + (tc % 16) * xa.hpt + hq % xa.hpt, xa.n_splits, xa.head_dim, d, merged);
+        piece[0] = pack_bf16x2(merged[0], merged[1]);
+        piece[1] = pack_bf16x2(merged[2], merged[3]);
+      }
+      *reinterpret_cast<u32x2_t*>(x_all + static_cast<size_t>(m) * x_all_row + kk) = piece;
+    }
+  } else {
+    SK_LOAD_X(kb0)
+  }
   int turn = 0;
   for (int kc = kb0; kc < kb1; kc += SK_KC, turn ^= 1) {
     // With one buffer every wave must have read the previous chunk of x before it is
@@ -197,17 +242,21 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
     // park what has arrived, then put the next chunk's loads in flight
 #pragma unroll
     for (int j = 0; j < SK_STEPS; ++j) *reinterpret_cast<u32x4_t*>(&wl[2 * j + half][8 * l32]) = regs[j];
+    if (!FROM_SPLITS) {
 #pragma unroll
-    for (int p = 0; p < XP; ++p) {
-      // (zeroed here, not at the load: a select right behind the load would make the wave
-      // wait for everything it has just put in flight)
-      const int e = threadIdx.x + p * W * 64;
-      const bool outside = m0 + e / (SK_KC / 8) >= M || kc + 8 * (e % (SK_KC / 8)) >= kb1;
-      *reinterpret_cast<u32x4_t*>(&xs[e / (SK_KC / 8)][8 * (e % (SK_KC / 8))]) = outside ? zero : xr[p];
+      for (int p = 0; p < XP; ++p) {
+        // (zeroed here, not at the load: a select right behind the load would make the wave
+        // wait for everything it has just put in flight)
+        const int e = threadIdx.x + p * W * 64;
+        const bool outside = m0 + e / (SK_KC / 8) >= M || kc + 8 * (e % (SK_KC / 8)) >= kb1;
+        *reinterpret_cast<u32x4_t*>(&xs[e / (SK_KC / 8)][8 * (e % (SK_KC / 8))]) = outside ? zero : xr[p];
+      }
     }
     if (kc + SK_KC < kb1) {
       SK_LOAD_W(kc + SK_KC)
-      SK_LOAD_X(kc + SK_KC)
+      if (!FROM_SPLITS) {
+        SK_LOAD_X(kc + SK_KC)
+      }
     }
     __syncthreads();
     // The operands of the steps are read from LDS ahead of the products that take them (all
@@ -220,7 +269,9 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
   {                                                                                          \
     a[U].u = *reinterpret_cast<const u32x4_t*>(&wl[r][32 * (U) + 8 * g]);                    \
     _Pragma("unroll") for (int t = 0; t < MT; ++t)                                           \
-        b[U][t].u = *reinterpret_cast<const u32x4_t*>(&xs[16 * t + r][32 * (U) + 8 * g]);    \
+        b[U][t].u = FROM_SPLITS                                                              \
+            ? *reinterpret_cast<const u32x4_t*>(x_all + static_cast<size_t>(16 * t + r) * x_all_row + (kc - kb0) + 32 * (U) + 8 * g) \
+            : *reinterpret_cast<const u32x4_t*>(&xs[16 * t + r][32 * (U) + 8 * g]);          \
   }
 #pragma unroll
     for (int u = 0; u < AHEAD; ++u) SK_READ(u)
@@ -355,8 +406,25 @@ extern "C" int yk_gemm_skinny_splits(int M, int N, int K) { return skinny_plan(M
 
 template <typename TO>
 static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, int M, int N, int K,
-                         int ldx, int ldw, int ldy, int waves, int k_block, int splits, int gated, hipStream_t stream) {
+                         int ldx, int ldw, int ldy, int waves, int k_block, int splits, int gated, hipStream_t stream,
+                         const AttnSplits* from_splits = nullptr) {
   const int mt = skinny_mt(M);
+  if (from_splits) {
+    // x is attention's unmerged splits: one kernel form (up to 16 rows, four waves, no activation)
+    if (mt != 1 || waves != 4 || gated || k_block > SK_SPLITS_MAX_K_BLOCK)
+      return yk_fail("gemm_mfma_skinny: unmerged attention feeds plain products of up to 16 rows only");
+    dim3 grid((N + 16 * waves - 1) / (16 * waves), 1, splits);
+    const size_t lds = (static_cast<size_t>(16) * (k_block + SK_PAD) + static_cast<size_t>(16 * waves) * SK_ROW) * sizeof(bf16_t);
+    static bool raised = false;
+    if (!raised) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_kernel<1, 4, TO, 0, true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+        return yk_fail("gemm_mfma_skinny: cannot raise the LDS limit");
+      raised = true;
+    }
+    gemm_mfma_skinny_kernel<1, 4, TO, 0, true><<<grid, dim3(256), lds, stream>>>(nullptr, w, part, y, M, N, K, 0, ldw, ldy, k_block, *from_splits);
+    return yk_check_launch("gemm_mfma_skinny (from attention splits)");
+  }
   dim3 grid((N + 16 * waves - 1) / (16 * waves), (M + 16 * mt - 1) / (16 * mt), splits);
   YK_REQUIRE(grid.y <= 65535, "gemm_mfma_skinny: too many rows for one launch");
   dim3 block(waves * 64);
@@ -365,12 +433,12 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, i
   if (mt == MT_ && waves == W_ && gated == G_) {                                                        \
     static bool raised = false; /* allow more than the default 64 KB of dynamic LDS, once */           \
     if (!raised) {                                                                                      \
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_kernel<MT_, W_, TO, G_>), \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_kernel<MT_, W_, TO, G_, false>), \
                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)    \
         return yk_fail("gemm_mfma_skinny: cannot raise the LDS limit");                                 \
       raised = true;                                                                                    \
     }                                                                                                   \
-    gemm_mfma_skinny_kernel<MT_, W_, TO, G_><<<grid, block, lds, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block); \
+    gemm_mfma_skinny_kernel<MT_, W_, TO, G_, false><<<grid, block, lds, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block, AttnSplits{}); \
     return yk_check_launch("gemm_mfma_skinny");                                                         \
   }
   SK_GO(1, 4, 0) SK_GO(2, 4, 0) SK_GO(4, 4, 0)
@@ -379,6 +447,34 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, i
   }
 #undef SK_GO
   return yk_fail("gemm_mfma_skinny: no kernel for this plan");
+}
+
+// The few-row product for checked arguments: plan, launch, and the reduction of the K slices
+// unless the caller keeps them.  x, or (from_splits) attention's unmerged splits in its place.
+static int skinny_product(const bf16_t* xp, const AttnSplits* from_splits, const bf16_t* wp, void* y, int y_dtype,
+                          float* workspace, size_t workspace_floats, int M, int N, int K, int ldx, int ldw, int ldy,
+                          int keep_splits, int gated, hipStream_t stream) {
+  int k_block = 0, waves = 4;
+  const int splits = skinny_plan(M, N, K, &waves, &k_block);
+  YK_REQUIRE(!gated || splits == 1, "gemm_mfma_skinny: a gated product cannot split K");
+  if (splits == 1 && !keep_splits) {
+    int rc = y_dtype == YK_F32
+                 ? launch_skinny<float>(xp, wp, nullptr, static_cast<float*>(y), M, N, K, ldx, ldw, ldy, waves, k_block, 1, gated, stream, from_splits)
+                 : launch_skinny<bf16_t>(xp, wp, nullptr, static_cast<bf16_t*>(y), M, N, K, ldx, ldw, ldy, waves, k_block, 1, gated, stream, from_splits);
+    return rc;
+  }
+  YK_REQUIRE(workspace && workspace_floats >= static_cast<size_t>(splits) * M * N,
+             "gemm_mfma_skinny: workspace too small");
+  if (launch_skinny<float>(xp, wp, workspace, nullptr, M, N, K, ldx, ldw, ldy, waves, k_block, splits, 0, stream, from_splits)) return -1;
+  if (keep_splits) return splits;
+  const size_t total = static_cast<size_t>(M) * N;
+  const int rb = 256;
+  const int rg = static_cast<int>(std::min<size_t>((total + rb - 1) / rb, 65535));
+  if (y_dtype == YK_F32)
+    reduce_splits_kernel<float><<<rg, rb, 0, stream>>>(workspace, static_cast<float*>(y), M, N, ldy, splits);
+  else
+    reduce_splits_kernel<bf16_t><<<rg, rb, 0, stream>>>(workspace, static_cast<bf16_t*>(y), M, N, ldy, splits);
+  return yk_check_launch("reduce_splits");
 }
 
 // keep_splits != 0: leave the K slices unreduced in `workspace` ([splits][M][N] float32) for
@@ -402,27 +498,48 @@ extern "C" int yk_gemm_mfma_skinny(const void* x, const void* w, void* y, int y_
   YK_REQUIRE(!gated || (N % 16 == 0 && y_dtype == YK_BF16 && !keep_splits), "gemm_mfma_skinny: a gated product needs N % 16 == 0 and a bfloat16 result");
   YK_REQUIRE(y_dtype == YK_F32 || y_dtype == YK_BF16, "gemm_mfma_skinny: unsupported output dtype");
   if (M == 0) return 0;
+  return skinny_product(static_cast<const bf16_t*>(x), nullptr, static_cast<const bf16_t*>(w), y, y_dtype, workspace,
+                        workspace_floats, M, N, K, ldx, ldw, ldy, keep_splits, gated, stream);
+}
+
+// Whether yk_gemm_mfma_skinny_from_attention takes a product of these sizes: up to 16 rows, and
+// a plan whose K slices are short enough for a workgroup to hold its whole slice of x.
+extern "C" int yk_gemm_skinny_from_attention_ok(int M, int N, int K) {
+  if (M <= 0 || M > 16 || N <= 0 || K < 8 || K % 8) return 0;
   int k_block = 0, waves = 4;
-  const int splits = skinny_plan(M, N, K, &waves, &k_block);
-  YK_REQUIRE(!gated || splits == 1, "gemm_mfma_skinny: a gated product cannot split K");
-  const bf16_t* xp = static_cast<const bf16_t*>(x);
-  const bf16_t* wp = static_cast<const bf16_t*>(w);
-  if (splits == 1 && !keep_splits) {
-    int rc = y_dtype == YK_F32
-                 ? launch_skinny<float>(xp, wp, nullptr, static_cast<float*>(y), M, N, K, ldx, ldw, ldy, waves, k_block, 1, gated, stream)
-                 : launch_skinny<bf16_t>(xp, wp, nullptr, static_cast<bf16_t*>(y), M, N, K, ldx, ldw, ldy, waves, k_block, 1, gated, stream);
-    return rc;
-  }
-  YK_REQUIRE(workspace && workspace_floats >= static_cast<size_t>(splits) * M * N,
-             "gemm_mfma_skinny: workspace too small");
-  if (launch_skinny<float>(xp, wp, workspace, nullptr, M, N, K, ldx, ldw, ldy, waves, k_block, splits, 0, stream)) return -1;
-  if (keep_splits) return splits;
-  const size_t total = static_cast<size_t>(M) * N;
-  const int rb = 256;
-  const int rg = static_cast<int>(std::min<size_t>((total + rb - 1) / rb, 65535));
-  if (y_dtype == YK_F32)
-    reduce_splits_kernel<float><<<rg, rb, 0, stream>>>(workspace, static_cast<float*>(y), M, N, ldy, splits);
-  else
-    reduce_splits_kernel<bf16_t><<<rg, rb, 0, stream>>>(workspace, static_cast<bf16_t*>(y), M, N, ldy, splits);
-  return yk_check_launch("reduce_splits");
+  skinny_plan(M, N, K, &waves, &k_block);
+  return waves == 4 && k_block <= SK_SPLITS_MAX_K_BLOCK;
+}
+
+// yk_gemm_mfma_skinny with x = the output of a yk_attn_mfma launch that left its splits in
+// `attn_workspace` (leave_splits): the product merges them while it stages x, rounding to
+// bfloat16 as yk_attn_combine would have stored them.  M tokens (at most 16), K = n_heads *
+// head_dim; token_col[m] = 16 * (the token's tile in that launch) + (its place in the tile).
+extern "C" int yk_gemm_mfma_skinny_from_attention(const float* attn_workspace, size_t attn_workspace_floats,
+                                                  const int32_t* token_col, int n_tiles, int n_splits,
+                                                  int n_heads, int n_kv, int head_dim, const void* w, void* y,
+                                                  int y_dtype, float* workspace, size_t workspace_floats, int M,
+                                                  int N, int ldw, int ldy, int keep_splits, hipStream_t stream) {
+  YK_REQUIRE(n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0 && head_dim > 0 && head_dim % 4 == 0, "gemm from attention: bad head sizes");
+  YK_REQUIRE(n_splits > 1 && n_tiles > 0 && attn_workspace && token_col, "gemm from attention: no splits to merge");
+  const int K = n_heads * head_dim;
+  YK_REQUIRE(M >= 0 && N > 0 && ldw % 8 == 0 && ldw >= K && ldy >= N && reinterpret_cast<uintptr_t>(w) % 16 == 0,
+             "gemm from attention: bad sizes or alignment");
+  YK_REQUIRE(y_dtype == YK_F32 || y_dtype == YK_BF16, "gemm from attention: unsupported output dtype");
+  YK_REQUIRE(yk_gemm_skinny_from_attention_ok(M, N, K) || M == 0, "gemm from attention: takes up to 16 rows and short K slices (ask yk_gemm_skinny_from_attention_ok)");
+  if (M == 0) return 0;
+  AttnSplits xa;
+  xa.hpt = attn_heads_per_tile(n_heads, n_kv);
+  xa.chunks = (n_heads / n_kv + xa.hpt - 1) / xa.hpt;
+  const size_t cols = static_cast<size_t>(n_tiles) * n_kv * xa.chunks * n_splits * 16;
+  YK_REQUIRE(attn_workspace_floats >= cols * (head_dim + 2), "gemm from attention: the attention workspace is too small for these tiles");
+  xa.o = attn_workspace;
+  xa.ml = attn_workspace + cols * head_dim;
+  xa.token_col = token_col;
+  xa.n_splits = n_splits;
+  xa.n_heads = n_heads;
+  xa.n_kv = n_kv;
+  xa.head_dim = head_dim;
+  return skinny_product(nullptr, &xa, static_cast<const bf16_t*>(w), y, y_dtype, workspace, workspace_floats, M, N, K, 0,
+                        ldw, ldy, keep_splits, 0, stream);
 }

@@ -165,3 +165,23 @@ def attention_tiles(hb: HostBatch, tokens_per_tile: int, min_span: int = 1, max_
     if longest_first:
         rows.sort(key=lambda row: -(row[3] + row[2]))
     return np.array(rows, dtype=np.int32).reshape(-1, 4)
+
+
+def attention_token_columns(hb: HostBatch, tokens_per_tile: int, min_span: int = 1, max_span: int = 1 << 30) -> np.ndarray:
+    """For every token of the batch, where ``attention_tiles`` with the same arguments (and
+    no reordering) put it: 16 * (its tile) + (its place among the tile's tokens), or -1 for
+    tokens of spans outside min_span..max_span.  A product that merges an attention's
+    unmerged splits while it reads them finds a token's columns through this."""
+    cols = np.full(hb.n_tokens, -1, dtype=np.int32)
+    tile = 0
+    for i in range(hb.n_seqs):
+        q0 = int(hb.seq_qstart[i])
+        ql = int(hb.seq_qlen[i])
+        if not min_span <= ql <= max_span:
+            continue
+        for t in range(0, ql, tokens_per_tile):
+            n = min(tokens_per_tile, ql - t)
+            cols[q0 + t : q0 + t + n] = 16 * tile + np.arange(n, dtype=np.int32)
+            tile += 1
+    return cols
+

@@ -77,7 +77,13 @@ _SIGNATURES = {
         _c_int,
     ),
     "yk_attn_mfma": (
-        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _vp],
+        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _c_int, _vp],
+        _c_int,
+    ),
+    "yk_attn_combine": ([_vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_size_t, _vp], _c_int),
+    "yk_gemm_skinny_from_attention_ok": ([_c_int, _c_int, _c_int], _c_int),
+    "yk_gemm_mfma_skinny_from_attention": (
+        [_vp, _c_size_t, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
         _c_int,
     ),
 }
@@ -95,13 +101,20 @@ _LATER_SIGNATURES = {
         "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
     },
 }
-_ABI = 7
+_ABI = 8
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
 # above it the vendor library does.
 SKINNY_MAX_ROWS = 64
 # Waves the attention launch aims at when it decides how far to split the keys.
 ATTN_TARGET_WAVES = 1024
+# Tokens of a step up to which an attention leaves its splits unmerged for the product that
+# follows.  Every workgroup of that product merges its own slice of them again, so the saved
+# kernel pays for few tokens only.  Measured at the 8B shape, 1,024-token contexts (ms a step,
+# merged by a kernel of its own / by the product): 1 token 3.439 / 3.381, 2 tokens 3.471 /
+# 3.427, 3 tokens 3.505 / 3.499, 4 tokens 3.506 / 3.526, 8 tokens 3.635 / 3.695.  The kernel
+# takes up to 16.
+MERGE_IN_PRODUCT_MAX_TOKENS = 2
 
 
 class SplitSum:
@@ -131,6 +144,32 @@ class SplitSum:
 
     def float(self) -> torch.Tensor:
         return self.reduce()
+
+
+class SplitAttention:
+    """The output of an attention whose keys were split across workgroups, not yet merged:
+    it stands for a bfloat16 tensor [tokens, heads * head_dim].  ``HipOps.linear`` merges the
+    splits while it stages them as its input where its kernel can (up to 16 tokens), which
+    saves the merging kernel; ``merge()`` gives the tensor itself.  It lives in the library's
+    workspace: consume it before the next attention is launched."""
+
+    def __init__(self, ops, workspace, tiles, token_cols, n_tokens, n_heads, n_kv, head_dim, n_splits):
+        self.ops, self.workspace, self.tiles, self.token_cols = ops, workspace, tiles, token_cols
+        self.n_heads, self.n_kv, self.head_dim, self.n_splits = n_heads, n_kv, head_dim, n_splits
+        self.shape = (n_tokens, n_heads * head_dim)
+        self.dtype = torch.bfloat16
+        self.device = workspace.device
+
+    def merge(self) -> torch.Tensor:
+        ops = self.ops
+        out = torch.empty(self.shape, dtype=self.dtype, device=self.device)
+        ops._check(
+            ops.lib.yk_attn_combine(
+                out.data_ptr(), self.tiles.data_ptr(), self.tiles.shape[0], self.head_dim, self.n_heads, self.n_kv,
+                self.n_splits, self.workspace.data_ptr(), self.workspace.numel(), ops._stream(),
+            )
+        )
+        return out
 
 
 class HipOps:
@@ -290,6 +329,11 @@ class HipOps:
     def linear(self, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, partial_ok: bool = False):
         """x [M, K] . w [N, K]^T -> [M, N].  With ``partial_ok`` the result may come as a
         ``SplitSum`` for a consumer that adds the slices itself."""
+        if isinstance(x, SplitAttention):
+            y = self._linear_from_attention(x, w, out_dtype, partial_ok)
+            if y is not None:
+                return y
+            x = x.merge()
         self._rows(x, "linear input")
         self._rows(w, "linear weight")
         m, k = x.shape
@@ -319,6 +363,29 @@ class HipOps:
         16 / 25, down-proj 48 / 76, qkv 24 / 26, gate/up 102 / 57; 3B shapes: 13 / 21, 24 / 43,
         17 / 21, 46 / 31; 70B shapes (8,192 columns and more): the library's everywhere."""
         return m <= 192 and -(-n // 256) < 32
+
+    def _linear_from_attention(self, x: "SplitAttention", w: torch.Tensor, out_dtype, partial_ok: bool):
+        """The few-row product fed by attention's unmerged splits, or None where it does not
+        apply (the caller then merges them first)."""
+        m, k = x.shape
+        n = w.shape[0]
+        if (w.dim() != 2 or w.dtype != torch.bfloat16 or w.shape[1] != k or w.stride(1) != 1 or w.stride(0) % 8
+                or w.data_ptr() % 16 or not self._ask("yk_gemm_skinny_from_attention_ok", m, n, k)):
+            return None
+        splits = self._ask("yk_gemm_skinny_splits", m, n, k)
+        keep = bool(partial_ok and splits > 1)
+        ws = self._gemm_ws(splits * m * n) if splits > 1 else None
+        y = None if keep else torch.empty((m, n), dtype=out_dtype, device=w.device)
+        rc = self.lib.yk_gemm_mfma_skinny_from_attention(
+            x.workspace.data_ptr(), x.workspace.numel(), x.token_cols.data_ptr(), x.tiles.shape[0], x.n_splits,
+            x.n_heads, x.n_kv, x.head_dim, w.data_ptr(), _ptr(y), _code(out_dtype), _ptr(ws),
+            0 if ws is None else ws.numel(), m, n, w.stride(0), n, int(keep), self._stream(),
+        )
+        if rc < 0:
+            raise KernelError(self.lib.yk_last_error().decode())
+        if keep:
+            return SplitSum(ws[: splits * m * n].view(splits, m, n), out_dtype)
+        return y
 
     def _library_f32_out(self) -> bool:
         """Whether this torch's matrix product takes bfloat16 operands and gives float32."""
@@ -470,13 +537,15 @@ class HipOps:
 
     def attention(self, qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size,
                   scale, window, ctx, group, tiles, long_tiles=None, plan=None, long_plan=None,
-                  long_col_tiles: int = 1) -> torch.Tensor:
+                  long_col_tiles: int = 1, token_cols=None):
         """Queries are the first n_heads heads of each row of ``qkv`` (whatever follows
         them in the row is skipped); keys and values come from the cache through the
         block table of ``group``.  ``long_tiles`` hold up to
         ``attention_long_span_tile(n_heads, n_kv, long_col_tiles)`` tokens each.  ``plan``
         overrides ``attention_plan`` and ``long_plan`` ``attention_long_splits`` (tests,
-        measurements)."""
+        measurements).  With ``token_cols`` (``attention_token_columns`` of the same short
+        tiles) the caller takes a ``SplitAttention`` as well: what a step of up to 16 tokens,
+        none of them in a long tile, leaves when its keys were split across workgroups."""
         self._rows(qkv, "qkv")
         n = qkv.shape[0]
         bt = ctx.arrays[f"block_table_g{group}"]
@@ -517,13 +586,17 @@ class HipOps:
             waves, splits = plan or self.attention_plan(n_tiles * n_kv * chunks, key_blocks)
             ws_floats = self._ask("yk_attn_mfma_workspace", n_tiles, n_heads, n_kv, head_dim, splits)
             ws = self._ws(ws_floats) if ws_floats else None
+            leave = bool(token_cols is not None and splits > 1 and n <= MERGE_IN_PRODUCT_MAX_TOKENS and (long_tiles is None or long_tiles.shape[0] == 0))
             self._check(
                 self.lib.yk_attn_mfma(
                     qkv.data_ptr(), qkv.stride(0), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                     tiles.data_ptr(), n_tiles, bt.data_ptr(), bt.shape[1], page_size, head_dim, n_heads, n_kv,
-                    float(scale), int(window), waves, splits, _ptr(ws), 0 if ws is None else ws.numel(), self._stream(),
+                    float(scale), int(window), waves, splits, _ptr(ws), 0 if ws is None else ws.numel(), int(leave),
+                    self._stream(),
                 )
             )
+            if leave:
+                return SplitAttention(self, ws, tiles, token_cols, n, n_heads, n_kv, head_dim, splits)
         else:
             self._check(
                 self.lib.yk_attn_generic(

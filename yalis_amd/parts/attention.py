@@ -20,7 +20,7 @@ import numpy as np
 import torch
 
 from ..config.specs import PartSpec
-from ..engine.batch import attention_tiles
+from ..engine.batch import attention_tiles, attention_token_columns
 from ..weights.loader import TensorSpec
 from .base import POSITIONS, KVNeed, Mixer, Runtime, register_mixer
 
@@ -105,6 +105,7 @@ class Attention(Mixer):
         none = np.zeros((0, 4), dtype=np.int32)
         return {
             f"attention_tiles_{tpt}_upto{big}": lambda hb: attention_tiles(hb, tpt, 1, big),
+            f"attention_token_columns_{tpt}_upto{big}": lambda hb: attention_token_columns(hb, tpt, 1, big),
             f"attention_long_tiles_{big}": lambda hb: attention_tiles(hb, big, big + 1, longest_first=True)
             if self.long_col_tiles(hb) == 1 else none,
             f"attention_long_tiles_{big2}": lambda hb: attention_tiles(hb, big2, big + 1, longest_first=True)
@@ -157,5 +158,6 @@ class Attention(Mixer):
             ctx.arrays[f"attention_tiles_{self.tokens_per_tile}_upto{self.long_tile}"],
             ctx.arrays[f"attention_long_tiles_{self.long_tile_2 if col_tiles == 2 else self.long_tile}"],
             long_col_tiles=col_tiles,
+            token_cols=ctx.arrays[f"attention_token_columns_{self.tokens_per_tile}_upto{self.long_tile}"],
         )
         return ops.linear(out, self.w_o, self.rt.act_dtype, partial_ok=True)
