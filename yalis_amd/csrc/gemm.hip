@@ -117,8 +117,9 @@ union Frag8 {
 //
 // A workgroup of W waves (W = blockDim.x / 64, chosen per shape by the host) owns 16*W
 // weight rows (16 per wave) and 16*MT rows of x over one slice of K (blockIdx.z).  K is
-// walked in chunks of 256.  The chunk of x is staged in LDS once for all waves.  Every wave
-// streams its own 16 weight rows with loads that cover two rows x 512 contiguous bytes
+// walked in chunks of KC = 256 or 128 (skinny_chunk).  The chunk of x is staged in LDS once for all
+// waves.  Every wave streams its own 16 weight rows with loads that cover two rows x 512 contiguous
+// bytes (four x 256 with the short chunks)
 // each (measured on MI355X: that pattern reads about a fifth faster than the 16 rows x 64
 // bytes the matrix-core operand layout would ask of memory directly), parks the chunk in a
 // wave-private piece of LDS and reads it back in operand layout; the next chunk's loads
@@ -133,9 +134,25 @@ constexpr int SK_MAX_WAVES = 8;
 
 // x is parked in two buffers by turns where that costs no resident workgroup (up to 16 rows
 // of x): then one barrier a chunk is enough.  Measured: 2 to 5 % on the 8B shapes.
-static constexpr int skinny_x_buffers(int mt) { return mt == 1 ? 2 : 1; }
-static size_t skinny_lds_bytes(int mt, int waves) {
-  return static_cast<size_t>(16 * mt * skinny_x_buffers(mt) + 16 * waves) * SK_ROW * sizeof(bf16_t);
+static constexpr int skinny_x_buffers(int mt, int kc) { return mt == 1 || kc < SK_KC ? 2 : 1; }
+static size_t skinny_lds_bytes(int mt, int waves, int kc) {
+  return static_cast<size_t>(16 * mt * skinny_x_buffers(mt, kc) + 16 * waves) * (kc + SK_PAD) * sizeof(bf16_t);
+}
+// Chunks are 256 or 128 elements of K long (with 128 a load covers four weight rows x 256
+// bytes).  Short chunks leave room for the two buffers of x and for three workgroups a compute
+// unit at any number of rows, and a workgroup gets going sooner, which counts where K is split
+// and a workgroup has a few chunks only; long chunks keep more bytes in flight per wave, which
+// counts where a workgroup walks the whole of K (gate/up).
+// Measured on the 8B shapes (us, chunks of 256 / 128): 64 rows: qkv 17.0 / 15.3, o-proj 12.4 /
+// 11.1, down 29.0 / 27.3, gate/up 59 / 56.7; 32 rows: qkv 12.8 / 11.5, o-proj 9.7 / 9.2, down
+// 24.0 / 22.3, but gate/up 46.2 / 48.2; 8 rows: qkv 11.0 / 10.1, o-proj 8.1 / 8.0, down 21.0 / 20.4,
+// but gate/up 40.2 / 46.6.
+static int skinny_chunk(int mt, int splits) {
+  if (const char* force = getenv("YALIS_SKINNY_CHUNK")) {  // 128 or 256: for measurements
+    const int kc = atoi(force);
+    if (kc == 128 || kc == 256) return kc;
+  }
+  return mt == 4 || splits > 1 ? 128 : SK_KC;
 }
 
 // Where the rows of x come from when they are the output of an attention whose keys were
@@ -151,21 +168,24 @@ struct AttnSplits {
 };
 constexpr int SK_SPLITS_MAX_K_BLOCK = 1024;  // a workgroup's whole slice of x then fits beside the weights
 
-template <int MT, int W, typename TO, int GATED, bool FROM_SPLITS>
+template <int MT, int W, typename TO, int GATED, bool FROM_SPLITS, int KC>
 __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, float* __restrict__ part,
     TO* __restrict__ y, int M, int N, int K, int ldx, int ldw, int ldy, int k_block, AttnSplits xa) {
   static_assert(!FROM_SPLITS || (MT == 1 && GATED == 0), "unmerged attention feeds plain products of up to 16 rows");
   extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
-  constexpr int XB = skinny_x_buffers(MT);
-  bf16_t(*xs0)[SK_ROW] = reinterpret_cast<bf16_t(*)[SK_ROW]>(lds);  // XB x [16 * MT][SK_ROW]
+  constexpr int STEPS = KC / 32;               // matrix-core steps per chunk
+  constexpr int ROW = KC + SK_PAD;             // an LDS row
+  constexpr int LPR = KC / 8, RPL = 64 / LPR;  // lanes that load one weight row's chunk; rows per load
+  constexpr int XB = skinny_x_buffers(MT, KC);
+  bf16_t(*xs0)[ROW] = reinterpret_cast<bf16_t(*)[ROW]>(lds);  // XB x [16 * MT][ROW]
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
   // FROM_SPLITS: the workgroup's whole slice of x, [16][k_block + SK_PAD], merged once before the loop
   const int x_all_row = k_block + SK_PAD;
   bf16_t* x_all = lds;
-  bf16_t(*wl)[SK_ROW] = reinterpret_cast<bf16_t(*)[SK_ROW]>(
-      lds + (FROM_SPLITS ? static_cast<size_t>(16) * x_all_row : static_cast<size_t>(16 * MT * XB) * SK_ROW) +
-      static_cast<size_t>(16 * wave) * SK_ROW);  // this wave's [16][SK_ROW]
+  bf16_t(*wl)[ROW] = reinterpret_cast<bf16_t(*)[ROW]>(
+      lds + (FROM_SPLITS ? static_cast<size_t>(16) * x_all_row : static_cast<size_t>(16 * MT * XB) * ROW) +
+      static_cast<size_t>(16 * wave) * ROW);  // this wave's [16][ROW]
   const int r = lane % 16, g = lane / 16;
   const int n0 = (blockIdx.x * W + wave) * 16;
   const int m0 = blockIdx.y * (16 * MT);
@@ -176,23 +196,24 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  // weights: load j of a chunk covers rows 2j (lanes 0..31) and 2j+1 (lanes 32..63), 16 bytes a lane
-  const int half = lane / 32, l32 = lane % 32;
-  const bf16_t* wrow[SK_STEPS];
+  // weights: load j of a chunk covers rows RPL * j .. RPL * j + RPL - 1 (two rows x 512 bytes with chunks
+  // of 256, four x 256 bytes with chunks of 128), 16 bytes a lane
+  const int half = lane / LPR, l32 = lane % LPR;
+  const bf16_t* wrow[STEPS];
 #pragma unroll
-  for (int j = 0; j < SK_STEPS; ++j) wrow[j] = w + static_cast<size_t>(min(n0 + 2 * j + half, N - 1)) * ldw;
+  for (int j = 0; j < STEPS; ++j) wrow[j] = w + static_cast<size_t>(min(n0 + RPL * j + half, N - 1)) * ldw;
   const int k_last = K - 8;
-  u32x4_t regs[SK_STEPS];
+  u32x4_t regs[STEPS];
 #define SK_LOAD_W(KC0)                                                                      \
   {                                                                                          \
     const int kk_ = min((KC0) + 8 * l32, k_last);                                            \
-    _Pragma("unroll") for (int j = 0; j < SK_STEPS; ++j)                                     \
+    _Pragma("unroll") for (int j = 0; j < STEPS; ++j)                                     \
         regs[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wrow[j] + kk_)); \
   }
   // x: the chunk's 16*MT rows x 32 pieces of 16 bytes are spread over the threads, XP each;
   // what lies outside M or the slice is loaded from a clamped address and parked as zero
-  constexpr int XP = 16 * MT * (SK_KC / 8) / (W * 64);
-  static_assert(XP * W * 64 == 16 * MT * (SK_KC / 8), "x pieces must divide evenly over the threads");
+  constexpr int XP = 16 * MT * (KC / 8) / (W * 64);
+  static_assert(XP * W * 64 == 16 * MT * (KC / 8), "x pieces must divide evenly over the threads");
   const u32x4_t zero = {0u, 0u, 0u, 0u};
   u32x4_t xr[XP];
 #pragma unroll
@@ -200,7 +221,7 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
 #define SK_LOAD_X(KC0)                                                                      \
   _Pragma("unroll") for (int p = 0; p < XP; ++p) {                                           \
     const int e_ = threadIdx.x + p * W * 64;                                                 \
-    const int m_ = m0 + e_ / (SK_KC / 8), k_ = (KC0) + 8 * (e_ % (SK_KC / 8));               \
+    const int m_ = m0 + e_ / (KC / 8), k_ = (KC0) + 8 * (e_ % (KC / 8));               \
     if (m_ < M) xr[p] = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(m_) * ldx + min(k_, k_last)); \
   }
 
@@ -233,29 +254,29 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
     SK_LOAD_X(kb0)
   }
   int turn = 0;
-  for (int kc = kb0; kc < kb1; kc += SK_KC, turn ^= 1) {
+  for (int kc = kb0; kc < kb1; kc += KC, turn ^= 1) {
     // With one buffer every wave must have read the previous chunk of x before it is
     // overwritten.  With two, the buffer written now was last read two chunks ago, and every
     // wave finished that before it passed the previous chunk's barrier.
     if (XB == 1) __syncthreads();
-    bf16_t(*xs)[SK_ROW] = xs0 + (XB == 2 ? turn * 16 * MT : 0);
+    bf16_t(*xs)[ROW] = xs0 + (XB == 2 ? turn * 16 * MT : 0);
     // park what has arrived, then put the next chunk's loads in flight
 #pragma unroll
-    for (int j = 0; j < SK_STEPS; ++j) *reinterpret_cast<u32x4_t*>(&wl[2 * j + half][8 * l32]) = regs[j];
+    for (int j = 0; j < STEPS; ++j) *reinterpret_cast<u32x4_t*>(&wl[RPL * j + half][8 * l32]) = regs[j];
     if (!FROM_SPLITS) {
 #pragma unroll
       for (int p = 0; p < XP; ++p) {
         // (zeroed here, not at the load: a select right behind the load would make the wave
         // wait for everything it has just put in flight)
         const int e = threadIdx.x + p * W * 64;
-        const bool outside = m0 + e / (SK_KC / 8) >= M || kc + 8 * (e % (SK_KC / 8)) >= kb1;
-        *reinterpret_cast<u32x4_t*>(&xs[e / (SK_KC / 8)][8 * (e % (SK_KC / 8))]) = outside ? zero : xr[p];
+        const bool outside = m0 + e / (KC / 8) >= M || kc + 8 * (e % (KC / 8)) >= kb1;
+        *reinterpret_cast<u32x4_t*>(&xs[e / (KC / 8)][8 * (e % (KC / 8))]) = outside ? zero : xr[p];
       }
     }
-    if (kc + SK_KC < kb1) {
-      SK_LOAD_W(kc + SK_KC)
+    if (kc + KC < kb1) {
+      SK_LOAD_W(kc + KC)
       if (!FROM_SPLITS) {
-        SK_LOAD_X(kc + SK_KC)
+        SK_LOAD_X(kc + KC)
       }
     }
     __syncthreads();
@@ -263,8 +284,8 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
     // of the chunk's at once where the registers allow, else two steps ahead): written the
     // plain way, one read then its product, the compiler reuses one register set and every
     // product waits for an LDS round trip.
-    constexpr int AHEAD = MT >= 4 ? 2 : (MT == 2 ? 3 : SK_STEPS);
-    Frag8 a[SK_STEPS], b[SK_STEPS][MT];
+    constexpr int AHEAD = MT >= 4 ? 2 : (MT == 2 ? 3 : STEPS);
+    Frag8 a[STEPS], b[STEPS][MT];
 #define SK_READ(U)                                                                          \
   {                                                                                          \
     a[U].u = *reinterpret_cast<const u32x4_t*>(&wl[r][32 * (U) + 8 * g]);                    \
@@ -277,8 +298,8 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
     for (int u = 0; u < AHEAD; ++u) SK_READ(u)
     __builtin_amdgcn_sched_barrier(0);  // (the scheduler would otherwise move the reads back to their products)
 #pragma unroll
-    for (int u = 0; u < SK_STEPS; ++u) {
-      if (u + AHEAD < SK_STEPS) {
+    for (int u = 0; u < STEPS; ++u) {
+      if (u + AHEAD < STEPS) {
         SK_READ(u + AHEAD)
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -372,7 +393,7 @@ static int skinny_plan(int M, int N, int K, int* waves_out, int* k_block_out) {
   long best_s = 1;
   for (int w : {4}) {  // measured: four waves per workgroup beat eight on every shape tried
     const long rblocks = (ntiles + w - 1) / w;
-    const double resident = std::min(20.0, static_cast<double>(160 * 1024 / skinny_lds_bytes(mt, w)) * w);
+    const double resident = std::min(20.0, static_cast<double>(160 * 1024 / skinny_lds_bytes(mt, w, SK_KC)) * w);
     for (long s = 1; s <= max_s; ++s) {
       const long per = (chunks + s - 1) / s;          // chunks per workgroup
       const long real = (chunks + per - 1) / per;     // slices that are not empty
@@ -417,28 +438,30 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, i
     const size_t lds = (static_cast<size_t>(16) * (k_block + SK_PAD) + static_cast<size_t>(16 * waves) * SK_ROW) * sizeof(bf16_t);
     static bool raised = false;
     if (!raised) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_kernel<1, 4, TO, 0, true>),
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_kernel<1, 4, TO, 0, true, SK_KC>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
         return yk_fail("gemm_mfma_skinny: cannot raise the LDS limit");
       raised = true;
     }
-    gemm_mfma_skinny_kernel<1, 4, TO, 0, true><<<grid, dim3(256), lds, stream>>>(nullptr, w, part, y, M, N, K, 0, ldw, ldy, k_block, *from_splits);
+    gemm_mfma_skinny_kernel<1, 4, TO, 0, true, SK_KC><<<grid, dim3(256), lds, stream>>>(nullptr, w, part, y, M, N, K, 0, ldw, ldy, k_block, *from_splits);
     return yk_check_launch("gemm_mfma_skinny (from attention splits)");
   }
   dim3 grid((N + 16 * waves - 1) / (16 * waves), (M + 16 * mt - 1) / (16 * mt), splits);
   YK_REQUIRE(grid.y <= 65535, "gemm_mfma_skinny: too many rows for one launch");
   dim3 block(waves * 64);
-  const size_t lds = skinny_lds_bytes(mt, waves);
-#define SK_GO(MT_, W_, G_)                                                                               \
-  if (mt == MT_ && waves == W_ && gated == G_) {                                                        \
+  const int kc = skinny_chunk(mt, splits);
+  const size_t lds = skinny_lds_bytes(mt, waves, kc);
+#define SK_GO(MT_, W_, G_) SK_GO_KC(MT_, W_, G_, 128) SK_GO_KC(MT_, W_, G_, 256)
+#define SK_GO_KC(MT_, W_, G_, KC_)                                                                       \
+  if (mt == MT_ && waves == W_ && gated == G_ && kc == KC_) {                                           \
     static bool raised = false; /* allow more than the default 64 KB of dynamic LDS, once */           \
     if (!raised) {                                                                                      \
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_kernel<MT_, W_, TO, G_, false>), \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_kernel<MT_, W_, TO, G_, false, KC_>), \
                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)    \
         return yk_fail("gemm_mfma_skinny: cannot raise the LDS limit");                                 \
       raised = true;                                                                                    \
     }                                                                                                   \
-    gemm_mfma_skinny_kernel<MT_, W_, TO, G_, false><<<grid, block, lds, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block, AttnSplits{}); \
+    gemm_mfma_skinny_kernel<MT_, W_, TO, G_, false, KC_><<<grid, block, lds, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block, AttnSplits{}); \
     return yk_check_launch("gemm_mfma_skinny");                                                         \
   }
   SK_GO(1, 4, 0) SK_GO(2, 4, 0) SK_GO(4, 4, 0)
@@ -446,6 +469,7 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, i
     SK_GO(1, 4, 1) SK_GO(2, 4, 1) SK_GO(4, 4, 1) SK_GO(1, 4, 2) SK_GO(2, 4, 2) SK_GO(4, 4, 2)
   }
 #undef SK_GO
+#undef SK_GO_KC
   return yk_fail("gemm_mfma_skinny: no kernel for this plan");
 }
 
