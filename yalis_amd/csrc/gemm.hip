@@ -140,19 +140,21 @@ static size_t skinny_lds_bytes(int mt, int waves, int kc) {
 }
 // Chunks are 256 or 128 elements of K long (with 128 a load covers four weight rows x 256
 // bytes).  Short chunks leave room for the two buffers of x and for three workgroups a compute
-// unit at any number of rows, and a workgroup gets going sooner, which counts where K is split
-// and a workgroup has a few chunks only; long chunks keep more bytes in flight per wave, which
-// counts where a workgroup walks the whole of K (gate/up).
+// unit at any number of rows, and a workgroup gets going sooner, which counts where a
+// workgroup walks a short slice of K; long chunks keep more bytes in flight per wave, which
+// counts where it walks a long one (gate/up, the output head, the slices of the 70B shape).
 // Measured on the 8B shapes (us, chunks of 256 / 128): 64 rows: qkv 17.0 / 15.3, o-proj 12.4 /
 // 11.1, down 29.0 / 27.3, gate/up 59 / 56.7; 32 rows: qkv 12.8 / 11.5, o-proj 9.7 / 9.2, down
 // 24.0 / 22.3, but gate/up 46.2 / 48.2; 8 rows: qkv 11.0 / 10.1, o-proj 8.1 / 8.0, down 21.0 / 20.4,
-// but gate/up 40.2 / 46.6.
-static int skinny_chunk(int mt, int splits) {
+// but gate/up 40.2 / 46.6; the 70B shape's decode step at 64 rows (slices of 2,048 to 8,192):
+// 36.9 / 37.7 ms, and its o-proj at 8 rows (slices of 2,048) is faster with long chunks too.  So:
+// short chunks for slices of up to 1,792, up to 4,096 with 64 rows of x.
+static int skinny_chunk(int mt, int k_block) {
   if (const char* force = getenv("YALIS_SKINNY_CHUNK")) {  // 128 or 256: for measurements
     const int kc = atoi(force);
     if (kc == 128 || kc == 256) return kc;
   }
-  return mt == 4 || splits > 1 ? 128 : SK_KC;
+  return k_block <= (mt == 4 ? 16 : 7) * SK_KC ? 128 : SK_KC;
 }
 
 // Where the rows of x come from when they are the output of an attention whose keys were
@@ -382,12 +384,16 @@ static int skinny_mt(int M) { return M <= 16 ? 1 : (M <= 32 ? 2 : 4); }
 // A caller that takes the slices unreduced needs splits * M * N floats.
 constexpr int SK_CUS = 256;
 
-static int skinny_plan(int M, int N, int K, int* waves_out, int* k_block_out) {
+static int skinny_plan(int M, int N, int K, bool gated, int* waves_out, int* k_block_out) {
   const int mt = skinny_mt(M);
   const long mtiles = (M + 16 * mt - 1) / (16 * mt);
   const long ntiles = (N + 15) / 16;
   const long chunks = (K + SK_KC - 1) / SK_KC;
-  const long max_s = std::max(1L, std::min(32L, chunks / 2));
+  // A product with the activation in its epilogue cannot split K; where its row blocks alone
+  // occupy every compute unit it is not split (the fused epilogue saves a kernel and a pass over
+  // the slices: the decode step of the 3B shape went 2.17 -> 2.10 ms at 8 rows, that of the 70B
+  // shape 26.1 -> 25.8).
+  const long max_s = gated && (ntiles + 3) / 4 * mtiles >= SK_CUS ? 1 : std::max(1L, std::min(32L, chunks / 2));
   double best = 1e300;
   int best_w = 4;
   long best_s = 1;
@@ -423,7 +429,8 @@ static int skinny_plan(int M, int N, int K, int* waves_out, int* k_block_out) {
   return static_cast<int>((K + k_block - 1) / k_block);
 }
 
-extern "C" int yk_gemm_skinny_splits(int M, int N, int K) { return skinny_plan(M, N, K, nullptr, nullptr); }
+// gated != 0: the plan of a product with the activation in its epilogue (1: it can be fused).
+extern "C" int yk_gemm_skinny_splits(int M, int N, int K, int gated) { return skinny_plan(M, N, K, gated != 0, nullptr, nullptr); }
 
 template <typename TO>
 static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, int M, int N, int K,
@@ -449,7 +456,7 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, i
   dim3 grid((N + 16 * waves - 1) / (16 * waves), (M + 16 * mt - 1) / (16 * mt), splits);
   YK_REQUIRE(grid.y <= 65535, "gemm_mfma_skinny: too many rows for one launch");
   dim3 block(waves * 64);
-  const int kc = skinny_chunk(mt, splits);
+  const int kc = skinny_chunk(mt, k_block);
   const size_t lds = skinny_lds_bytes(mt, waves, kc);
 #define SK_GO(MT_, W_, G_) SK_GO_KC(MT_, W_, G_, 128) SK_GO_KC(MT_, W_, G_, 256)
 #define SK_GO_KC(MT_, W_, G_, KC_)                                                                       \
@@ -479,7 +486,7 @@ static int skinny_product(const bf16_t* xp, const AttnSplits* from_splits, const
                           float* workspace, size_t workspace_floats, int M, int N, int K, int ldx, int ldw, int ldy,
                           int keep_splits, int gated, hipStream_t stream) {
   int k_block = 0, waves = 4;
-  const int splits = skinny_plan(M, N, K, &waves, &k_block);
+  const int splits = skinny_plan(M, N, K, gated != 0, &waves, &k_block);
   YK_REQUIRE(!gated || splits == 1, "gemm_mfma_skinny: a gated product cannot split K");
   if (splits == 1 && !keep_splits) {
     int rc = y_dtype == YK_F32
@@ -531,7 +538,7 @@ extern "C" int yk_gemm_mfma_skinny(const void* x, const void* w, void* y, int y_
 extern "C" int yk_gemm_skinny_from_attention_ok(int M, int N, int K) {
   if (M <= 0 || M > 16 || N <= 0 || K < 8 || K % 8) return 0;
   int k_block = 0, waves = 4;
-  skinny_plan(M, N, K, &waves, &k_block);
+  skinny_plan(M, N, K, false, &waves, &k_block);
   return waves == 4 && k_block <= SK_SPLITS_MAX_K_BLOCK;
 }
 

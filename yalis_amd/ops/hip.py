@@ -58,7 +58,7 @@ _SIGNATURES = {
         [_vp, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
         _c_int,
     ),
-    "yk_gemm_skinny_splits": ([_c_int, _c_int, _c_int], _c_int),
+    "yk_gemm_skinny_splits": ([_c_int, _c_int, _c_int, _c_int], _c_int),
     "yk_gemm_mfma_skinny": (
         [_vp, _vp, _vp, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
         _c_int,
@@ -101,7 +101,7 @@ _LATER_SIGNATURES = {
         "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
     },
 }
-_ABI = 8
+_ABI = 9
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
 # above it the vendor library does.
@@ -372,7 +372,7 @@ class HipOps:
         if (w.dim() != 2 or w.dtype != torch.bfloat16 or w.shape[1] != k or w.stride(1) != 1 or w.stride(0) % 8
                 or w.data_ptr() % 16 or not self._ask("yk_gemm_skinny_from_attention_ok", m, n, k)):
             return None
-        splits = self._ask("yk_gemm_skinny_splits", m, n, k)
+        splits = self._ask("yk_gemm_skinny_splits", m, n, k, 0)
         keep = bool(partial_ok and splits > 1)
         ws = self._gemm_ws(splits * m * n) if splits > 1 else None
         y = None if keep else torch.empty((m, n), dtype=out_dtype, device=w.device)
@@ -439,7 +439,7 @@ class HipOps:
             group == self.GATE_UP_GROUP and 0 < m <= SKINNY_MAX_ROWS and x.dtype == bf and w_gate_up.dtype == bf and out_dtype == bf
             and w_gate_up.shape[1] == k and k % 8 == 0 and x.stride(0) % 8 == 0 and w_gate_up.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0 and n % 16 == 0
-            and self._ask("yk_gemm_skinny_splits", m, n, k) == 1
+            and self._ask("yk_gemm_skinny_splits", m, n, k, 1) == 1
         )
         if not fused:
             return self.gated_act(self.linear(x, w_gate_up, out_dtype, partial_ok=True), activation, out_dtype, group=group)
@@ -455,7 +455,7 @@ class HipOps:
     def gemm_mfma_skinny(self, x, w, out_dtype, partial_ok: bool = False):
         m, k = x.shape
         n = w.shape[0]
-        splits = self._ask("yk_gemm_skinny_splits", m, n, k)
+        splits = self._ask("yk_gemm_skinny_splits", m, n, k, 0)
         keep = bool(partial_ok and splits > 1)
         ws = self._gemm_ws(splits * m * n) if splits > 1 else None
         y = None if keep else torch.empty((m, n), dtype=out_dtype, device=x.device)
