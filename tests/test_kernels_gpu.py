@@ -142,6 +142,23 @@ def test_gemm_mfma_skinny(ops, m, n, k, od):
         close(got, want, 1e-2, 2**-8)
 
 
+@pytest.mark.parametrize("chunk", ["128", "256"])
+def test_gemm_mfma_skinny_chunk_lengths(ops, chunk, monkeypatch):
+    """The few-row product walks K in chunks of 256 or 128, chosen by the length of a
+    workgroup's slice; here each length is forced in turn on every row-tile count, on split
+    and unsplit products, on K that is no multiple of the chunk, and on the fused activation."""
+    monkeypatch.setenv("YALIS_SKINNY_CHUNK", chunk)
+    for m, n, k in [(8, 200, 4096), (3, 515, 200), (24, 130, 2056), (40, 96, 1000), (64, 520, 328), (100, 64, 4096)]:
+        x = rnd((m, k), torch.bfloat16, 6)
+        w = rnd((n, k), torch.bfloat16, 7)
+        close(ops.gemm_mfma_skinny(x, w, torch.float32), x.double().cpu() @ w.double().cpu().T, 2e-5 * math.sqrt(k), 1e-5)
+    for m, k, inter in [(8, 4096, 512), (30, 392, 200), (64, 1024, 264)]:
+        x = rnd((m, k), torch.bfloat16, 30, 0.7)
+        packed, group = ops.pack_gate_up(rnd((inter, k), torch.bfloat16, 31, 0.05), rnd((inter, k), torch.bfloat16, 32, 0.05))
+        got = ops.gate_up_act(x, packed, group, "silu", torch.bfloat16)
+        assert torch.equal(got, ops.gated_act(ops.linear(x, packed, torch.bfloat16), "silu", torch.bfloat16, group=group))
+
+
 def test_gemm_mfma_operand_order(ops):
     """One-hot operands name the element each lane must hold: y[m, n] = x[m, kx] * w[n, kx]
     for a single k picks out any mismatch between the two operands' k order."""
