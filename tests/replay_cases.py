@@ -102,6 +102,40 @@ def trace_mixed(reqs, sizes=PORTIONS, decode_tail: int = 12, max_live: int = 4) 
     return steps
 
 
+def trace_random(reqs, seed: int, max_live: int = 4) -> List[dict]:
+    """A trace cut at random: up to ``max_live`` requests at a time, each step a random
+    subset of them (at least one), each with a random number of its next tokens (often one,
+    sometimes many, rarely all that is left)."""
+    import random
+
+    rng = random.Random(seed)
+    waiting = list(reqs.items())
+    rng.shuffle(waiting)
+    live: List[Tuple[str, List[int], int]] = []
+    steps = []
+    while waiting or live:
+        while waiting and len(live) < max_live and (not live or rng.random() < 0.7):
+            rid, toks = waiting.pop(0)
+            live.append((rid, toks, 0))
+        chosen = [i for i in range(len(live)) if rng.random() < 0.75] or [rng.randrange(len(live))]
+        entries, ends, nxt = [], [], []
+        for i, (rid, toks, done) in enumerate(live):
+            if i not in chosen:
+                nxt.append((rid, toks, done))
+                continue
+            left = len(toks) - done
+            kind = rng.random()
+            size = 1 if kind < 0.4 else (left if kind > 0.95 else rng.randint(1, min(left, rng.choice([2, 3, 7, 16, 33, 64]))))
+            entries.append({"id": rid, "tokens": toks[done : done + size], "want": list(range(size))})
+            if done + size == len(toks):
+                ends.append(rid)
+            else:
+                nxt.append((rid, toks, done + size))
+        steps.append({"step": len(steps), "entries": entries, "end": ends})
+        live = nxt
+    return steps
+
+
 def pages_needed(steps: List[dict], reqs, page_size: int) -> int:
     """The most pages live requests hold at any time, each request counted at its full
     length rounded up to whole pages."""

@@ -86,6 +86,23 @@ FULL_WIDTH = {
     "vocab_size": 128256, "rms_norm_eps": 1e-5, "rope_theta": 500000.0, "rope_scaling": None,
     "max_position_embeddings": 8192, "tie_word_embeddings": False,
 }
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name,seed", [("A", 1), ("B", 2), ("C", 3), ("D", 4), ("E", 5), ("C", 6), ("D", 7)])
+def test_replay_cut_at_random(backend, name, seed):
+    """Random subsets of up to four live requests a step, random numbers of tokens each, a
+    pool just large enough: the logits are the plain implementation's, and no page is lost."""
+    device, dtype = backend
+    cfg, weights, reqs, want = setup(name, dtype)
+    steps = C.trace_random(reqs, seed)
+    page = PAGE[name]
+    n_pages = C.pages_needed(steps, reqs, page)
+    runner = C.make_runner(cfg, weights, dtype, device, ops_for(device), page, n_pages)
+    got, _ = C.run_trace(runner, steps)
+    C.assert_matches(got, want, dtype == "bfloat16", f"{name}/random {seed}")
+    runner.pages.audit()
+    assert runner.pages.live_requests() == 0 and runner.pages.free_pages(0) == n_pages
+
+
 _full_width = {}
 
 
@@ -107,7 +124,8 @@ def test_full_width_replay(dtype):
     bf16 = dtype == "bfloat16"
     weights, reqs, want = full_width_setup(bf16)
     runner = None
-    for mode, make in (("whole", C.trace_whole), ("tail", C.trace_tail), ("portions", C.trace_portions), ("mixed", C.trace_mixed)):
+    for mode, make in (("whole", C.trace_whole), ("tail", C.trace_tail), ("portions", C.trace_portions), ("mixed", C.trace_mixed),
+                       ("random", lambda r: C.trace_random(r, 11))):
         steps = make(reqs)
         n_pages = C.pages_needed(steps, reqs, 64)
         del runner
