@@ -232,13 +232,15 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
   // otherwise ask for addresses a whole number of rows apart at every moment, which crowd onto
   // few memory channels: where the rows are a multiple of 4 KiB apart, that is (measured at the 8B
   // shape, 8 rows: gate/up 40.2 -> 37.6 us; the decode step 3.60 -> 3.53 ms, that of the 70B shape
-  // 25.9 -> 25.1; with rows 6 KiB apart, the 3B shape, it cost half a percent).  (The unit does not
+  // 25.9 -> 25.1; with rows 6 KiB apart, the 3B shape, it cost half a percent; with 64 rows of x,
+  // where every workgroup stages as many bytes of x as of the weight and those reads are shared only
+  // by workgroups at the same place, gate/up went 56.9 -> 59.4 us, so not there).  (The unit does not
   // depend on the chunk length, so the order of the sums does not either.)
   const int n_chunks = (kb1 - kb0 + KC - 1) / KC;
   constexpr int PER_UNIT = SK_KC / KC;              // chunks in a unit of 256
   const int n_units = (kb1 - kb0 + SK_KC - 1) / SK_KC;
   const int slots = PER_UNIT * n_units;             // the last one may lie beyond the slice
-  const int first_slot = ldw % 2048 == 0 ? static_cast<int>(blockIdx.x % n_units) * PER_UNIT : 0;
+  const int first_slot = MT < 4 && ldw % 2048 == 0 ? static_cast<int>(blockIdx.x % n_units) * PER_UNIT : 0;
   const bool last_missing = slots > n_chunks;
   const int missing_at = slots - 1 - first_slot;    // where the last slot comes in this workgroup's order
   auto chunk_start = [&](int i) {
