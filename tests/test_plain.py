@@ -190,3 +190,114 @@ def test_sampling_rules():
     u = P.race_uniforms(3, 0, 1000)
     assert 0 < u.min() and u.max() < 1 and abs(u.mean() - 0.5) < 0.05
     assert not (P.race_uniforms(3, 1, 1000) == u).all() and not (P.race_uniforms(4, 0, 1000) == u).all()
+
+
+# ----------------------------------------------------------------- the block's wiring
+def _wiring_holds(layer_fn, cfg, seed=0):
+    """What yalis/external/model.py:414-439 (parallel_residual=False, identity post-norms)
+    says of one layer, checked on ``layer_fn(cfg, weights, 0, x, positions)`` with library
+    routines only:  x1 = x + o_proj(attention(norm_1(x)));  out = x1 + mlp(norm_2(x1)).
+    Raises AssertionError at the first statement that does not hold."""
+    w = P.random_weights(cfg, seed)
+    # larger projections than the usual 0.02, so that each branch changes the residual by
+    # about as much as the residual itself: a branch fed from the wrong place then shows
+    for n in list(w):
+        if n.endswith("proj.weight"):
+            w[n] = w[n] * 8.0
+    c = cfg["hidden_size"]
+    eps = cfg["rms_norm_eps"]
+    t = 11
+    g = torch.Generator().manual_seed(seed + 1)
+    x = torch.randn(t, c, generator=g)
+    pos = torch.arange(3, 3 + t)
+    p = "model.layers.0."
+
+    def mlp(h):
+        return (F.silu(h @ w[p + "mlp.gate_proj.weight"].T) * (h @ w[p + "mlp.up_proj.weight"].T)) @ w[p + "mlp.down_proj.weight"].T
+
+    def without(*names):
+        z = dict(w)
+        for n in names:
+            z[p + n] = torch.zeros_like(w[p + n])
+        return z
+
+    # both branches silent: the layer is the identity (a norm on the residual path, as in a
+    # post-norm block, would change x here)
+    both = layer_fn(cfg, without("self_attn.o_proj.weight", "mlp.down_proj.weight"), 0, x, pos)
+    assert torch.equal(both, x), "with o_proj and down_proj zero a pre-norm layer is the identity"
+    # attention silent: what is left is x + mlp(norm_2(x)), with norm_2's own weight
+    no_attn = layer_fn(cfg, without("self_attn.o_proj.weight"), 0, x, pos)
+    want = x + mlp(F.rms_norm(x, (c,), w[p + "post_attention_layernorm.weight"], eps))
+    assert torch.allclose(no_attn, want, atol=1e-5), "the feed-forward reads norm_2 of the residual"
+    # feed-forward silent: x1 = x + attention branch, which reads norm_1(x)
+    x1 = layer_fn(cfg, without("mlp.down_proj.weight"), 0, x, pos)
+    n_head, n_group = cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    d = cfg["head_dim"]
+    h = F.rms_norm(x, (c,), w[p + "input_layernorm.weight"], eps)
+    cos, sin = P.rope_cos_sin(pos, P.rope_inv_freq(d, cfg["rope_theta"], cfg.get("rope_scaling")))
+    q = P.apply_rope((h @ w[p + "self_attn.q_proj.weight"].T).view(t, n_head, d), cos, sin)
+    k = P.apply_rope((h @ w[p + "self_attn.k_proj.weight"].T).view(t, n_group, d), cos, sin)
+    v = (h @ w[p + "self_attn.v_proj.weight"].T).view(t, n_group, d)
+    a = F.scaled_dot_product_attention(
+        q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None], is_causal=True, enable_gqa=True
+    )[0].transpose(0, 1).reshape(t, n_head * d)
+    assert torch.allclose(x1, x + a @ w[p + "self_attn.o_proj.weight"].T, atol=1e-5), "the attention reads norm_1 of the residual"
+    # both: the feed-forward reads the residual AFTER the attention was added (sequential, not
+    # parallel: a parallel block would feed it norm_2(x))
+    full = layer_fn(cfg, w, 0, x, pos)
+    want = x1 + mlp(F.rms_norm(x1, (c,), w[p + "post_attention_layernorm.weight"], eps))
+    assert torch.allclose(full, want, atol=1e-5), "the feed-forward reads the residual after the attention's contribution"
+    apart = (full - (x1 + mlp(F.rms_norm(x, (c,), w[p + "post_attention_layernorm.weight"], eps)))).abs().max()
+    assert apart > 1e-2, "the two arrangements must differ on this input for the pin to mean anything"
+
+
+def _parallel_residual_layer(cfg, weights, layer, x, positions, rounder=P._identity, window=None):
+    """A deliberate mistake: x + attention(norm_1(x)) + mlp(norm_2(x)) (the reference's
+    parallel_residual=True arrangement, yalis/external/model.py:427-431), built from the
+    plain implementation's own branches."""
+    p = f"model.layers.{layer}."
+    silent_mlp = dict(weights)
+    silent_mlp[p + "mlp.down_proj.weight"] = torch.zeros_like(weights[p + "mlp.down_proj.weight"])
+    silent_attn = dict(weights)
+    silent_attn[p + "self_attn.o_proj.weight"] = torch.zeros_like(weights[p + "self_attn.o_proj.weight"])
+    attn = P.layer_forward(cfg, silent_mlp, layer, x, positions) - x
+    ff = P.layer_forward(cfg, silent_attn, layer, x, positions) - x
+    return x + attn + ff
+
+
+def _post_norm_layer(cfg, weights, layer, x, positions, rounder=P._identity, window=None):
+    """Another: the norms applied after the residual sums instead of before the branches."""
+    p = f"model.layers.{layer}."
+    c, eps = cfg["hidden_size"], cfg["rms_norm_eps"]
+    ones = dict(weights)
+    ones[p + "input_layernorm.weight"] = torch.ones(c)
+    ones[p + "post_attention_layernorm.weight"] = torch.ones(c)
+    return P.rms_norm(P.layer_forward(cfg, ones, layer, x, positions), weights[p + "post_attention_layernorm.weight"], eps)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_block_wiring(name):
+    """The arrangement of a layer is pinned by library routines alone, and the pin has
+    teeth: a parallel-residual layer and a post-norm layer both fail it.  (The reference's own
+    tests compare whole models with another library's model code at run time,
+    tests/basic_correctness/test_yalis_vs_hf.py:53-100; that library's model code is not a
+    source here, so the wiring is pinned by these identities instead.)"""
+    cfg = ALL[name]
+    _wiring_holds(P.layer_forward, cfg)
+    with pytest.raises(AssertionError):
+        _wiring_holds(_parallel_residual_layer, cfg)
+    with pytest.raises(AssertionError):
+        _wiring_holds(_post_norm_layer, cfg)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_silent_branches_reduce_the_model_to_no_layers(name):
+    """With every o_proj and down_proj zero the whole model equals the model without
+    layers (embedding, final norm, head), whatever the other weights are."""
+    cfg = ALL[name]
+    w = P.random_weights(cfg, seed=3)
+    for i in range(cfg["num_hidden_layers"]):
+        for n in ("self_attn.o_proj.weight", "mlp.down_proj.weight"):
+            w[f"model.layers.{i}.{n}"] = torch.zeros_like(w[f"model.layers.{i}.{n}"])
+    toks = torch.randint(0, cfg["vocab_size"], (9,), generator=torch.Generator().manual_seed(4)).tolist()
+    assert torch.equal(P.forward(cfg, w, toks), P.forward(cfg, w, toks, n_layers=0))
