@@ -20,8 +20,11 @@
 // in the reference, which compares with the k-th value), and tokens tied with the one that
 // crosses top_p are dropped together (the reference's sort leaves their order undefined).
 #include <algorithm>
+#include <mutex>
+#include <string>
 
 #include "common.h"
+#include "no_alloc.h"
 
 __device__ __forceinline__ uint64_t mix64(uint64_t z) {
   z += 0x9E3779B97F4A7C15ull;
@@ -137,6 +140,56 @@ extern "C" int yk_argmax(const float* logits, int32_t* out, int n_rows, int voca
   }
   argmax_kernel<<<n_rows, 1024, 0, stream>>>(logits, out, vocab);
   return yk_check_launch("argmax");
+}
+
+// ------------------------------------------------- argmax without any allocation (no_alloc.h)
+// The partial results of argmax_part_kernel for up to YK_ARGMAX_STATIC_MAX_ROWS rows: the
+// values, then the indices.  In host code this name is only a handle for
+// hipGetSymbolAddress: the device address it yields (one per GPU) is what kernels get.
+static __device__ __align__(256) unsigned char yk_static_scratch[YK_ARGMAX_STATIC_MAX_ROWS * ARGMAX_CHUNKS * (sizeof(float) + sizeof(int32_t))];
+
+constexpr int YK_MAX_DEVICES = 64;
+static void* yk_static_scratch_ptr[YK_MAX_DEVICES];  // per device, null until looked up
+static std::mutex yk_static_scratch_lock;
+
+// The current device's copy of the array, looked up at the first call on that device.
+static void* static_scratch_of_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= YK_MAX_DEVICES) {
+    yk_fail("argmax_static: cannot tell the current device");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(yk_static_scratch_lock);
+  if (!yk_static_scratch_ptr[dev]) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(yk_static_scratch));
+    if (e != hipSuccess || !p) {
+      yk_fail(std::string("argmax_static: hipGetSymbolAddress failed: ") + hipGetErrorString(e));
+      return nullptr;
+    }
+    yk_static_scratch_ptr[dev] = p;
+  }
+  return yk_static_scratch_ptr[dev];
+}
+
+extern "C" int yk_argmax_static_setup(void) { return static_scratch_of_current_device() ? 0 : -1; }
+
+extern "C" int yk_argmax_static(const float* logits, int32_t* out, int n_rows, int vocab, hipStream_t stream) {
+  YK_REQUIRE(n_rows >= 0 && vocab > 0, "argmax_static: bad sizes");
+  YK_REQUIRE(n_rows <= YK_ARGMAX_STATIC_MAX_ROWS,
+             "argmax_static: more rows than the static scratch holds (" + std::to_string(YK_ARGMAX_STATIC_MAX_ROWS) + ")");
+  if (n_rows == 0) return 0;
+  YK_REQUIRE(logits && out, "argmax_static: null argument");
+  void* scratch = static_scratch_of_current_device();
+  if (!scratch) return -1;
+  // every row goes through the two kernels (slices of a short row may be empty: they hold the
+  // "nothing" entry, which never wins), so that the scratch is what carries the result
+  float* pv = static_cast<float*>(scratch);
+  int32_t* pi = reinterpret_cast<int32_t*>(pv + static_cast<size_t>(n_rows) * ARGMAX_CHUNKS);
+  argmax_part_kernel<<<dim3(n_rows, ARGMAX_CHUNKS), 256, 0, stream>>>(logits, pv, pi, vocab);
+  if (yk_check_launch("argmax_part (static scratch)")) return -1;
+  argmax_final_kernel<<<n_rows, 64, 0, stream>>>(pv, pi, out);
+  return yk_check_launch("argmax_final (static scratch)");
 }
 
 // ------------------------------------------------------------------------- sampling

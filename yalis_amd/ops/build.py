@@ -32,7 +32,7 @@ KERNEL_LIBS = {
     "sampling": ["runtime.hip", "sampling.hip"],
     "probe": ["runtime.hip", "probe.hip"],
 }
-HEADERS = ["common.h"]
+HEADERS = ["common.h", "no_alloc.h"]
 
 HIPCC_FLAGS = [
     "-O3",
