@@ -480,6 +480,122 @@ def test_attention_splits_merged_by_the_product(ops, plan, h, g, d, page, monkey
     close(got, want, 2e-2, 2**-6)
 
 
+def _bits(t):
+    return t.contiguous().view(torch.int16)
+
+
+@pytest.mark.parametrize("plan", [None, (1, 1), (4, 1), (4, 3), (1, 4)])
+@pytest.mark.parametrize("slices", [1, 3])
+@pytest.mark.parametrize("h,g,d,rd,page,inter", [
+    (32, 8, 128, 128, 64, False), (6, 2, 128, 128, 64, False), (6, 3, 64, 32, 16, False), (8, 1, 64, 64, 128, True),
+    (32, 1, 128, 64, 32, False), (24, 8, 128, 128, 64, False), (4, 4, 64, 0, 64, False),
+])
+def test_attention_rotates_and_appends_in_its_launch(ops, plan, slices, h, g, d, rd, page, inter):
+    """A step of single tokens: rotary + append inside the attention launch give the bits of
+    rotary + append followed by attention, in the output and in the pages, whether the
+    projection comes as bfloat16 rows or as float32 K slices, however the keys are divided,
+    with the token's own key first, last or in the middle of a block of 64 (the slot it goes to
+    holds NaN before), in tiled and in plain pages; and both agree with the plain reference."""
+    from yalis_amd.ops.hip import RopeInLaunch, SplitSum
+
+    cached = [0, 1, 31, 32, 63, 64, 65, 700, 1500, 127, 190]
+    n = len(cached)
+    gen = torch.Generator().manual_seed(31)
+    n_pages = sum(-(-(c + 1) // page) for c in cached) + 3
+    order = torch.randperm(n_pages, generator=gen).tolist()
+    kc = torch.full((n_pages, g, page, d), float("nan"), dtype=torch.bfloat16)
+    vc = torch.full((n_pages, g, d, page), float("nan"), dtype=torch.bfloat16)
+    seqs, used = [], 0
+    for c in cached:
+        n_p = -(-(c + 1) // page)
+        table = np.array(order[used : used + n_p], dtype=np.int32)
+        used += n_p
+        k = torch.randn((c, g, d), generator=gen).to(torch.bfloat16)
+        v = torch.randn((c, g, d), generator=gen).to(torch.bfloat16)
+        for pos in range(c):
+            kc[table[pos // page], :, pos % page, :] = k[pos]
+            vc[table[pos // page], :, :, pos % page] = v[pos]
+        seqs.append(SeqSpan(tokens=[0], first_position=c, block_tables=[table], state_slot=0))
+    hb = build_host_batch(seqs, 1, page)
+    tpt, big = ops.attention_tokens_per_tile(h, g), ops.attention_long_span_tile(h, g)
+    arrays = named_arrays(hb, {"tiles": lambda b: attention_tiles(b, tpt, 1, big), "cols": lambda b: attention_token_columns(b, tpt, 1, big)})
+    dev = {k: torch.from_numpy(np.ascontiguousarray(v)).to(DEV) for k, v in arrays.items()}
+    ctx = types.SimpleNamespace(arrays=dev, max_ctx=hb.max_ctx, max_qlen=1)
+    cols = (h + 2 * g) * d
+    if slices == 1:
+        raw = (torch.randn((n, cols), generator=gen) * 1.2).to(torch.bfloat16).to(DEV)
+        give = lambda: raw.clone()
+        summed = raw.float().cpu()
+    else:
+        parts = (torch.randn((slices, n, cols), generator=gen) * 0.7).to(DEV)
+        give = lambda: SplitSum(parts.clone(), torch.bfloat16)
+        summed = (parts[0] + parts[1] + parts[2]).to(torch.bfloat16).float().cpu()
+    cos, sin = _tables(rd, 1600) if rd else (None, None)
+    scale = 1.0 / math.sqrt(d)
+    positions, slots = dev["positions"], dev["slots_g0"]
+    # rotary + append, then attention
+    kc_a, vc_a = device_cache(ops, kc.clone(), vc.clone())
+    q = ops.rope_append(give(), h, g, d, positions, cos, sin, rd, inter, kc_a, vc_a, slots, page)
+    out_a = ops.attention(q, h, g, d, kc_a, vc_a, page, scale, 0, ctx, 0, dev["tiles"], plan=plan)
+    # both in one launch
+    kc_b, vc_b = device_cache(ops, kc.clone(), vc.clone())
+    out_b = ops.attention(give(), h, g, d, kc_b, vc_b, page, scale, 0, ctx, 0, dev["tiles"], plan=plan,
+                          rope=RopeInLaunch(cos, sin, rd, inter, True))
+    assert torch.isfinite(out_b.float()).all()
+    assert torch.equal(_bits(out_a), _bits(out_b))
+    assert torch.equal(_bits(kc_a), _bits(kc_b)) and torch.equal(_bits(vc_a), _bits(vc_b))
+    # queries only, against pages that already hold the tokens' keys and values (a run entry
+    # that reads another entry's cache)
+    q_rows = give()
+    q_rows = SplitSum(q_rows.tensor[:, :, : h * d].contiguous(), torch.bfloat16) if slices > 1 else q_rows[:, : h * d].contiguous()
+    out_c = ops.attention(q_rows, h, g, d, kc_b, vc_b, page, scale, 0, ctx, 0, dev["tiles"], plan=plan,
+                          rope=RopeInLaunch(cos, sin, rd, inter, False))
+    assert torch.equal(_bits(out_a), _bits(out_c))
+    # the plain reference
+    qkv_r = summed.clone()
+    kc_r, vc_r = kc.float(), vc.float()
+    cpu = {k: torch.from_numpy(np.ascontiguousarray(v)) for k, v in arrays.items()}
+    R.rope_append(qkv_r, h, g, d, cpu["positions"], None if cos is None else cos.cpu(), None if sin is None else sin.cpu(), rd, inter, kc_r, vc_r, cpu["slots_g0"], page)
+    kc_r, vc_r = kc_r.to(torch.bfloat16).float(), vc_r.to(torch.bfloat16).float()
+    q_r = qkv_r.view(n, -1, d)[:, :h].reshape(n, h * d).to(torch.bfloat16).float()
+    want = R.attention(q_r, h, g, d, kc_r, vc_r, page, scale, 0, types.SimpleNamespace(arrays=cpu), 0, None)
+    close(out_b, want, 2e-2, 2**-6)
+
+
+def test_attention_with_rotary_inside_leaves_splits_for_the_product(ops):
+    """One or two tokens whose keys are split across workgroups: the launch with rotary inside
+    leaves its splits unmerged too, and merged they are the two-kernel path's output."""
+    from yalis_amd.ops.hip import RopeInLaunch, SplitAttention
+
+    h, g, d, page = 32, 8, 128, 64
+    gen = torch.Generator().manual_seed(5)
+    cached = [1100, 300]
+    n_pages = 30
+    kc = torch.randn((n_pages, g, page, d), generator=gen).to(torch.bfloat16)
+    vc = torch.randn((n_pages, g, d, page), generator=gen).to(torch.bfloat16)
+    tables = [np.arange(0, 18, dtype=np.int32), np.arange(20, 25, dtype=np.int32)]
+    seqs = [SeqSpan(tokens=[0], first_position=c, block_tables=[t], state_slot=0) for c, t in zip(cached, tables)]
+    hb = build_host_batch(seqs, 1, page)
+    tpt, big = ops.attention_tokens_per_tile(h, g), ops.attention_long_span_tile(h, g)
+    arrays = named_arrays(hb, {"tiles": lambda b: attention_tiles(b, tpt, 1, big), "cols": lambda b: attention_token_columns(b, tpt, 1, big)})
+    dev = {k: torch.from_numpy(np.ascontiguousarray(v)).to(DEV) for k, v in arrays.items()}
+    ctx = types.SimpleNamespace(arrays=dev, max_ctx=hb.max_ctx, max_qlen=1)
+    raw = torch.randn((2, (h + 2 * g) * d), generator=gen).to(torch.bfloat16).to(DEV)
+    cos, sin = _tables(d, 1200)
+    kc_a, vc_a = device_cache(ops, kc.clone(), vc.clone())
+    q = ops.rope_append(raw.clone(), h, g, d, dev["positions"], cos, sin, d, False, kc_a, vc_a, dev["slots_g0"], page)
+    out_a = ops.attention(q, h, g, d, kc_a, vc_a, page, 0.09, 0, ctx, 0, dev["tiles"], plan=(4, 4))
+    kc_b, vc_b = device_cache(ops, kc.clone(), vc.clone())
+    got = ops.attention(raw.clone(), h, g, d, kc_b, vc_b, page, 0.09, 0, ctx, 0, dev["tiles"], plan=(4, 4), token_cols=dev["cols"],
+                        rope=RopeInLaunch(cos, sin, d, False, True))
+    assert isinstance(got, SplitAttention)
+    assert torch.equal(_bits(got.merge()), _bits(out_a)) and torch.equal(_bits(kc_a), _bits(kc_b)) and torch.equal(_bits(vc_a), _bits(vc_b))
+    # refused for steps that hold more than single tokens
+    ctx.max_qlen = 2
+    with pytest.raises(Exception, match="single tokens"):
+        ops.attention(raw.clone(), h, g, d, kc_b, vc_b, page, 0.09, 0, ctx, 0, dev["tiles"], rope=RopeInLaunch(cos, sin, d, False, True))
+
+
 @pytest.mark.parametrize("col_tiles", [1, 2])
 @pytest.mark.parametrize("splits", [1, 2, 5, 16])
 @pytest.mark.parametrize("h,g,d,page", [(8, 2, 128, 64), (6, 3, 64, 16), (32, 1, 128, 32), (6, 2, 64, 128)])

@@ -169,18 +169,61 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // 64 keys lies in one page, its page is looked up once, and every load instruction reads
 // 1 KiB of consecutive memory instead of 16 rows x 64 bytes (measured at 64 requests of 1,024
 // tokens: 46 us a layer against 58).
-template <int D, int W, bool TILED>
+//
+// ROPE: the launch also does what rotary + append would have done before it, for steps whose
+// tiles hold one token each (single decoded tokens).  The queries are then not read from `q`
+// but made from the projection's raw output rows [query heads | key heads | value heads]
+// (bfloat16, or the unreduced float32 K slices of the product): every workgroup sums the
+// slices of its heads, rotates them by the token's angle and parks them in LDS in bfloat16,
+// with the arithmetic and roundings of rope_append_kernel, so the bits are those of the
+// two-kernel path.  The token's own key and value are not in the pages yet: the one workgroup
+// (per kv head and split) whose share of the keys holds the token's position makes them too,
+// puts them into its operand registers in place of what the pages gave, and (chunk 0 only)
+// stores them in the pages for later steps.  Nobody reads that slot of the pages as a number
+// in this launch.
+struct RopeSrc {
+  const void* src;      // [tokens][src_stride] rows, n_splits slices split_stride elements apart
+  int src_f32;          // 1: float32 (slices are summed, the sum rounded when round_sum), 0: bfloat16
+  int n_splits;
+  size_t split_stride;
+  int round_sum;
+  int src_stride;
+  const float* cos_t;   // [max_positions][rotary_dim / 2] (null when rotary_dim == 0)
+  const float* sin_t;
+  int rotary_dim, interleaved, max_positions;
+  int append;           // 1: src holds the token's key and value heads too; they go to the pages
+  bf16_t* k_write;      // the same pages as k_cache / v_cache, writable
+  bf16_t* v_write;
+};
+
+__device__ __forceinline__ float rope_src_value(const RopeSrc& rs, size_t row, int idx) {
+  if (!rs.src_f32) return bf16_to_f32(static_cast<const bf16_t*>(rs.src)[row + idx]);
+  const float* p = static_cast<const float*>(rs.src) + row + idx;
+  float a = 0.f;
+  for (int s0 = 0; s0 < rs.n_splits; s0 += 8) {  // up to eight slices in flight; added in order
+    float d[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) d[j] = p[static_cast<size_t>(min(s0 + j, rs.n_splits - 1)) * rs.split_stride];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (s0 + j < rs.n_splits) a += d[j];
+  }
+  return as_output(a, rs.round_sum);
+}
+
+template <int D, int W, bool TILED, bool ROPE>
 __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ block_table, int table_width,
     int page_size, int n_heads, int n_kv, int hpt, int chunks, float scale_log2, int window,
-    int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml) {
+    int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml, RopeSrc rs) {
   constexpr int KS = D / 32;  // matrix-core steps over the head dimension
   constexpr int DT = D / 16;  // output tiles over the head dimension
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, gq = lane / 16;
   const int t = blockIdx.x;
-  const int seq = tiles[4 * t], tok0 = tiles[4 * t + 1], ntok = tiles[4 * t + 2], pos0 = tiles[4 * t + 3];
+  const int seq = tiles[4 * t], tok0 = tiles[4 * t + 1], pos0 = tiles[4 * t + 3];
+  const int ntok = ROPE ? 1 : tiles[4 * t + 2];
   const int g = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
   const int qpk = n_heads / n_kv;
   const int h_base = g * qpk + chunk * hpt;
@@ -211,7 +254,54 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
 
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
   AFrag8 qf[KS];
-  {
+  // ROPE: the block of 64 keys that holds the token's own position, and whether this workgroup
+  // is the one that makes the token's key and value (its share of the keys holds that block)
+  const int kb_new = pos0 / 64;
+  const bool makes_kv = ROPE && rs.append && kb_new >= wg_lo && kb_new < wg_hi;
+  __shared__ __attribute__((aligned(16))) bf16_t q_s[ROPE ? 16 : 1][ROPE ? D : 8];
+  __shared__ __attribute__((aligned(16))) bf16_t kv_s[2][ROPE ? D : 8];  // the token's key, its value
+  if (ROPE) {
+    const int pos = min(max(pos0, 0), rs.max_positions - 1);
+    const int half = rs.rotary_dim / 2;
+    const size_t row = static_cast<size_t>(tok0) * rs.src_stride;
+    const float* cs = rs.cos_t ? rs.cos_t + static_cast<size_t>(pos) * half : nullptr;
+    const float* sn = rs.sin_t ? rs.sin_t + static_cast<size_t>(pos) * half : nullptr;
+    // D / 2 items a head: a rotated pair, or two neighbours beyond the rotated part
+    const int heads_rot = heads_here + (makes_kv ? 1 : 0);
+    for (int item = threadIdx.x; item < heads_rot * (D / 2); item += 64 * W) {
+      const int hq = item / (D / 2), i = item % (D / 2);
+      const bool is_k = hq == heads_here;
+      const int base = (is_k ? n_heads + g : h_base + hq) * D;
+      bf16_t* dst = is_k ? kv_s[0] : q_s[hq];
+      if (i < half) {
+        const int ia = rs.interleaved ? 2 * i : i;
+        const int ib = rs.interleaved ? 2 * i + 1 : i + half;
+        const float a = rope_src_value(rs, row, base + ia), b = rope_src_value(rs, row, base + ib);
+        const float c = cs[i], sv = sn[i];
+        dst[ia] = f32_to_bf16(rot_first(a, b, c, sv));
+        dst[ib] = f32_to_bf16(rot_second(a, b, c, sv));
+      } else {
+        const int d = rs.rotary_dim + 2 * (i - half);
+        dst[d] = f32_to_bf16(rope_src_value(rs, row, base + d));
+        dst[d + 1] = f32_to_bf16(rope_src_value(rs, row, base + d + 1));
+      }
+    }
+    if (makes_kv)
+      for (int d = threadIdx.x; d < D; d += 64 * W) kv_s[1][d] = f32_to_bf16(rope_src_value(rs, row, (n_heads + n_kv + g) * D + d));
+    __syncthreads();
+    if (makes_kv && chunk == 0) {
+      // into the pages, for the steps that follow
+      const int slot = pos0 % page_size;
+      const size_t slab = (static_cast<size_t>(max(0, bt[min(pos0 / page_size, table_width - 1)])) * n_kv + g) * page_size * D;
+      for (int d = threadIdx.x; d < D; d += 64 * W) {
+        rs.k_write[slab + cache_k_offset(TILED, page_size, D, slot, d)] = kv_s[0][d];
+        rs.v_write[slab + cache_v_offset(TILED, page_size, D, slot, d)] = kv_s[1][d];
+      }
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      qf[ks].u = col_ok ? *reinterpret_cast<const u32x4_t*>(&q_s[hh][32 * ks + 8 * gq]) : zero4;
+  } else {
     const bf16_t* qp = q + static_cast<size_t>(tok0 + (col_ok ? tt : 0)) * q_stride +
                        static_cast<size_t>(h_base + (col_ok ? hh : 0)) * D + 8 * gq;
 #pragma unroll
@@ -220,6 +310,10 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
       if (!col_ok) qf[ks].u = zero4;
     }
   }
+  // where the token's own key sits among a block's score rows and value pieces
+  const int new_j = pos0 % 64, new_u = new_j / 32;
+  const int new_sb = (new_j % 8) / 4, new_r = 4 * ((new_j % 32) / 8) + new_j % 4;  // key row of the score products
+  const int new_gq = (new_j % 32) / 8, new_e = new_j % 8;                          // value piece and place in it
   float m = -INFINITY, l = 0.f;
   f32x4_t acc[DT];
 #pragma unroll
@@ -264,7 +358,20 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
   }                                                                                                \
   }
 
-  if (my_lo < my_hi) ATT_LOAD_K(my_lo)
+  // ROPE: the token's own key replaces what the pages gave for its slot
+#define ATT_PUT_NEW_K(KB)                                                                          \
+  if (ROPE && makes_kv && (KB) == kb_new && r == new_r) {                                          \
+    _Pragma("unroll") for (int u = 0; u < 2; ++u)                                                  \
+    _Pragma("unroll") for (int sb = 0; sb < 2; ++sb)                                               \
+      if (u == new_u && sb == new_sb && mine((KB), u)) {                                           \
+        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                          \
+            kf[u][sb][ks].u = *reinterpret_cast<const u32x4_t*>(&kv_s[0][32 * ks + 8 * gq]);       \
+      }                                                                                            \
+  }
+  if (my_lo < my_hi) {
+    ATT_LOAD_K(my_lo)
+    ATT_PUT_NEW_K(my_lo)
+  }
   for (int kb = my_lo; kb < my_hi; ++kb) {
     // values of this block: lane (r, gq) holds 8 consecutive keys of value row 16*dt + r
     AFrag8 vf[2][DT];
@@ -310,7 +417,10 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
         for (int ks = 0; ks < KS; ++ks)
           s[u][sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][sb][ks].v, qf[ks].v, s[u][sb], 0, 0, 0);
       }
-    if (kb + 1 < my_hi) ATT_LOAD_K(kb + 1)
+    if (kb + 1 < my_hi) {
+      ATT_LOAD_K(kb + 1)
+      ATT_PUT_NEW_K(kb + 1)
+    }
     float tmax = -INFINITY;
     // a block that every column sees whole needs no mask (columns that stand for nothing
     // compute on zeros and are never stored)
@@ -369,6 +479,22 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
             if (key + e >= hi) vf[u][dt].h[e] = 0;
       }
     }
+    if (ROPE && makes_kv && kb == kb_new && gq == new_gq) {
+      // the token's own value: element new_e of this lane's piece of every value row, put in
+      // with word masks (an index into the registers would not stay in registers)
+      const uint32_t keep = new_e % 2 ? 0x0000ffffu : 0xffff0000u;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+        if (u == new_u && (u == 0 ? mine0 : mine1)) {
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) {
+            const uint32_t v = static_cast<uint32_t>(kv_s[1][16 * dt + r]) << (new_e % 2 ? 16 : 0);
+#pragma unroll
+            for (int wd = 0; wd < 4; ++wd)
+              if (wd == new_e / 2) vf[u][dt].u[wd] = (vf[u][dt].u[wd] & keep) | v;
+          }
+        }
+    }
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -376,6 +502,7 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
         acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[u][dt].v, pf[u].v, acc[dt], 0, 0, 0);
   }
 #undef ATT_LOAD_K
+#undef ATT_PUT_NEW_K
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
 
@@ -838,17 +965,17 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
 // Short spans (single tokens, short portions): tiles of up to yk_attn_tokens_per_tile tokens.
 // leave_splits != 0 with n_splits > 1: the splits stay unmerged in the workspace (`out` is not
 // written) for a consumer that merges them itself or for yk_attn_combine.
-extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* k_cache,
-                            const void* v_cache, const int32_t* tiles, int n_tiles,
-                            const int32_t* block_table, int table_width, int page_size,
-                            int head_dim, int n_heads, int n_kv, float scale, int window,
+// rope: null, or where the launch makes its queries (and the tokens' keys and values) from.
+static int launch_attn_mfma(const void* q, int q_stride, void* out, const void* k_cache, const void* v_cache,
+                            const int32_t* tiles, int n_tiles, const int32_t* block_table, int table_width,
+                            int page_size, int head_dim, int n_heads, int n_kv, float scale, int window,
                             int n_waves, int n_splits, float* workspace, size_t workspace_floats,
-                            int leave_splits, hipStream_t stream) {
+                            int leave_splits, const RopeSrc* rope, hipStream_t stream) {
   YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_mfma: bad head counts");
   YK_REQUIRE(n_waves == 1 || n_waves == 4, "attn_mfma: a workgroup has 1 or 4 waves");
   YK_REQUIRE(yk_attn_mfma_supported(head_dim), "attn_mfma: head_dim must be 64 or 128");
   YK_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_mfma: page_size must be a multiple of 16");
-  YK_REQUIRE(q_stride % 8 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0,
+  YK_REQUIRE(rope || (q_stride % 8 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0),
              "attn_mfma: query rows must be 16-byte aligned");
   YK_REQUIRE(reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0,
              "attn_mfma: cache must be 16-byte aligned");
@@ -866,18 +993,21 @@ extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* 
   const float scale_log2 = scale * 1.4426950408889634f;
   dim3 grid(n_tiles, n_kv * chunks, n_splits), block(64 * n_waves);
   const bool tiled = cache_is_tiled(YK_BF16, head_dim, page_size);
+  const RopeSrc rs = rope ? *rope : RopeSrc{};
 #define YK_ARGS                                                                                    \
       static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out),                          \
       static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), tiles, block_table, \
-      table_width, page_size, n_heads, n_kv, hpt, chunks, scale_log2, window, n_splits, ws_o, ws_ml
-#define YK_LAUNCH(DD)                                                                              \
+      table_width, page_size, n_heads, n_kv, hpt, chunks, scale_log2, window, n_splits, ws_o, ws_ml, rs
+#define YK_LAUNCH_R(DD, RR)                                                                        \
   if (tiled) {                                                                                     \
-    if (n_waves == 1) attn_mfma_kernel<DD, 1, true><<<grid, block, 0, stream>>>(YK_ARGS);          \
-    else attn_mfma_kernel<DD, 4, true><<<grid, block, 0, stream>>>(YK_ARGS);                       \
+    if (n_waves == 1) attn_mfma_kernel<DD, 1, true, RR><<<grid, block, 0, stream>>>(YK_ARGS);      \
+    else attn_mfma_kernel<DD, 4, true, RR><<<grid, block, 0, stream>>>(YK_ARGS);                   \
   } else {                                                                                         \
-    if (n_waves == 1) attn_mfma_kernel<DD, 1, false><<<grid, block, 0, stream>>>(YK_ARGS);         \
-    else attn_mfma_kernel<DD, 4, false><<<grid, block, 0, stream>>>(YK_ARGS);                      \
-  }                                                                                                \
+    if (n_waves == 1) attn_mfma_kernel<DD, 1, false, RR><<<grid, block, 0, stream>>>(YK_ARGS);     \
+    else attn_mfma_kernel<DD, 4, false, RR><<<grid, block, 0, stream>>>(YK_ARGS);                  \
+  }
+#define YK_LAUNCH(DD)                                                                              \
+  if (rope) { YK_LAUNCH_R(DD, true) } else { YK_LAUNCH_R(DD, false) }                              \
   if (yk_check_launch("attn_mfma")) return -1;                                                     \
   if (n_splits > 1 && !leave_splits) {                                                             \
     attn_combine_kernel<DD><<<dim3(n_tiles, n_kv * chunks), 256, 0, stream>>>(                     \
@@ -890,8 +1020,63 @@ extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* 
     YK_LAUNCH(128)
   }
 #undef YK_LAUNCH
+#undef YK_LAUNCH_R
 #undef YK_ARGS
   return 0;
+}
+
+extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* k_cache,
+                            const void* v_cache, const int32_t* tiles, int n_tiles,
+                            const int32_t* block_table, int table_width, int page_size,
+                            int head_dim, int n_heads, int n_kv, float scale, int window,
+                            int n_waves, int n_splits, float* workspace, size_t workspace_floats,
+                            int leave_splits, hipStream_t stream) {
+  return launch_attn_mfma(q, q_stride, out, k_cache, v_cache, tiles, n_tiles, block_table, table_width, page_size,
+                          head_dim, n_heads, n_kv, scale, window, n_waves, n_splits, workspace, workspace_floats,
+                          leave_splits, nullptr, stream);
+}
+
+// yk_attn_mfma for a step of single tokens (every tile holds ONE token), with rotary + append
+// inside the launch: `src` holds the projection's output rows [n_heads query heads | n_kv key
+// heads | n_kv value heads] (src_dtype bfloat16 with n_src_splits == 1, or float32 with the
+// product's unreduced K slices [n_src_splits][tokens][src_stride], whose sum is rounded to
+// bfloat16 when round_sum).  The queries are rotated as yk_rope_append rotates them; with
+// append != 0 the tokens' rotated keys and their values are used by the launch and stored in
+// the pages (k_cache, v_cache are written), with append == 0 the rows hold queries only and
+// the pages already have the tokens' keys and values.
+extern "C" int yk_attn_mfma_rope(const void* src, int src_dtype, int n_src_splits, int round_sum, int src_stride,
+                                 int n_tokens, const float* cos_t, const float* sin_t, int rotary_dim,
+                                 int interleaved, int max_positions, int append, void* out, void* k_cache,
+                                 void* v_cache, const int32_t* tiles, int n_tiles, const int32_t* block_table,
+                                 int table_width, int page_size, int head_dim, int n_heads, int n_kv, float scale,
+                                 int window, int n_waves, int n_splits, float* workspace, size_t workspace_floats,
+                                 int leave_splits, hipStream_t stream) {
+  YK_REQUIRE(src && (src_dtype == YK_F32 || src_dtype == YK_BF16), "attn_mfma_rope: the rows must be float32 or bfloat16");
+  YK_REQUIRE(n_src_splits >= 1 && (n_src_splits == 1 || src_dtype == YK_F32), "attn_mfma_rope: unreduced slices must be float32");
+  YK_REQUIRE(n_tokens >= n_tiles && n_tiles >= 0, "attn_mfma_rope: one tile a token");
+  YK_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0,
+             "attn_mfma_rope: rotary_dim must be even and at most head_dim");
+  YK_REQUIRE(rotary_dim == 0 || (cos_t && sin_t && max_positions > 0), "attn_mfma_rope: missing table");
+  YK_REQUIRE(n_heads > 0 && n_kv > 0 && src_stride >= (n_heads + (append ? 2 * n_kv : 0)) * head_dim,
+             "attn_mfma_rope: row stride too small");
+  RopeSrc rs;
+  rs.src = src;
+  rs.src_f32 = src_dtype == YK_F32;
+  rs.n_splits = n_src_splits;
+  rs.split_stride = static_cast<size_t>(n_tokens) * src_stride;
+  rs.round_sum = round_sum;
+  rs.src_stride = src_stride;
+  rs.cos_t = rotary_dim ? cos_t : nullptr;
+  rs.sin_t = rotary_dim ? sin_t : nullptr;
+  rs.rotary_dim = rotary_dim;
+  rs.interleaved = interleaved;
+  rs.max_positions = rotary_dim ? max_positions : 1;
+  rs.append = append != 0;
+  rs.k_write = static_cast<bf16_t*>(k_cache);
+  rs.v_write = static_cast<bf16_t*>(v_cache);
+  return launch_attn_mfma(nullptr, 0, out, k_cache, v_cache, tiles, n_tiles, block_table, table_width, page_size,
+                          head_dim, n_heads, n_kv, scale, window, n_waves, n_splits, workspace, workspace_floats,
+                          leave_splits, &rs, stream);
 }
 
 // The second half of yk_attn_mfma for a launch that was told to leave its splits in the

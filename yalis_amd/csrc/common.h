@@ -121,6 +121,12 @@ __device__ __forceinline__ float as_output(float v, int round_sum) {
   return round_sum ? to_f32<bf16_t>(from_f32<bf16_t>(v)) : v;
 }
 
+// Rotation of a pair (a, b) by the angle with cosine c and sine s: a' = a c - b s, b' = b c + a s.
+// One rounding of b*s (or a*s), then a fused multiply-add: written out so that every kernel
+// that rotates (rotary + append on its own, or inside the attention launch) gives the same bits.
+__device__ __forceinline__ float rot_first(float a, float b, float c, float s) { return fmaf(a, c, -__fmul_rn(b, s)); }
+__device__ __forceinline__ float rot_second(float a, float b, float c, float s) { return fmaf(b, c, __fmul_rn(a, s)); }
+
 // ------------------------------------------------ attention whose keys were split across workgroups
 // Heads of one kv head that share a wave of the matrix-core attention (its 16 columns hold
 // 16 / heads_per_tile tokens of those heads); a kv group with more heads takes several

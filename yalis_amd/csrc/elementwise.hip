@@ -312,10 +312,7 @@ extern "C" int yk_add_rmsnorm(float* residual, const void* delta, int delta_dtyp
 // (position, pair index i): a' = a cos - b sin, b' = b cos + a sin; pairs are
 // (i, i + rotary_dim/2) ("half") or (2i, 2i + 1) ("interleaved"); elements beyond
 // rotary_dim pass unchanged.
-// one rounding of b*s (or a*s), then a fused multiply-add: written out so that every kernel
-// that rotates gives the same bits
-__device__ __forceinline__ float rot_first(float a, float b, float c, float s) { return fmaf(a, c, -__fmul_rn(b, s)); }
-__device__ __forceinline__ float rot_second(float a, float b, float c, float s) { return fmaf(b, c, __fmul_rn(a, s)); }
+// (rot_first, rot_second: common.h)
 
 template <typename TS, typename T>
 __global__ void rope_append_kernel(const TS* src, int n_splits, size_t split_stride, int round_sum,

@@ -80,6 +80,11 @@ _SIGNATURES = {
         [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _c_int, _vp],
         _c_int,
     ),
+    "yk_attn_mfma_rope": (
+        [_vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _c_int,
+         _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _c_int, _vp],
+        _c_int,
+    ),
     "yk_attn_combine": ([_vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_size_t, _vp], _c_int),
     "yk_gemm_skinny_from_attention_ok": ([_c_int, _c_int, _c_int], _c_int),
     "yk_gemm_mfma_skinny_from_attention": (
@@ -101,7 +106,7 @@ _LATER_SIGNATURES = {
         "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
     },
 }
-_ABI = 9
+_ABI = 10
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
 # above it the vendor library does.
@@ -170,6 +175,16 @@ class SplitAttention:
             )
         )
         return out
+
+
+class RopeInLaunch:
+    """What ``HipOps.attention`` needs to rotate and append inside its own launch: the float32
+    tables [positions, rotary_dim / 2] (None with rotary_dim 0), how pairs are formed, and
+    whether the projection's rows hold keys and values to append (False: queries only, the
+    pages already hold this step's keys and values)."""
+
+    def __init__(self, cos, sin, rotary_dim: int, interleaved: bool, append: bool):
+        self.cos, self.sin, self.rotary_dim, self.interleaved, self.append = cos, sin, int(rotary_dim), bool(interleaved), bool(append)
 
 
 class HipOps:
@@ -535,9 +550,14 @@ class HipOps:
             return 1
         return max(1, min(-(-768 // workgroups), key_blocks // 8, 16))
 
+    def attention_can_rotate(self, act_dtype: torch.dtype, head_dim: int) -> bool:
+        """Whether ``attention`` takes ``rope=`` for such a mixer: the matrix-core kernel for
+        short spans can rotate queries and append keys and values itself."""
+        return act_dtype == torch.bfloat16 and bool(self._ask("yk_attn_mfma_supported", head_dim))
+
     def attention(self, qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size,
                   scale, window, ctx, group, tiles, long_tiles=None, plan=None, long_plan=None,
-                  long_col_tiles: int = 1, token_cols=None):
+                  long_col_tiles: int = 1, token_cols=None, rope: Optional["RopeInLaunch"] = None):
         """Queries are the first n_heads heads of each row of ``qkv`` (whatever follows
         them in the row is skipped); keys and values come from the cache through the
         block table of ``group``.  ``long_tiles`` hold up to
@@ -545,7 +565,16 @@ class HipOps:
         overrides ``attention_plan`` and ``long_plan`` ``attention_long_splits`` (tests,
         measurements).  With ``token_cols`` (``attention_token_columns`` of the same short
         tiles) the caller takes a ``SplitAttention`` as well: what a step of up to 16 tokens,
-        none of them in a long tile, leaves when its keys were split across workgroups."""
+        none of them in a long tile, leaves when its keys were split across workgroups.
+
+        ``rope`` (only where ``attention_can_rotate``, and only for steps whose spans are single
+        tokens): ``qkv`` is then the projection's raw output (a tensor or a ``SplitSum``) and
+        the launch does what ``rope_append`` would have done before it: it rotates the queries
+        and, with ``rope.append``, rotates the tokens' keys, uses them and their values, and
+        stores both in the pages."""
+        if rope is not None:
+            return self._attention_rope(qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size, scale, window,
+                                        ctx, group, tiles, plan, token_cols, rope)
         self._rows(qkv, "qkv")
         n = qkv.shape[0]
         bt = ctx.arrays[f"block_table_g{group}"]
@@ -606,6 +635,54 @@ class HipOps:
                     self._stream(),
                 )
             )
+        return out
+
+    def _attention_rope(self, qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size, scale, window,
+                        ctx, group, tiles, plan, token_cols, rope: "RopeInLaunch"):
+        n_splits_src, round_sum, src = 1, 0, qkv
+        if isinstance(qkv, SplitSum):
+            n_splits_src, round_sum, src = qkv.n_splits, qkv.round_sum, qkv.tensor
+            n, cols = qkv.shape
+            src_stride = cols
+        else:
+            self._rows(qkv, "qkv")
+            n, cols = qkv.shape
+            src_stride = qkv.stride(0)
+        if ctx.max_qlen != 1 or tiles.shape[0] != n:
+            raise KernelError("attention with rotary inside takes steps of single tokens only")
+        if not self.attention_can_rotate(k_cache.dtype, head_dim):
+            raise KernelError("attention with rotary inside needs bfloat16 pages and a head size of 64 or 128")
+        if cols != (n_heads + (2 * n_kv if rope.append else 0)) * head_dim:
+            raise KernelError(f"projection rows have {cols} elements, expected {(n_heads + (2 * n_kv if rope.append else 0)) * head_dim}")
+        if tuple(k_cache.shape[1:]) != (n_kv, page_size, head_dim) or tuple(v_cache.shape[1:]) != (n_kv, head_dim, page_size):
+            raise KernelError(f"cache pages have shapes {tuple(k_cache.shape)}, {tuple(v_cache.shape)}")
+        max_pos = 0
+        if rope.rotary_dim:
+            cos, sin = rope.cos, rope.sin
+            if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.shape != sin.shape or cos.shape[1] != rope.rotary_dim // 2:
+                raise KernelError("rotary tables must be float32 [positions, rotary_dim/2]")
+            max_pos = cos.shape[0]
+        bt = ctx.arrays[f"block_table_g{group}"]
+        out = torch.empty((n, n_heads * head_dim), dtype=torch.bfloat16, device=src.device)
+        hpt = self._ask("yk_attn_heads_per_tile", n_heads, n_kv)
+        chunks = -(-(n_heads // n_kv) // hpt)
+        key_blocks = max(1, -(-ctx.max_ctx // 64))
+        waves, splits = plan or self.attention_plan(n * n_kv * chunks, key_blocks)
+        ws_floats = self._ask("yk_attn_mfma_workspace", n, n_heads, n_kv, head_dim, splits)
+        ws = self._ws(ws_floats) if ws_floats else None
+        leave = bool(token_cols is not None and splits > 1 and n <= MERGE_IN_PRODUCT_MAX_TOKENS)
+        self._check(
+            self.lib.yk_attn_mfma_rope(
+                src.data_ptr(), _code(src.dtype), n_splits_src, round_sum, src_stride, n,
+                _ptr(rope.cos) if rope.rotary_dim else None, _ptr(rope.sin) if rope.rotary_dim else None,
+                int(rope.rotary_dim), int(bool(rope.interleaved)), max_pos, int(bool(rope.append)),
+                out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), tiles.data_ptr(), n, bt.data_ptr(), bt.shape[1],
+                page_size, head_dim, n_heads, n_kv, float(scale), int(window), waves, splits, _ptr(ws),
+                0 if ws is None else ws.numel(), int(leave), self._stream(),
+            )
+        )
+        if leave:
+            return SplitAttention(self, ws, tiles, token_cols, n, n_heads, n_kv, head_dim, splits)
         return out
 
     # ----------------------------------------------------------------- activation

@@ -55,8 +55,22 @@ class Attention(Mixer):
         # tokens or twice as many (`long_tiles_of`: the step's choice)
         self.long_tile = rt.ops.attention_long_span_tile(self.n_heads, self.n_kv)
         self.long_tile_2 = rt.ops.attention_long_span_tile(self.n_heads, self.n_kv, 2)
+        self.layout = f"h{self.n_heads}g{self.n_kv}"
         self.group = None
         self.w_qkv = self.w_q = self.w_o = None
+        # whether the kernel library's attention can rotate and append inside its own launch
+        # for steps of single tokens (one kernel fewer per layer), and what it needs for that
+        can = getattr(rt.ops, "attention_can_rotate", None)
+        self.rotates_in_launch = bool(can is not None and can(rt.act_dtype, self.head_dim))
+        if self.rotates_in_launch:
+            from ..ops.hip import RopeInLaunch
+
+            p = self.position
+            self.rope_in_launch = {
+                append: RopeInLaunch(None if p is None else p.cos, None if p is None else p.sin,
+                                     0 if p is None else p.rotary_dim, False if p is None else p.interleaved, append)
+                for append in (False, True)
+            }
 
     # ---- what it needs
     def tensor_specs(self) -> Dict[str, TensorSpec]:
@@ -103,12 +117,14 @@ class Attention(Mixer):
         tpt = self.tokens_per_tile
         big, big2 = self.long_tile, self.long_tile_2
         none = np.zeros((0, 4), dtype=np.int32)
+        # (the long tiles carry the head layout in their names: which of the two lists a step
+        # fills depends on it, and layers with another layout must not read this one's choice)
         return {
             f"attention_tiles_{tpt}_upto{big}": lambda hb: attention_tiles(hb, tpt, 1, big),
             f"attention_token_columns_{tpt}_upto{big}": lambda hb: attention_token_columns(hb, tpt, 1, big),
-            f"attention_long_tiles_{big}": lambda hb: attention_tiles(hb, big, big + 1, longest_first=True)
+            f"attention_long_tiles_{big}_{self.layout}": lambda hb: attention_tiles(hb, big, big + 1, longest_first=True)
             if self.long_col_tiles(hb) == 1 else none,
-            f"attention_long_tiles_{big2}": lambda hb: attention_tiles(hb, big2, big + 1, longest_first=True)
+            f"attention_long_tiles_{big2}_{self.layout}": lambda hb: attention_tiles(hb, big2, big + 1, longest_first=True)
             if self.long_col_tiles(hb) == 2 else none,
         }
 
@@ -124,10 +140,21 @@ class Attention(Mixer):
             qkv = ops.linear(h, self.w_q, self.rt.act_dtype, partial_ok=True)
             n_kv_rows = 0
         k_cache, v_cache = site.kv()
-        col_tiles = ctx.memo.get("attention_long_col_tiles")
+        memo_key = f"attention_long_col_tiles_{self.layout}"
+        col_tiles = ctx.memo.get(memo_key)
         if col_tiles is None:
-            col_tiles = ctx.memo["attention_long_col_tiles"] = self.long_col_tiles(ctx.host)
+            col_tiles = ctx.memo[memo_key] = self.long_col_tiles(ctx.host)
         pos = self.position
+        tiles = ctx.arrays[f"attention_tiles_{self.tokens_per_tile}_upto{self.long_tile}"]
+        token_cols = ctx.arrays[f"attention_token_columns_{self.tokens_per_tile}_upto{self.long_tile}"]
+        if ctx.max_qlen == 1 and self.rotates_in_launch:
+            # a step of single tokens: rotary + append happen inside the attention launch
+            out = ops.attention(
+                qkv, self.n_heads, self.n_kv, self.head_dim, k_cache, v_cache, self.rt.page_size, self.scale,
+                0 if self.window is None else int(self.window), ctx, site.group, tiles, token_cols=token_cols,
+                rope=self.rope_in_launch[bool(n_kv_rows)],
+            )
+            return ops.linear(out, self.w_o, self.rt.act_dtype, partial_ok=True)
         q = ops.rope_append(
             qkv,
             self.n_heads,
@@ -155,9 +182,9 @@ class Attention(Mixer):
             0 if self.window is None else int(self.window),
             ctx,
             site.group,
-            ctx.arrays[f"attention_tiles_{self.tokens_per_tile}_upto{self.long_tile}"],
-            ctx.arrays[f"attention_long_tiles_{self.long_tile_2 if col_tiles == 2 else self.long_tile}"],
+            tiles,
+            ctx.arrays[f"attention_long_tiles_{self.long_tile_2 if col_tiles == 2 else self.long_tile}_{self.layout}"],
             long_col_tiles=col_tiles,
-            token_cols=ctx.arrays[f"attention_token_columns_{self.tokens_per_tile}_upto{self.long_tile}"],
+            token_cols=token_cols,
         )
         return ops.linear(out, self.w_o, self.rt.act_dtype, partial_ok=True)
