@@ -83,6 +83,23 @@ def test_add_rmsnorm(ops, width, rows, act, wdtype):
                 close(got, want, 1e-3, 2**-8)
 
 
+@pytest.mark.parametrize("width", [192, 4096, 1001])
+@pytest.mark.parametrize("tdtype", [torch.float32, torch.bfloat16])
+def test_add_rmsnorm_starts_from_embedding_rows(ops, width, tdtype):
+    """The first norm gathers the embedding's rows itself: the residual it leaves and the
+    normed rows are those of the embedding kernel followed by the norm."""
+    table = rnd((515, width), tdtype, 70)
+    ids = torch.tensor([0, 514, 3, 3, 77, 200, 1], dtype=torch.int32, device=DEV)
+    w = rnd((width,), tdtype, 71) + 1
+    res_a = ops.embed(ids, table)
+    out_a = ops.add_rmsnorm(res_a, None, w, 1e-5, False, torch.bfloat16)
+    res_b, rows = ops.embedded_rows(ids, table)
+    res_b.fill_(float("nan"))  # never read
+    out_b = ops.add_rmsnorm(res_b, rows, w, 1e-5, False, torch.bfloat16)
+    assert torch.equal(res_a, res_b) and torch.equal(out_a, out_b)
+    assert torch.equal(rows.gather(), res_a)
+
+
 def test_gather_add_rmsnorm(ops):
     res = rnd((20, 320), torch.float32, 1)
     delta = rnd((20, 320), torch.bfloat16, 2)

@@ -182,8 +182,8 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // stores them in the pages for later steps.  Nobody reads that slot of the pages as a number
 // in this launch.
 struct RopeSrc {
-  const void* src;      // [tokens][src_stride] rows, n_splits slices split_stride elements apart
-  int src_f32;          // 1: float32 (slices are summed, the sum rounded when round_sum), 0: bfloat16
+  const void* src;      // [tokens][src_stride] rows, n_splits slices split_stride elements apart:
+                        // float32 (slices are summed, the sum rounded when round_sum) or bfloat16
   int n_splits;
   size_t split_stride;
   int round_sum;
@@ -192,34 +192,46 @@ struct RopeSrc {
   const float* sin_t;
   int rotary_dim, interleaved, max_positions;
   int append;           // 1: src holds the token's key and value heads too; they go to the pages
-  bf16_t* k_write;      // the same pages as k_cache / v_cache, writable
-  bf16_t* v_write;
 };
 
-__device__ __forceinline__ float rope_src_value(const RopeSrc& rs, size_t row, int idx) {
-  if (!rs.src_f32) return bf16_to_f32(static_cast<const bf16_t*>(rs.src)[row + idx]);
-  const float* p = static_cast<const float*>(rs.src) + row + idx;
-  float a = 0.f;
-  for (int s0 = 0; s0 < rs.n_splits; s0 += 8) {  // up to eight slices in flight; added in order
-    float d[8];
+// Up to eight slices of one element, all asked for before any is used (a slice index beyond
+// the last is clamped and its value dropped, so that the loads carry no condition).
+// SRC 1: bfloat16 rows (one slice); SRC 2: float32 slices.
+template <int SRC>
+__device__ __forceinline__ void rope_src_load8(const void* src, size_t row, int idx, const size_t (&slice)[8], float (&d)[8]) {
+  if (SRC == 1) {
+    d[0] = bf16_to_f32(static_cast<const bf16_t*>(src)[row + idx]);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) d[j] = p[static_cast<size_t>(min(s0 + j, rs.n_splits - 1)) * rs.split_stride];
+    for (int j = 1; j < 8; ++j) d[j] = 0.f;
+  } else {
+    const float* p = static_cast<const float*>(src) + row + idx;
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
-      if (s0 + j < rs.n_splits) a += d[j];
+    for (int j = 0; j < 8; ++j) d[j] = p[slice[j]];
   }
-  return as_output(a, rs.round_sum);
+}
+// where the slices s0 .. s0 + 7 start (clamped to the last)
+__device__ __forceinline__ void rope_src_slices(int s0, int n_splits, size_t split_stride, size_t (&slice)[8]) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j) slice[j] = static_cast<size_t>(min(s0 + j, n_splits - 1)) * split_stride;
+}
+// added in the order of the slices, as every other consumer of a product's slices adds them
+__device__ __forceinline__ float rope_src_add8(float acc, const float (&d)[8], int s0, int n_splits) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    if (s0 + j < n_splits) acc += d[j];
+  return acc;
 }
 
-template <int D, int W, bool TILED, bool ROPE>
+template <int D, int W, bool TILED, int SRC>
 __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
-    const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const bf16_t* k_cache, const bf16_t* v_cache,  // (written too, with ROPE: the token's own slot)
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ block_table, int table_width,
     int page_size, int n_heads, int n_kv, int hpt, int chunks, float scale_log2, int window,
     int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml, RopeSrc rs) {
   constexpr int KS = D / 32;  // matrix-core steps over the head dimension
   constexpr int DT = D / 16;  // output tiles over the head dimension
+  constexpr bool ROPE = SRC != 0;  // SRC 0: queries from `q`; 1, 2: rotary + append in here (rope_src_load8)
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, gq = lane / 16;
   const int t = blockIdx.x;
   const int seq = tiles[4 * t], tok0 = tiles[4 * t + 1], pos0 = tiles[4 * t + 3];
@@ -253,67 +265,6 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
   const int last_page_col = min(table_width - 1, (hi - 1) / page_size);
 
   const u32x4_t zero4 = {0u, 0u, 0u, 0u};
-  AFrag8 qf[KS];
-  // ROPE: the block of 64 keys that holds the token's own position, and whether this workgroup
-  // is the one that makes the token's key and value (its share of the keys holds that block)
-  const int kb_new = pos0 / 64;
-  const bool makes_kv = ROPE && rs.append && kb_new >= wg_lo && kb_new < wg_hi;
-  __shared__ __attribute__((aligned(16))) bf16_t q_s[ROPE ? 16 : 1][ROPE ? D : 8];
-  __shared__ __attribute__((aligned(16))) bf16_t kv_s[2][ROPE ? D : 8];  // the token's key, its value
-  if (ROPE) {
-    const int pos = min(max(pos0, 0), rs.max_positions - 1);
-    const int half = rs.rotary_dim / 2;
-    const size_t row = static_cast<size_t>(tok0) * rs.src_stride;
-    const float* cs = rs.cos_t ? rs.cos_t + static_cast<size_t>(pos) * half : nullptr;
-    const float* sn = rs.sin_t ? rs.sin_t + static_cast<size_t>(pos) * half : nullptr;
-    // D / 2 items a head: a rotated pair, or two neighbours beyond the rotated part
-    const int heads_rot = heads_here + (makes_kv ? 1 : 0);
-    for (int item = threadIdx.x; item < heads_rot * (D / 2); item += 64 * W) {
-      const int hq = item / (D / 2), i = item % (D / 2);
-      const bool is_k = hq == heads_here;
-      const int base = (is_k ? n_heads + g : h_base + hq) * D;
-      bf16_t* dst = is_k ? kv_s[0] : q_s[hq];
-      if (i < half) {
-        const int ia = rs.interleaved ? 2 * i : i;
-        const int ib = rs.interleaved ? 2 * i + 1 : i + half;
-        const float a = rope_src_value(rs, row, base + ia), b = rope_src_value(rs, row, base + ib);
-        const float c = cs[i], sv = sn[i];
-        dst[ia] = f32_to_bf16(rot_first(a, b, c, sv));
-        dst[ib] = f32_to_bf16(rot_second(a, b, c, sv));
-      } else {
-        const int d = rs.rotary_dim + 2 * (i - half);
-        dst[d] = f32_to_bf16(rope_src_value(rs, row, base + d));
-        dst[d + 1] = f32_to_bf16(rope_src_value(rs, row, base + d + 1));
-      }
-    }
-    if (makes_kv)
-      for (int d = threadIdx.x; d < D; d += 64 * W) kv_s[1][d] = f32_to_bf16(rope_src_value(rs, row, (n_heads + n_kv + g) * D + d));
-    __syncthreads();
-    if (makes_kv && chunk == 0) {
-      // into the pages, for the steps that follow
-      const int slot = pos0 % page_size;
-      const size_t slab = (static_cast<size_t>(max(0, bt[min(pos0 / page_size, table_width - 1)])) * n_kv + g) * page_size * D;
-      for (int d = threadIdx.x; d < D; d += 64 * W) {
-        rs.k_write[slab + cache_k_offset(TILED, page_size, D, slot, d)] = kv_s[0][d];
-        rs.v_write[slab + cache_v_offset(TILED, page_size, D, slot, d)] = kv_s[1][d];
-      }
-    }
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      qf[ks].u = col_ok ? *reinterpret_cast<const u32x4_t*>(&q_s[hh][32 * ks + 8 * gq]) : zero4;
-  } else {
-    const bf16_t* qp = q + static_cast<size_t>(tok0 + (col_ok ? tt : 0)) * q_stride +
-                       static_cast<size_t>(h_base + (col_ok ? hh : 0)) * D + 8 * gq;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      qf[ks].u = *reinterpret_cast<const u32x4_t*>(qp + 32 * ks);
-      if (!col_ok) qf[ks].u = zero4;
-    }
-  }
-  // where the token's own key sits among a block's score rows and value pieces
-  const int new_j = pos0 % 64, new_u = new_j / 32;
-  const int new_sb = (new_j % 8) / 4, new_r = 4 * ((new_j % 32) / 8) + new_j % 4;  // key row of the score products
-  const int new_gq = (new_j % 32) / 8, new_e = new_j % 8;                          // value piece and place in it
   float m = -INFINITY, l = 0.f;
   f32x4_t acc[DT];
 #pragma unroll
@@ -325,11 +276,13 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
   auto page_of = [&](int key) { return max(0, bt[min(key / page_size, last_page_col)]); };
 
   AFrag8 kf[2][2][KS];
-#define ATT_LOAD_K(KB)                                                                            \
+#define ATT_LOAD_K(KB) ATT_LOAD_K_AT(KB, page_of((KB) * 64))
+  // PAGE0: the page of the block's first key, for tiled pages (looked up by the caller)
+#define ATT_LOAD_K_AT(KB, PAGE0)                                                                  \
   {                                                                                                \
   if (TILED) {                                                                                     \
     const int key0 = (KB) * 64;                                                                    \
-    const bf16_t* kp = k_cache + (static_cast<size_t>(page_of(key0)) * n_kv + g) * page_size * D + \
+    const bf16_t* kp = k_cache + (static_cast<size_t>(PAGE0) * n_kv + g) * page_size * D +         \
                        static_cast<size_t>(key0 % page_size) * D + 8 * lane;                       \
     _Pragma("unroll") for (int u = 0; u < 2; ++u) {                                                \
       if (mine((KB), u)) {                                                                         \
@@ -358,6 +311,36 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
   }                                                                                                \
   }
 
+  // values of a block: lane (r, gq) holds 8 consecutive keys of value row 16*dt + r
+  AFrag8 vf[2][DT];
+#define ATT_LOAD_V_AT(KB, PAGE0)                                                                   \
+  {                                                                                                \
+  if (TILED) {                                                                                     \
+    const int key0 = (KB) * 64;                                                                    \
+    const bf16_t* vp = v_cache + (static_cast<size_t>(PAGE0) * n_kv + g) * D * page_size +         \
+                       static_cast<size_t>(key0 % page_size) * D + 8 * lane;                       \
+    _Pragma("unroll") for (int u = 0; u < 2; ++u) {                                                \
+      if (mine((KB), u)) {                                                                         \
+        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt)                                          \
+            vf[u][dt].u = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(vp + (u * DT + dt) * 512)); \
+      } else {                                                                                     \
+        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) vf[u][dt].u = zero4;                     \
+      }                                                                                            \
+    }                                                                                              \
+  } else {                                                                                         \
+    _Pragma("unroll") for (int u = 0; u < 2; ++u) {                                                \
+      if (mine((KB), u)) {                                                                         \
+        const int key = (KB) * 64 + 32 * u + 8 * gq;                                               \
+        const bf16_t* vp = v_cache + (static_cast<size_t>(page_of(key)) * n_kv + g) * D * page_size + key % page_size; \
+        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt)                                          \
+            vf[u][dt].u = *reinterpret_cast<const u32x4_t*>(vp + static_cast<size_t>(16 * dt + r) * page_size); \
+      } else {                                                                                     \
+        _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) vf[u][dt].u = zero4;                     \
+      }                                                                                            \
+    }                                                                                              \
+  }                                                                                                \
+  }
+
   // ROPE: the token's own key replaces what the pages gave for its slot
 #define ATT_PUT_NEW_K(KB)                                                                          \
   if (ROPE && makes_kv && (KB) == kb_new && r == new_r) {                                          \
@@ -368,44 +351,133 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
             kf[u][sb][ks].u = *reinterpret_cast<const u32x4_t*>(&kv_s[0][32 * ks + 8 * gq]);       \
       }                                                                                            \
   }
+  AFrag8 qf[KS];
+  // ROPE: the block of 64 keys that holds the token's own position, and whether this workgroup
+  // is the one that makes the token's key and value (its share of the keys holds that block)
+  const int kb_new = pos0 / 64;
+  const bool makes_kv = ROPE && rs.append && kb_new >= wg_lo && kb_new < wg_hi;
+  __shared__ __attribute__((aligned(16))) bf16_t q_s[ROPE ? 16 : 1][ROPE ? D : 8];
+  __shared__ __attribute__((aligned(16))) bf16_t kv_s[2][ROPE ? D : 8];  // the token's key, its value
+  // ROPE: items of two elements: D / 2 a head (a rotated pair, or two neighbours beyond the
+  // rotated part) for the query heads, then, where this workgroup makes them, for the key head
+  // and (never rotated) the value head.  A thread takes two items a round, T apart (the second
+  // only where the workgroup has more items than threads), and asks for everything both need
+  // before it uses any of it: in most launches there is one round, and one wait for memory.
+  constexpr int T = 64 * W;
+  if (ROPE) {
+    const int items = (heads_here + (makes_kv ? 2 : 0)) * (D / 2);
+    const int half = rs.rotary_dim / 2;
+    const size_t row = static_cast<size_t>(tok0) * rs.src_stride;
+    const size_t at = static_cast<size_t>(min(max(pos0, 0), rs.max_positions - 1)) * half;
+    // (without a table the loads below read a valid word that is never used)
+    const float* cs = half > 0 ? rs.cos_t + at : reinterpret_cast<const float*>(tiles);
+    const float* sn = half > 0 ? rs.sin_t + at : reinterpret_cast<const float*>(tiles);
+    const int half_m1 = max(half - 1, 0);
+    const int src_splits = SRC == 2 ? rs.n_splits : 1;
+    const size_t src_split_stride = rs.split_stride;
+    // the page of the first block is asked for first: the keys' addresses wait for it, and a
+    // wait for an older load leaves the younger ones in flight
+    const int first_page = my_lo < my_hi ? page_of(my_lo * 64) : 0;
+    // one round; LOAD_K: the first block's keys are asked for while the round's rows are on
+    // their way (the first round is straight-line code: its loads are all issued before the
+    // first of them is waited for; rows of more than eight slices finish in a loop)
+    auto round = [&](int first, auto load_k) {
+      const bool two = first + T < items;  // the same for every thread
+      int ia[2], ib[2], base[2];
+      bf16_t* dst[2];
+      bool rot[2], ok[2];
+      float c[2], sv[2], acc_a[2], acc_b[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int item = first + j * T + static_cast<int>(threadIdx.x);
+        ok[j] = item < items;
+        const int it = ok[j] ? item : 0;
+        const int hq = it / (D / 2), i = it % (D / 2);
+        const bool is_k = hq == heads_here, is_v = hq == heads_here + 1;
+        base[j] = (is_v ? n_heads + n_kv + g : (is_k ? n_heads + g : h_base + hq)) * D;
+        dst[j] = is_v ? kv_s[1] : (is_k ? kv_s[0] : q_s[hq]);
+        rot[j] = !is_v && i < half;
+        ia[j] = rot[j] ? (rs.interleaved ? 2 * i : i) : (is_v ? 2 * i : rs.rotary_dim + 2 * (i - half));
+        ib[j] = rot[j] ? (rs.interleaved ? 2 * i + 1 : i + half) : ia[j] + 1;
+        c[j] = cs[min(i, half_m1)];  // (clamped: asked for whether the pair rotates or not)
+        sv[j] = sn[min(i, half_m1)];
+      }
+      float da0[8], db0[8], da1[8], db1[8];
+      size_t slice[8];
+      rope_src_slices(0, src_splits, src_split_stride, slice);
+      rope_src_load8<SRC>(rs.src, row, base[0] + ia[0], slice, da0);
+      rope_src_load8<SRC>(rs.src, row, base[0] + ib[0], slice, db0);
+      if (two) {
+        rope_src_load8<SRC>(rs.src, row, base[1] + ia[1], slice, da1);
+        rope_src_load8<SRC>(rs.src, row, base[1] + ib[1], slice, db1);
+      }
+      load_k();
+      acc_a[0] = rope_src_add8(0.f, da0, 0, src_splits);
+      acc_b[0] = rope_src_add8(0.f, db0, 0, src_splits);
+      acc_a[1] = acc_b[1] = 0.f;
+      if (two) {
+        acc_a[1] = rope_src_add8(0.f, da1, 0, src_splits);
+        acc_b[1] = rope_src_add8(0.f, db1, 0, src_splits);
+      }
+      for (int s0 = 8; s0 < src_splits; s0 += 8) {
+        rope_src_slices(s0, src_splits, src_split_stride, slice);
+        rope_src_load8<SRC>(rs.src, row, base[0] + ia[0], slice, da0);
+        rope_src_load8<SRC>(rs.src, row, base[0] + ib[0], slice, db0);
+        rope_src_load8<SRC>(rs.src, row, base[1] + ia[1], slice, da1);
+        rope_src_load8<SRC>(rs.src, row, base[1] + ib[1], slice, db1);
+        acc_a[0] = rope_src_add8(acc_a[0], da0, s0, src_splits);
+        acc_b[0] = rope_src_add8(acc_b[0], db0, s0, src_splits);
+        acc_a[1] = rope_src_add8(acc_a[1], da1, s0, src_splits);
+        acc_b[1] = rope_src_add8(acc_b[1], db1, s0, src_splits);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        if (ok[j] && (j == 0 || two)) {
+          const float a = as_output(acc_a[j], rs.round_sum), b = as_output(acc_b[j], rs.round_sum);
+          dst[j][ia[j]] = f32_to_bf16(rot[j] ? rot_first(a, b, c[j], sv[j]) : a);
+          dst[j][ib[j]] = f32_to_bf16(rot[j] ? rot_second(a, b, c[j], sv[j]) : b);
+        }
+    };
+    round(0, [&]() {
+      if (my_lo < my_hi) {
+        ATT_LOAD_K_AT(my_lo, first_page)
+        ATT_LOAD_V_AT(my_lo, first_page)
+      }
+    });
+    for (int first = 2 * T; first < items; first += 2 * T) round(first, []() {});
+    __syncthreads();
+    if (makes_kv && chunk == 0) {
+      // into the pages, for the steps that follow
+      const int slot = pos0 % page_size;
+      const size_t slab = (static_cast<size_t>(max(0, bt[min(pos0 / page_size, table_width - 1)])) * n_kv + g) * page_size * D;
+      for (int d = threadIdx.x; d < D; d += 64 * W) {
+        const_cast<bf16_t*>(k_cache)[slab + cache_k_offset(TILED, page_size, D, slot, d)] = kv_s[0][d];
+        const_cast<bf16_t*>(v_cache)[slab + cache_v_offset(TILED, page_size, D, slot, d)] = kv_s[1][d];
+      }
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      qf[ks].u = col_ok ? *reinterpret_cast<const u32x4_t*>(&q_s[hh][32 * ks + 8 * gq]) : zero4;
+  } else {
+    const bf16_t* qp = q + static_cast<size_t>(tok0 + (col_ok ? tt : 0)) * q_stride +
+                       static_cast<size_t>(h_base + (col_ok ? hh : 0)) * D + 8 * gq;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      qf[ks].u = *reinterpret_cast<const u32x4_t*>(qp + 32 * ks);
+      if (!col_ok) qf[ks].u = zero4;
+    }
+  }
+  // where the token's own key sits among a block's score rows and value pieces
+  const int new_j = pos0 % 64, new_u = new_j / 32;
+  const int new_sb = (new_j % 8) / 4, new_r = 4 * ((new_j % 32) / 8) + new_j % 4;  // key row of the score products
+  const int new_gq = (new_j % 32) / 8, new_e = new_j % 8;                          // value piece and place in it
   if (my_lo < my_hi) {
-    ATT_LOAD_K(my_lo)
+    if (!ROPE) ATT_LOAD_K(my_lo)
     ATT_PUT_NEW_K(my_lo)
   }
   for (int kb = my_lo; kb < my_hi; ++kb) {
-    // values of this block: lane (r, gq) holds 8 consecutive keys of value row 16*dt + r
-    AFrag8 vf[2][DT];
     const bool mine0 = mine(kb, 0), mine1 = mine(kb, 1);
-    if (TILED) {
-      const int key0 = kb * 64;
-      const bf16_t* vp = v_cache + (static_cast<size_t>(page_of(key0)) * n_kv + g) * D * page_size +
-                         static_cast<size_t>(key0 % page_size) * D + 8 * lane;
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        if (u == 0 ? mine0 : mine1) {
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt)
-            vf[u][dt].u = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(vp + (u * DT + dt) * 512));
-        } else {
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) vf[u][dt].u = zero4;
-        }
-      }
-    } else {
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        if (u == 0 ? mine0 : mine1) {
-          const int key = kb * 64 + 32 * u + 8 * gq;
-          const bf16_t* vp = v_cache + (static_cast<size_t>(page_of(key)) * n_kv + g) * D * page_size + key % page_size;
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt)
-            vf[u][dt].u = *reinterpret_cast<const u32x4_t*>(vp + static_cast<size_t>(16 * dt + r) * page_size);
-        } else {
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) vf[u][dt].u = zero4;
-        }
-      }
-    }
+    if (!(ROPE && kb == my_lo)) ATT_LOAD_V_AT(kb, page_of(kb * 64))  // (ROPE: the first block's are on their way)
     // scores
     f32x4_t s[2][2];
 #pragma unroll
@@ -502,6 +574,8 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
         acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[u][dt].v, pf[u].v, acc[dt], 0, 0, 0);
   }
 #undef ATT_LOAD_K
+#undef ATT_LOAD_K_AT
+#undef ATT_LOAD_V_AT
 #undef ATT_PUT_NEW_K
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
@@ -970,7 +1044,7 @@ static int launch_attn_mfma(const void* q, int q_stride, void* out, const void* 
                             const int32_t* tiles, int n_tiles, const int32_t* block_table, int table_width,
                             int page_size, int head_dim, int n_heads, int n_kv, float scale, int window,
                             int n_waves, int n_splits, float* workspace, size_t workspace_floats,
-                            int leave_splits, const RopeSrc* rope, hipStream_t stream) {
+                            int leave_splits, const RopeSrc* rope, bool rope_f32, hipStream_t stream) {
   YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_mfma: bad head counts");
   YK_REQUIRE(n_waves == 1 || n_waves == 4, "attn_mfma: a workgroup has 1 or 4 waves");
   YK_REQUIRE(yk_attn_mfma_supported(head_dim), "attn_mfma: head_dim must be 64 or 128");
@@ -1007,7 +1081,7 @@ static int launch_attn_mfma(const void* q, int q_stride, void* out, const void* 
     else attn_mfma_kernel<DD, 4, false, RR><<<grid, block, 0, stream>>>(YK_ARGS);                  \
   }
 #define YK_LAUNCH(DD)                                                                              \
-  if (rope) { YK_LAUNCH_R(DD, true) } else { YK_LAUNCH_R(DD, false) }                              \
+  if (!rope) { YK_LAUNCH_R(DD, 0) } else if (rope_f32) { YK_LAUNCH_R(DD, 2) } else { YK_LAUNCH_R(DD, 1) } \
   if (yk_check_launch("attn_mfma")) return -1;                                                     \
   if (n_splits > 1 && !leave_splits) {                                                             \
     attn_combine_kernel<DD><<<dim3(n_tiles, n_kv * chunks), 256, 0, stream>>>(                     \
@@ -1033,7 +1107,7 @@ extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* 
                             int leave_splits, hipStream_t stream) {
   return launch_attn_mfma(q, q_stride, out, k_cache, v_cache, tiles, n_tiles, block_table, table_width, page_size,
                           head_dim, n_heads, n_kv, scale, window, n_waves, n_splits, workspace, workspace_floats,
-                          leave_splits, nullptr, stream);
+                          leave_splits, nullptr, false, stream);
 }
 
 // yk_attn_mfma for a step of single tokens (every tile holds ONE token), with rotary + append
@@ -1061,7 +1135,6 @@ extern "C" int yk_attn_mfma_rope(const void* src, int src_dtype, int n_src_split
              "attn_mfma_rope: row stride too small");
   RopeSrc rs;
   rs.src = src;
-  rs.src_f32 = src_dtype == YK_F32;
   rs.n_splits = n_src_splits;
   rs.split_stride = static_cast<size_t>(n_tokens) * src_stride;
   rs.round_sum = round_sum;
@@ -1072,11 +1145,9 @@ extern "C" int yk_attn_mfma_rope(const void* src, int src_dtype, int n_src_split
   rs.interleaved = interleaved;
   rs.max_positions = rotary_dim ? max_positions : 1;
   rs.append = append != 0;
-  rs.k_write = static_cast<bf16_t*>(k_cache);
-  rs.v_write = static_cast<bf16_t*>(v_cache);
   return launch_attn_mfma(nullptr, 0, out, k_cache, v_cache, tiles, n_tiles, block_table, table_width, page_size,
                           head_dim, n_heads, n_kv, scale, window, n_waves, n_splits, workspace, workspace_floats,
-                          leave_splits, &rs, stream);
+                          leave_splits, &rs, src_dtype == YK_F32, stream);
 }
 
 // The second half of yk_attn_mfma for a launch that was told to leave its splits in the

@@ -108,26 +108,36 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float4 v) {
 // (as_output, in common.h: the sum of a product's K slices is rounded as the product's
 // output would have been)
 
+// the row of an embedding table that token `src` of the step names (ids are checked on the
+// host; clamped here so that a bad id cannot read out of bounds)
+__device__ __forceinline__ size_t table_row(const int32_t* __restrict__ ids, size_t src, int table_rows) {
+  const int id = ids[src];
+  return static_cast<size_t>(id < 0 ? 0 : (id >= table_rows ? table_rows - 1 : id));
+}
+
 // ------------------------------------------------------------- residual add + RMS norm
 // For row r (source row rows[r] when rows is given):
 //   v = residual[src] + sum over s of delta[s][src]   (float32; delta may be absent;
 //       n_splits > 1: delta holds the unreduced K slices of a product, float32)
 //   residual[src] = v                                  (only when rows is null)
 //   out[r] = v * rsqrt(mean(v^2) + eps) * (weight [+ 1])
+// With table_ids the residual stream starts here: `delta` is an embedding table, v =
+// table[table_ids[src]] (the residual is not read, and written as in the plain form).
 // General form: any width, two passes over the row.
 template <typename TD, typename TW, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
                                    int n_splits, size_t split_stride, int round_sum,
                                    const int32_t* __restrict__ rows, const TW* __restrict__ weight,
-                                   TO* __restrict__ out, int width, float eps, int unit_offset) {
+                                   TO* __restrict__ out, int width, float eps, int unit_offset,
+                                   const int32_t* __restrict__ table_ids, int table_rows) {
   __shared__ float scratch[17];
   const int r = blockIdx.x;
   const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
   float* res = residual + src * width;
-  const TD* del = delta ? delta + src * width : nullptr;
+  const TD* del = delta ? delta + (table_ids ? table_row(table_ids, src, table_rows) : src) * width : nullptr;
   float ss = 0.f;
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
-    float v = res[c];
+    float v = table_ids ? 0.f : res[c];
     if (del) {
       float d = 0.f;
       for (int s = 0; s < n_splits; ++s) d += to_f32<TD>(del[s * split_stride + c]);
@@ -160,19 +170,19 @@ template <typename TD, typename TW, typename TO, int NORM_IT>
 __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(
     float* __restrict__ residual, const TD* __restrict__ delta, int n_splits, size_t split_stride,
     int round_sum, const int32_t* __restrict__ rows, const TW* __restrict__ weight, TO* __restrict__ out,
-    int width, float eps, int unit_offset) {
+    int width, float eps, int unit_offset, const int32_t* __restrict__ table_ids, int table_rows) {
   __shared__ float scratch[17];
   const int r = blockIdx.x;
   const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
   float* res = residual + src * width;
-  const TD* del = delta ? delta + src * width : nullptr;
+  const TD* del = delta ? delta + (table_ids ? table_row(table_ids, src, table_rows) : src) * width : nullptr;
   float4 v[NORM_IT], w[NORM_IT], ds[NORM_IT];
   float ss = 0.f;
 #pragma unroll
   for (int it = 0; it < NORM_IT; ++it) {
     const int c = (threadIdx.x + it * blockDim.x) * 4;
     if (c < width) {
-      v[it] = load4<float>(res + c);
+      v[it] = table_ids ? make_float4(0.f, 0.f, 0.f, 0.f) : load4<float>(res + c);
       w[it] = load4<TW>(weight + c);
     }
   }
@@ -241,7 +251,8 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(
 template <typename TD, typename TW, typename TO>
 static int launch_add_rmsnorm(float* residual, const void* delta, int n_splits, size_t split_stride,
                               int round_sum, const int32_t* rows, const void* weight, void* out, int n_rows,
-                              int width, float eps, int unit_offset, hipStream_t stream) {
+                              int width, float eps, int unit_offset, const int32_t* table_ids, int table_rows,
+                              hipStream_t stream) {
   const bool aligned = width % 4 == 0 && reinterpret_cast<uintptr_t>(residual) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(delta) % 16 == 0 && reinterpret_cast<uintptr_t>(weight) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(out) % 16 == 0 && split_stride % 4 == 0;
@@ -254,7 +265,7 @@ static int launch_add_rmsnorm(float* residual, const void* delta, int n_splits, 
 #define YK_NORM(IT)                                                                           \
     add_rmsnorm_vec_kernel<TD, TW, TO, IT><<<n_rows, threads, 0, stream>>>(                   \
         residual, static_cast<const TD*>(delta), n_splits, split_stride, round_sum, rows,     \
-        static_cast<const TW*>(weight), static_cast<TO*>(out), width, eps, unit_offset)
+        static_cast<const TW*>(weight), static_cast<TO*>(out), width, eps, unit_offset, table_ids, table_rows)
     if (pieces <= 1) YK_NORM(1);
     else if (pieces <= 2) YK_NORM(2);
     else if (pieces <= 4) YK_NORM(4);
@@ -263,19 +274,23 @@ static int launch_add_rmsnorm(float* residual, const void* delta, int n_splits, 
   } else {
     add_rmsnorm_kernel<TD, TW, TO><<<n_rows, width >= 2048 ? 512 : 256, 0, stream>>>(
         residual, static_cast<const TD*>(delta), n_splits, split_stride, round_sum, rows,
-        static_cast<const TW*>(weight), static_cast<TO*>(out), width, eps, unit_offset);
+        static_cast<const TW*>(weight), static_cast<TO*>(out), width, eps, unit_offset, table_ids, table_rows);
   }
   return yk_check_launch("add_rmsnorm");
 }
 
 // delta may be null (then delta_dtype is ignored); rows may be null.  n_splits > 1 needs
 // float32 delta laid out [n_splits][rows of the residual][width]; round_sum: the slices' sum
-// is rounded to bfloat16 before it is added.
+// is rounded to bfloat16 before it is added.  table_ids (null, or one id per residual row):
+// delta is an embedding table of table_rows rows and the residual starts as its rows
+// table_ids[.] (n_splits 1, no rows).
 extern "C" int yk_add_rmsnorm(float* residual, const void* delta, int delta_dtype, int n_splits,
                               int round_sum, const int32_t* rows, const void* weight, int weight_dtype, void* out,
                               int out_dtype, int n_rows, int n_residual_rows, int width, float eps,
-                              int unit_offset, hipStream_t stream) {
+                              int unit_offset, const int32_t* table_ids, int table_rows, hipStream_t stream) {
   YK_REQUIRE(n_rows >= 0 && width > 0 && n_residual_rows >= 0, "add_rmsnorm: bad sizes");
+  YK_REQUIRE(!table_ids || (delta && n_splits == 1 && !rows && table_rows > 0 && !round_sum),
+             "add_rmsnorm: an embedding table comes whole, with one id per row of the residual");
   YK_REQUIRE(eps >= 0.f, "add_rmsnorm: eps must not be negative");
   YK_REQUIRE(n_splits >= 1, "add_rmsnorm: bad split count");
   YK_REQUIRE(n_splits == 1 || delta_dtype == YK_F32, "add_rmsnorm: unreduced slices must be float32");
@@ -287,7 +302,7 @@ extern "C" int yk_add_rmsnorm(float* residual, const void* delta, int delta_dtyp
   const size_t stride = static_cast<size_t>(n_residual_rows) * width;
 #define YK_CASE(DD, TD, WD, TW, OD, TO)                                  \
   if (delta_dtype == DD && weight_dtype == WD && out_dtype == OD)        \
-    return launch_add_rmsnorm<TD, TW, TO>(residual, delta, n_splits, stride, round_sum, rows, weight, out, n_rows, width, eps, unit_offset, stream);
+    return launch_add_rmsnorm<TD, TW, TO>(residual, delta, n_splits, stride, round_sum, rows, weight, out, n_rows, width, eps, unit_offset, table_ids, table_rows, stream);
   YK_CASE(YK_F32, float, YK_F32, float, YK_F32, float)
   YK_CASE(YK_F32, float, YK_F32, float, YK_BF16, bf16_t)
   YK_CASE(YK_F32, float, YK_BF16, bf16_t, YK_F32, float)

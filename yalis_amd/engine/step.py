@@ -81,7 +81,9 @@ class _Uploader:
         self.events: List[Optional[torch.cuda.Event]] = [None, None]
         self.turn = 0
 
-    def upload(self, buf: np.ndarray) -> torch.Tensor:
+    def upload(self, buf: np.ndarray, into: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``into``: a device buffer of at least ``buf.size`` ints to fill (a captured graph's
+        own); by default a new tensor."""
         if not self.cuda:
             return torch.from_numpy(buf.copy())
         i = self.turn
@@ -92,7 +94,7 @@ class _Uploader:
             self.bufs[i] = torch.empty(max(4096, 2 * buf.size), dtype=torch.int32, pin_memory=True)
         stage = self.bufs[i][: buf.size]
         stage.numpy()[:] = buf
-        dev = torch.empty(buf.size, dtype=torch.int32, device=self.device)
+        dev = torch.empty(buf.size, dtype=torch.int32, device=self.device) if into is None else into[: buf.size]
         dev.copy_(stage, non_blocking=True)
         ev = torch.cuda.Event()
         ev.record()
@@ -294,7 +296,7 @@ class ModelRunner:
         else:
             if layout != entry.layout:
                 raise RuntimeError("a decode step's integer arrays changed shape under a captured graph")
-            entry.ints.copy_(self._uploader.upload(buf), non_blocking=True)
+            self._uploader.upload(buf, into=entry.ints)
             self._feed_tokens(entry.ints, layout, len(spans), token_source, token_index is not None)
         entry.graph.replay()
         self.graph_replays += 1

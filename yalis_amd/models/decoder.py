@@ -150,8 +150,12 @@ class DecoderModel:
     # -------------------------------------------------------------------------- run
     def forward(self, ctx) -> torch.Tensor:
         """Run the step's tokens; returns float32 logits [wanted rows, vocab]."""
-        residual = self.embedding.forward(ctx.arrays["token_ids"])
-        delta = None
+        first = self.blocks[self.spec.run_order[0].layer]
+        begin = getattr(self.embedding, "begin", None)
+        if begin is not None:
+            residual, delta = begin(ctx.arrays["token_ids"], bool(getattr(first, "takes_embedded_rows", False)))
+        else:
+            residual, delta = self.embedding.forward(ctx.arrays["token_ids"]), None
         for i, e in enumerate(self.spec.run_order):
             delta = self.blocks[e.layer].forward(residual, delta, ctx, ctx.site(i))
         rows = ctx.arrays["logit_rows"]

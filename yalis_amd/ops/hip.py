@@ -45,7 +45,7 @@ _SIGNATURES = {
     "yk_cache_tiled": ([_c_int, _c_int, _c_int], _c_int),
     "yk_embed": ([_vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_add_rmsnorm": (
-        [_vp, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp],
+        [_vp, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp, _c_int, _vp],
         _c_int,
     ),
     "yk_rope_append": (
@@ -149,6 +149,25 @@ class SplitSum:
 
     def float(self) -> torch.Tensor:
         return self.reduce()
+
+
+class EmbeddedRows:
+    """The rows of an embedding table that a step's tokens name, not yet gathered: it stands
+    for a tensor [tokens, width] with which a residual stream starts.  The norm kernel that
+    comes first gathers the rows itself (``add_rmsnorm`` with this as ``delta`` fills the
+    residual and normalises it in one pass); ``gather()`` gives the tensor (float32)."""
+
+    def __init__(self, ops, token_ids: torch.Tensor, table: torch.Tensor):
+        self.ops, self.token_ids, self.table = ops, token_ids, table
+        self.shape = (token_ids.numel(), table.shape[1])
+        self.dtype = torch.float32
+        self.device = table.device
+
+    def gather(self) -> torch.Tensor:
+        return self.ops.embed(self.token_ids, self.table)
+
+    def float(self) -> torch.Tensor:
+        return self.gather()
 
 
 class SplitAttention:
@@ -309,6 +328,13 @@ class HipOps:
         )
         return out
 
+    def embedded_rows(self, token_ids: torch.Tensor, table: torch.Tensor):
+        """(an uninitialised float32 residual [tokens, width], the ``EmbeddedRows`` that the
+        first ``add_rmsnorm`` fills it from): the embedding without a kernel of its own."""
+        self._rows(table, "embed table")
+        residual = torch.empty((token_ids.numel(), table.shape[1]), dtype=torch.float32, device=table.device)
+        return residual, EmbeddedRows(self, token_ids, table)
+
     # ----------------------------------------------------------------------- norm
     def _norm(self, residual, delta, rows, weight, eps, unit_offset, out_dtype, n_out):
         self._rows(residual, "residual")
@@ -318,7 +344,16 @@ class HipOps:
         if weight.numel() != width:
             raise KernelError(f"norm weight has {weight.numel()} elements, rows have {width}")
         n_splits, round_sum = 1, 0
-        if isinstance(delta, SplitSum):
+        table_ids, table_rows = None, 0
+        if isinstance(delta, EmbeddedRows):
+            if rows is not None or tuple(delta.shape) != tuple(residual.shape):
+                raise KernelError(f"embedded rows {tuple(delta.shape)} start a residual of their own shape, got {tuple(residual.shape)}")
+            table_ids, delta = delta.token_ids, delta.table
+            self._rows(delta, "embedding table")
+            if not delta.is_contiguous() or table_ids.dtype != torch.int32:
+                raise KernelError("the embedding table must be contiguous and the token ids int32")
+            table_rows = delta.shape[0]
+        elif isinstance(delta, SplitSum):
             n_splits, round_sum, delta = delta.n_splits, delta.round_sum, delta.tensor
             if tuple(delta.shape[1:]) != tuple(residual.shape):
                 raise KernelError(f"delta {tuple(delta.shape[1:])} does not match the residual {tuple(residual.shape)}")
@@ -329,7 +364,8 @@ class HipOps:
             self.lib.yk_add_rmsnorm(
                 residual.data_ptr(), _ptr(delta), 0 if delta is None else _code(delta.dtype), n_splits, round_sum,
                 _ptr(rows), weight.data_ptr(), _code(weight.dtype), out.data_ptr(), _code(out_dtype),
-                n_out, residual.shape[0], width, float(eps), int(bool(unit_offset)), self._stream(),
+                n_out, residual.shape[0], width, float(eps), int(bool(unit_offset)), _ptr(table_ids), table_rows,
+                self._stream(),
             )
         )
         return out

@@ -100,6 +100,10 @@ class FeedForward(Part):
 
 
 class Norm(Part):
+    # True when ``add_norm`` hands ``delta`` to a kernel library that understands an embedding's
+    # ungathered rows (``ops.embedded_rows``) in its place
+    takes_embedded_rows = False
+
     def add_norm(self, residual: torch.Tensor, delta: Optional[torch.Tensor]) -> torch.Tensor:
         """residual (float32, [N, size]) += delta in place when delta is given;
         returns norm(residual) in the activation dtype."""
@@ -118,6 +122,11 @@ class Block:
     """The arrangement of norms, mixer and feed-forward around the residual.
     Built from four finished parts: (mixer_norm, mixer, feed_forward_norm,
     feed_forward)."""
+
+    # True when the block's first act is ``add_norm(residual, delta)`` of a norm that takes an
+    # embedding's ungathered rows as ``delta`` (``Norm.takes_embedded_rows``): the model then
+    # starts the residual stream inside that norm's kernel.
+    takes_embedded_rows = False
 
     def parts(self):
         raise NotImplementedError

@@ -22,6 +22,10 @@ class PreNormBlock(Block):
         self.feed_forward_norm = feed_forward_norm
         self.feed_forward = feed_forward
 
+    @property
+    def takes_embedded_rows(self):
+        return bool(getattr(self.mixer_norm, "takes_embedded_rows", False))
+
     def parts(self):
         return (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward)
 

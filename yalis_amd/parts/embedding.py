@@ -39,6 +39,16 @@ class TokenEmbedding(Part):
         """The float32 residual stream [N, hidden]."""
         return self.rt.ops.embed(token_ids, self.table)
 
+    def begin(self, token_ids: torch.Tensor, lazily: bool):
+        """(residual, delta) with which the first block starts: the gathered rows and nothing
+        to add, or, ``lazily`` and where the kernel library can, an unfilled residual and the
+        rows as a pending contribution that the first norm's kernel gathers itself (a block says
+        through ``takes_embedded_rows`` whether its first norm does)."""
+        make = getattr(self.rt.ops, "embedded_rows", None)
+        if lazily and make is not None:
+            return make(token_ids, self.table)
+        return self.forward(token_ids), None
+
 
 @register_head("lm_head")
 class LMHead(Part):

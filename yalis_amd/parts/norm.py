@@ -29,6 +29,7 @@ class RMSNorm(Norm):
         self.eps = float(params["eps"])
         self.unit_offset = bool(params.get("unit_offset", False))
         self.weight: Optional[torch.Tensor] = None
+        self.takes_embedded_rows = hasattr(rt.ops, "embedded_rows")
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         return {self.name: TensorSpec((self.size,), "float", ("one_plus_normal", 0.1))}
