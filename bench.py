@@ -20,29 +20,7 @@ import time
 HBM_GBPS = 8000.0  # MI355X published peaks
 BF16_FLOPS = 2.5e15
 
-LLAMA3_8B = {
-    "architectures": ["LlamaForCausalLM"],
-    "hidden_size": 4096,
-    "num_hidden_layers": 32,
-    "num_attention_heads": 32,
-    "num_key_value_heads": 8,
-    "head_dim": 128,
-    "intermediate_size": 14336,
-    "vocab_size": 128256,
-    "rms_norm_eps": 1e-5,
-    "rope_theta": 500000.0,
-    "rope_scaling": None,
-    "max_position_embeddings": 8192,
-    "tie_word_embeddings": False,
-}
-_LLAMA3_SCALING = {"rope_type": "llama3", "low_freq_factor": 1.0, "high_freq_factor": 4.0,
-                   "original_max_position_embeddings": 8192}
-# further shapes (not the default): --shape 3b / 70b
-LLAMA32_3B = dict(LLAMA3_8B, hidden_size=3072, num_hidden_layers=28, num_attention_heads=24, intermediate_size=8192,
-                  rope_scaling=dict(_LLAMA3_SCALING, factor=32.0), tie_word_embeddings=True)
-LLAMA31_70B = dict(LLAMA3_8B, hidden_size=8192, num_hidden_layers=80, num_attention_heads=64, intermediate_size=28672,
-                   rope_scaling=dict(_LLAMA3_SCALING, factor=8.0))
-SHAPES = {"8b": ("Llama-3-8B", LLAMA3_8B), "3b": ("Llama-3.2-3B", LLAMA32_3B), "70b": ("Llama-3.1-70B", LLAMA31_70B)}
+from yalis_amd.models.presets import SHAPES  # name -> (label, config.json dictionary)
 
 
 def machine_probe(cfg: dict) -> int:
@@ -153,7 +131,7 @@ def main() -> int:
     ap.add_argument("--mixed", action="store_true", help="measure mixed steps instead: 32 decode streams beside portions of 4,096-token prompts")
     ap.add_argument("--portion", type=int, default=480, help="tokens of a prompt portion in --mixed steps (with the 32 decoded tokens: 512 rows, as the scheduler cuts under a budget of 512)")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel (for hardware counters)")
-    ap.add_argument("--shape", choices=sorted(SHAPES), default="8b", help="layer sizes (default: the 8B shape of the headline)")
+    ap.add_argument("--shape", choices=("8b", "3b", "70b"), default="8b", help="layer sizes (default: the 8B shape of the headline)")
     ap.add_argument("--sample", action="store_true", help="time instead the choice of a token alone (greedy and each sampling rule) at the shape's vocabulary for --batch rows")
     ap.add_argument("--probe", action="store_true", help="measure instead what a plain streaming read and a plain matrix-core loop reach on this card")
     args = ap.parse_args()

@@ -12,7 +12,14 @@ from yalis_amd.config.registry import get_architecture, known_architectures, loa
 from yalis_amd.config.runtime import EngineConfig, InferenceConfig, ModelConfig
 from yalis_amd.engine.factory import spec_from_config, tensor_specs_for
 from yalis_amd.models.llama import LlamaConfig
-from yalis_amd.weights.loader import TensorSpec, WeightsError, load_tensors, target_dtype
+from yalis_amd.weights.loader import TensorSpec, WeightsError, open_tensors, target_dtype
+
+
+def load_tensors(folder, specs, engine_dtype, device):
+    """Every tensor of ``specs`` through the loader that generation uses (``open_tensors``:
+    the folder is checked as a whole, then each tensor is read when asked for)."""
+    source = open_tensors(folder, specs, {n: 1 for n in specs}, engine_dtype, device)
+    return {n: source[n] for n in specs}
 from yalis_amd.weights.random_init import write_random_model
 from yalis_amd.weights.safetensors_io import SafetensorsError, index_folder, read_tensor, write_dict
 
@@ -167,6 +174,34 @@ def test_random_folder_loads_back_bit_exact(tmp_path):
     f32 = write_random_model(str(tmp_path / "a32"), TINY_A, seed=0, dtype="float32")
     assert load_tensors(f32, tensor_specs_for(TINY_A), "bfloat16", "cpu")["model.norm.weight"].dtype == torch.float32
     assert json.load(open(os.path.join(folder, "config.json")))["architectures"] == ["LlamaForCausalLM"]
+
+
+def test_sixteen_bit_floats_of_the_other_kind_and_wide_matrices(tmp_path, caplog):
+    """A checkpoint stored in float16: the bfloat16 engine refuses it (one error naming every
+    such tensor), the float32 engine widens it exactly.  Matrices stored in 32 bits stay so in
+    the bfloat16 engine, which says so once."""
+    import logging
+
+    specs = tensor_specs_for(TINY_A)
+    folder = write_random_model(str(tmp_path / "h"), TINY_A, seed=0, dtype="bfloat16")
+    tensors = {n: read_tensor(e).to(torch.float16) for n, e in index_folder(folder).items()}
+    write_dict(os.path.join(folder, "model.safetensors"), tensors)
+    with pytest.raises(WeightsError, match="float16") as e:
+        load_tensors(folder, specs, "bfloat16", "cpu")
+    assert len(e.value.wrong_kind) == len(specs)
+    wide = load_tensors(folder, specs, "float32", "cpu")
+    assert all(t.dtype == torch.float32 for t in wide.values())
+    assert torch.equal(wide["lm_head.weight"], tensors["lm_head.weight"].float())
+    f32 = write_random_model(str(tmp_path / "w"), TINY_A, seed=0, dtype="float32")
+    log = logging.getLogger("yalis_amd")
+    log.propagate = True  # (the package's loggers keep to themselves; the test listens in)
+    try:
+        with caplog.at_level(logging.WARNING, logger="yalis_amd"):
+            got = load_tensors(f32, specs, "bfloat16", "cpu")
+    finally:
+        log.propagate = False
+    assert got["lm_head.weight"].dtype == torch.float32
+    assert sum("stored in 32 bits" in r.getMessage() for r in caplog.records) == 1
 
 
 def test_one_error_lists_everything_wrong(tmp_path):

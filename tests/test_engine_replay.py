@@ -20,8 +20,8 @@ BACKENDS = [
 
 # prompt lengths of the brief's two tiny configurations, and own ones for C and D
 LENGTHS = {"A": [5, 17, 32, 61, 77, 40], "B": [1, 40, 130, 66, 25, 90], "C": [50, 3, 97, 140, 64, 31], "D": [33, 129, 70, 2, 65],
-           "E": [44, 9, 120, 71, 36]}
-PAGE = {"A": 16, "B": 32, "C": 16, "D": 64, "E": 48}
+           "E": [44, 9, 120, 71, 36], "F": [70, 129, 200, 5, 64, 150]}
+PAGE = {"A": 16, "B": 32, "C": 16, "D": 64, "E": 48, "F": 64}
 
 _ops_cache = {}
 
@@ -41,7 +41,7 @@ _plain_cache = {}
 
 def setup(name, dtype):
     cfg = ALL[name]
-    weights = P.random_weights(cfg, seed={"A": 0, "B": 1, "C": 2, "D": 3, "E": 4}[name])
+    weights = P.random_weights(cfg, seed={"A": 0, "B": 1, "C": 2, "D": 3, "E": 4, "F": 5}[name])
     reqs = C.make_requests(cfg, LENGTHS[name], seed=10)
     key = (name, dtype == "bfloat16")
     if key not in _plain_cache:
@@ -50,7 +50,7 @@ def setup(name, dtype):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F"])
 @pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
 def test_replay_modes(backend, name, mode):
     device, dtype = backend
@@ -87,7 +87,7 @@ FULL_WIDTH = {
     "max_position_embeddings": 8192, "tie_word_embeddings": False,
 }
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("name,seed", [("A", 1), ("B", 2), ("C", 3), ("D", 4), ("E", 5), ("C", 6), ("D", 7)])
+@pytest.mark.parametrize("name,seed", [("A", 1), ("B", 2), ("C", 3), ("D", 4), ("E", 5), ("C", 6), ("D", 7), ("F", 8), ("F", 9)])
 def test_replay_cut_at_random(backend, name, seed):
     """Random subsets of up to four live requests a step, random numbers of tokens each, a
     pool just large enough: the logits are the plain implementation's, and no page is lost."""
@@ -199,10 +199,12 @@ def test_first_tokens(backend):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-def test_far_key_across_pages(backend):
+@pytest.mark.parametrize("page", [16, 64])
+def test_far_key_across_pages(backend, page):
     """Random weights give flat attention, which would hide a lost far key.  Here the
     last token equals an early one and the query/key projections of one head are scaled
-    up, so that head looks hundreds of tokens back."""
+    up, so that head looks hundreds of tokens back.  Pages of 16 tokens are kept in the
+    plain order, those of 64 (bfloat16) in the order the matrix-core attention loads them."""
     device, dtype = backend
     cfg = ALL["C"]
     weights = P.random_weights(cfg, seed=2)
@@ -211,9 +213,18 @@ def test_far_key_across_pages(backend):
     toks = C.make_requests(cfg, [300], seed=6)["r0"]
     toks[-1] = toks[3]
     want = C.plain_logits(cfg, weights, {"r0": toks}, dtype == "bfloat16")
-    runner = C.make_runner(cfg, weights, dtype, device, ops_for(device), 16, 19)
+    runner = C.make_runner(cfg, weights, dtype, device, ops_for(device), page, -(-300 // page))
     got, _ = C.run_trace(runner, C.trace_tail({"r0": toks}, tail=8))
     C.assert_matches(got, want, dtype == "bfloat16", "far key")
+    # The bfloat16 tolerance is wide (a few times 2^-8 of the largest logit), so the last token
+    # is held to more: with another token in the early place the plain implementation's last
+    # logits move by `moved`; the engine's stay within a third of that of the right ones, which a
+    # lost or stale key at that place would not.
+    other = list(toks)
+    other[3] = (other[3] + 1) % cfg["vocab_size"]
+    moved = (C.plain_logits(cfg, weights, {"r0": other}, dtype == "bfloat16")["r0"][-1] - want["r0"][-1]).abs().max().item()
+    assert moved > 2 * C.tolerance(want["r0"], dtype == "bfloat16")
+    assert (got["r0"][-1] - want["r0"][-1]).abs().max().item() < moved / 3
 
 
 @pytest.mark.gpu
@@ -242,3 +253,94 @@ def test_graph_replays_match_eager_steps(dtype):
     assert torch.equal(outs[True]["a"], outs[False]["a"]), "a replayed step differs from the eager step"
     assert torch.equal(outs[True]["b"], outs[False]["b"])
     C.assert_matches({"r3": torch.cat([want["r3"][:0], outs[True]["a"]])}, {"r3": want["r3"][100:]}, dtype == "bfloat16", "graph decode")
+
+
+def _many_requests_trace(cfg, n_live, seed):
+    """``n_live`` short requests: whole prompts eight to a step, then steps that hold one token of
+    every request still running; request i decodes 3 + i % 4 tokens, so that a quarter of the
+    requests drops out of each of the last steps."""
+    g = torch.Generator().manual_seed(seed)
+    reqs, prompt_len = {}, {}
+    for i in range(n_live):
+        n_prompt, tail = 3 + (7 * i) % 38, 3 + i % 4
+        reqs[f"q{i}"] = torch.randint(0, cfg["vocab_size"], (n_prompt + tail,), generator=g).tolist()
+        prompt_len[f"q{i}"] = n_prompt
+    steps = []
+    names = list(reqs)
+    for i in range(0, n_live, 8):
+        steps.append({"step": len(steps), "end": [], "entries": [
+            {"id": r, "tokens": reqs[r][: prompt_len[r]], "want": list(range(prompt_len[r]))} for r in names[i : i + 8]]})
+    for d in range(6):
+        entries = [{"id": r, "tokens": [reqs[r][prompt_len[r] + d]], "want": [0]} for r in names if prompt_len[r] + d < len(reqs[r])]
+        ends = [e["id"] for e in entries if prompt_len[e["id"]] + d + 1 == len(reqs[e["id"]])]
+        steps.append({"step": len(steps), "entries": entries, "end": ends})
+    return reqs, steps
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("graphs", [True, False], ids=["graphs", "eager"])
+@pytest.mark.parametrize("dtype,n_live", [("bfloat16", 24), ("bfloat16", 64), ("bfloat16", 80), ("bfloat16", 130), ("float32", 80)])
+def test_decode_steps_of_many_requests(dtype, n_live, graphs):
+    """Decode steps of 24 to 130 live requests (the 32- and 64-row forms of the few-row
+    product inside captured graphs, a graph per number of requests as requests drop out; above
+    64 requests no graph, the vendor library's products and its float32 output head), with
+    three query heads a kv head over tiled pages."""
+    cfg = ALL["F"]
+    weights = P.random_weights(cfg, seed=5)
+    reqs, steps = _many_requests_trace(cfg, n_live, seed=40 + n_live)
+    want = C.plain_logits(cfg, weights, reqs, dtype == "bfloat16")
+    runner = C.make_runner(cfg, weights, dtype, "cuda:0", ops_for("cuda:0"), 64, n_live, max_seqs=n_live)
+    runner.use_graphs = graphs
+    got, _ = C.run_trace(runner, steps)
+    C.assert_matches(got, want, dtype == "bfloat16", f"{n_live} live requests")
+    # (steps of more than 64 requests are never replayed; once enough requests have dropped
+    # out, the later steps of such a run are)
+    assert runner.graph_replays == 0 if not graphs else (runner.graph_replays == 6 if n_live <= 64 else runner.graph_replays < 6)
+    runner.pages.audit()
+    assert runner.pages.live_requests() == 0 and runner.pages.free_pages(0) == n_live
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["whole", "portions", "mixed"])
+def test_long_spans_that_look_pages_up_in_the_block_table(mode):
+    """The kernel for long spans keeps the page ids of the keys a workgroup walks in LDS when
+    they are at most 2,048, else it looks each up in the block table.  With that limit lowered to
+    two, every long span here (up to nine pages of 16 tokens) goes the second way."""
+    ops = ops_for("cuda:0")
+    cfg, weights, reqs, want = setup("C", "bfloat16")
+    steps = {"whole": C.trace_whole, "portions": C.trace_portions, "mixed": C.trace_mixed}[mode](reqs)
+    runner = C.make_runner(cfg, weights, "bfloat16", "cuda:0", ops, 16, C.pages_needed(steps, reqs, 16))
+    kept = ops.long_span_pages_in_lds
+    ops.long_span_pages_in_lds = 2
+    try:
+        got, _ = C.run_trace(runner, steps)
+    finally:
+        ops.long_span_pages_in_lds = kept
+    C.assert_matches(got, want, True, f"page ids from the block table/{mode}")
+
+
+@pytest.mark.gpu
+def test_full_width_replay_eight_layers_float32(capsys):
+    """The widths of the 8B shape at a quarter of its depth, true float32: the largest
+    difference from the plain implementation over whole prompts and over single tokens stays
+    under 1e-4 (it is printed: run with -s to see it)."""
+    cfg = dict(FULL_WIDTH, num_hidden_layers=8)
+    weights = P.random_weights(cfg, seed=9)
+    reqs = C.make_requests(cfg, [45, 18], seed=12)
+    want = C.plain_logits(cfg, weights, reqs, False)
+    worst = 0.0
+    for mode, make in (("whole", C.trace_whole), ("tail", lambda r: C.trace_tail(r, tail=6))):
+        steps = make(reqs)
+        runner = C.make_runner(cfg, weights, "float32", "cuda:0", ops_for("cuda:0"), 64, C.pages_needed(steps, reqs, 64))
+        got, _ = C.run_trace(runner, steps)
+        worst = max(worst, max((got[r] - want[r]).abs().max().item() for r in reqs))
+        C.assert_matches(got, want, False, f"full width, 8 layers/{mode}", f32_tol=1e-4)
+        del runner
+    # how much of that is the engine's and how much the plain implementation's own float32
+    # rounding: both against the plain implementation in float64 (not asserted: for the record)
+    exact = {r: P.forward(cfg, weights, t, dtype=torch.float64).float() for r, t in reqs.items()}
+    ours = max((got[r] - exact[r]).abs().max().item() for r in reqs)
+    theirs = max((want[r] - exact[r]).abs().max().item() for r in reqs)
+    with capsys.disabled():
+        print(f"\n[full width, 8 layers, float32] largest difference from the plain implementation: {worst:.3e} (bound 1e-4); "
+              f"from its float64 form: engine {ours:.3e}, plain float32 {theirs:.3e}")

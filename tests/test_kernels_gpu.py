@@ -159,12 +159,19 @@ def test_gemm_mfma_skinny(ops, m, n, k, od):
         close(got, want, 1e-2, 2**-8)
 
 
-@pytest.mark.parametrize("chunk", ["128", "256"])
-def test_gemm_mfma_skinny_chunk_lengths(ops, chunk, monkeypatch):
+@pytest.fixture
+def forced(ops):
+    """``forced(chunk=, waves=, slices=)`` forces the few-row product's plan for one test."""
+    yield ops.force_skinny_plan
+    ops.force_skinny_plan()
+
+
+@pytest.mark.parametrize("chunk", [128, 256])
+def test_gemm_mfma_skinny_chunk_lengths(ops, chunk, forced):
     """The few-row product walks K in chunks of 256 or 128, chosen by the length of a
     workgroup's slice; here each length is forced in turn on every row-tile count, on split
     and unsplit products, on K that is no multiple of the chunk, and on the fused activation."""
-    monkeypatch.setenv("YALIS_SKINNY_CHUNK", chunk)
+    forced(chunk=chunk)
     for m, n, k in [(8, 200, 4096), (3, 515, 200), (24, 130, 2056), (40, 96, 1000), (64, 520, 328), (100, 64, 4096)]:
         x = rnd((m, k), torch.bfloat16, 6)
         w = rnd((n, k), torch.bfloat16, 7)
@@ -174,6 +181,26 @@ def test_gemm_mfma_skinny_chunk_lengths(ops, chunk, monkeypatch):
         packed, group = ops.pack_gate_up(rnd((inter, k), torch.bfloat16, 31, 0.05), rnd((inter, k), torch.bfloat16, 32, 0.05))
         got = ops.gate_up_act(x, packed, group, "silu", torch.bfloat16)
         assert torch.equal(got, ops.gated_act(ops.linear(x, packed, torch.bfloat16), "silu", torch.bfloat16, group=group))
+
+
+def test_forced_slice_counts_reach_the_consumers(ops, forced):
+    """The number of K slices a product leaves behind is what the launch says it wrote, also
+    when the plan is forced after the library was first asked about the shape."""
+    from yalis_amd.ops.hip import SplitSum
+
+    x, w = rnd((8, 4096), torch.bfloat16, 61), rnd((520, 4096), torch.bfloat16, 62)
+    want = x.double().cpu() @ w.double().cpu().T
+    auto = ops.linear(x, w, torch.bfloat16, partial_ok=True)
+    for slices in (1, 3, 16):
+        forced(slices=slices)
+        y = ops.linear(x, w, torch.bfloat16, partial_ok=True)
+        assert (y.n_splits if isinstance(y, SplitSum) else 1) == slices
+        close(y.reduce() if isinstance(y, SplitSum) else y, want, 2e-2, 2**-7)
+    forced()
+    again = ops.linear(x, w, torch.bfloat16, partial_ok=True)
+    assert (again.n_splits if isinstance(again, SplitSum) else 1) == (auto.n_splits if isinstance(auto, SplitSum) else 1)
+    with pytest.raises(Exception, match="128 or 256"):
+        forced(chunk=100)
 
 
 def test_gemm_mfma_operand_order(ops):

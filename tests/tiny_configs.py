@@ -113,4 +113,30 @@ TINY_E = {
     "tie_word_embeddings": True,
 }
 
-ALL = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
+# Three query heads on each of two kv heads at head size 128 (the head layout of Llama-3.2-3B):
+# with pages of 64 tokens the matrix-core attention runs over tiled pages with tiles of
+# 5 tokens x 3 heads, one column of every wave standing for nothing.
+TINY_F = {
+    "architectures": ["LlamaForCausalLM"],
+    "model_type": "llama",
+    "hidden_size": 264,
+    "num_hidden_layers": 2,
+    "num_attention_heads": 6,
+    "num_key_value_heads": 2,
+    "head_dim": 128,
+    "intermediate_size": 392,
+    "vocab_size": 777,
+    "rms_norm_eps": 2e-6,
+    "rope_theta": 500000.0,
+    "rope_scaling": {
+        "rope_type": "llama3",
+        "factor": 32.0,
+        "low_freq_factor": 1.0,
+        "high_freq_factor": 4.0,
+        "original_max_position_embeddings": 96,
+    },
+    "max_position_embeddings": 768,
+    "tie_word_embeddings": True,
+}
+
+ALL = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "F": TINY_F}

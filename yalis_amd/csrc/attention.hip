@@ -654,7 +654,7 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ block_table, int table_width,
     int page_size, int n_heads, int n_kv, int hpt, int chunks, float scale_log2, int window,
-    int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml) {
+    int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml, int pages_lds_limit) {
   constexpr int KS = D / 32, DT = D / 16;
   constexpr int KROW = D + 8;   // bf16 elements per parked key row
   constexpr int VROW = 64 + 8;  // bf16 elements per parked value row
@@ -700,7 +700,8 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
   constexpr int PAGES_LDS = 2048;
   __shared__ int32_t pages_s[PAGES_LDS];
   const int first_col = min(last_page_col, max(0, kb_lo) * 64 / page_size);
-  const bool pages_in_lds = last_page_col - first_col < PAGES_LDS;
+  // (pages_lds_limit: at most PAGES_LDS; tests lower it to walk the other way with short tables)
+  const bool pages_in_lds = last_page_col - first_col < min(PAGES_LDS, pages_lds_limit);
   if (pages_in_lds)
     for (int c = first_col + threadIdx.x; c <= last_page_col; c += 256) pages_s[c - first_col] = max(0, bt[c]);
   const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
@@ -979,12 +980,14 @@ extern "C" size_t yk_attn_mfma_workspace(int n_tiles, int n_heads, int n_kv, int
 }
 
 // Long spans: ``tiles`` hold up to yk_attn_long_tile_tokens tokens each (one workgroup a tile).
+// pages_lds_limit: a workgroup keeps the page ids of the keys it walks in LDS when they are fewer
+// than this (and than the kernel's own 2,048), else it looks each up in the block table.
 extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, const void* k_cache,
                                     const void* v_cache, const int32_t* tiles, int n_tiles,
                                     const int32_t* block_table, int table_width, int page_size,
                                     int head_dim, int n_heads, int n_kv, float scale, int window,
                                     int n_splits, int col_tiles, float* workspace, size_t workspace_floats,
-                                    hipStream_t stream) {
+                                    int pages_lds_limit, hipStream_t stream) {
   YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_mfma_prefill: bad head counts");
   YK_REQUIRE(col_tiles == 1 || col_tiles == 2, "attn_mfma_prefill: a wave has 1 or 2 column tiles");
   YK_REQUIRE(yk_attn_mfma_supported(head_dim), "attn_mfma_prefill: head_dim must be 64 or 128");
@@ -1011,12 +1014,12 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
     attn_mfma_prefill_kernel<DD, BIP, 1><<<grid, block, 0, stream>>>(                                            \
       static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),   \
       static_cast<const bf16_t*>(v_cache), tiles, block_table, table_width, page_size, n_heads, n_kv, hpt, chunks, \
-      scale_log2, window, n_splits, ws_o, ws_ml);                                                                \
+      scale_log2, window, n_splits, ws_o, ws_ml, pages_lds_limit);                                               \
   else                                                                                                       \
     attn_mfma_prefill_kernel<DD, BIP, 2><<<grid, block, 0, stream>>>(                                            \
       static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),   \
       static_cast<const bf16_t*>(v_cache), tiles, block_table, table_width, page_size, n_heads, n_kv, hpt, chunks, \
-      scale_log2, window, n_splits, ws_o, ws_ml)
+      scale_log2, window, n_splits, ws_o, ws_ml, pages_lds_limit)
   const bool bip = cache_is_tiled(YK_BF16, head_dim, page_size);
   if (head_dim == 64) {
     if (bip) { YK_PF(64, true); } else { YK_PF(64, false); }

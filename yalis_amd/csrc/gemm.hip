@@ -14,8 +14,6 @@
 // The reference runs these products through nn.Linear / cuBLAS
 // (yalis/external/model.py:63-65, 449, 462-466, 717-722).
 #include <algorithm>
-#include <cstdio>
-#include <cstdlib>
 
 #include "common.h"
 
@@ -149,11 +147,11 @@ static size_t skinny_lds_bytes(int mt, int waves, int kc) {
 // but gate/up 40.2 / 46.6; the 70B shape's decode step at 64 rows (slices of 2,048 to 8,192):
 // 36.9 / 37.7 ms, and its o-proj at 8 rows (slices of 2,048) is faster with long chunks too.  So:
 // short chunks for slices of up to 1,792, up to 4,096 with 64 rows of x.
+// What yk_gemm_skinny_force set (0: the library decides): for tests and measurements only.
+static int g_force_chunk = 0, g_force_waves = 0, g_force_slices = 0;
+
 static int skinny_chunk(int mt, int k_block) {
-  if (const char* force = getenv("YALIS_SKINNY_CHUNK")) {  // 128 or 256: for measurements
-    const int kc = atoi(force);
-    if (kc == 128 || kc == 256) return kc;
-  }
+  if (g_force_chunk) return g_force_chunk;
   return k_block <= (mt == 4 ? 16 : 7) * SK_KC ? 128 : SK_KC;
 }
 
@@ -439,17 +437,26 @@ static int skinny_plan(int M, int N, int K, bool gated, int* waves_out, int* k_b
       }
     }
   }
-  if (const char* force = getenv("YALIS_SKINNY_PLAN")) {  // "waves,slices": for measurements
-    int fw = 0, fs = 0;
-    if (sscanf(force, "%d,%d", &fw, &fs) == 2 && (fw == 4 || fw == 8) && fs >= 1) {
-      best_w = fw;
-      best_s = std::min<long>(fs, chunks);
-    }
-  }
+  if (g_force_waves) best_w = g_force_waves;
+  if (g_force_slices) best_s = std::min<long>(g_force_slices, chunks);
   int k_block = static_cast<int>((chunks + best_s - 1) / best_s) * SK_KC;
   if (waves_out) *waves_out = best_w;
   if (k_block_out) *k_block_out = k_block;
   return static_cast<int>((K + k_block - 1) / k_block);
+}
+
+// For tests and measurements: force the few-row product's chunk length (128 or 256), its waves a
+// workgroup (4) and its number of K slices; 0 leaves a choice to the library.  Process-wide:
+// set it before the products it is meant for and clear it after (a caller that remembers
+// yk_gemm_skinny_splits must ask again).
+extern "C" int yk_gemm_skinny_force(int chunk, int waves, int slices) {
+  YK_REQUIRE(chunk == 0 || chunk == 128 || chunk == 256, "gemm_skinny_force: chunks are 128 or 256 long");
+  YK_REQUIRE(waves == 0 || waves == 4, "gemm_skinny_force: a workgroup has 4 waves");
+  YK_REQUIRE(slices >= 0, "gemm_skinny_force: bad slice count");
+  g_force_chunk = chunk;
+  g_force_waves = waves;
+  g_force_slices = slices;
+  return 0;
 }
 
 // gated != 0: the plan of a product with the activation in its epilogue (1: it can be fused).

@@ -16,9 +16,12 @@ from ..config.reader import read_config_json
 from ..config.runtime import EngineConfig, InferenceConfig, ModelConfig
 from ..sampling.sampler import Sampler, SamplingParams
 from .factory import load_runner, random_runner
+from ..utils.logger import get_logger, gpu_memory_info
 from ..utils.timers import Timers
 from .scheduler import Request, Scheduled, Scheduler
-from .step import StepEntry
+from .step import ModelRunner, StepEntry
+
+logger = get_logger("engine")
 
 
 def print_rank0(*args, **kwargs) -> None:
@@ -35,37 +38,65 @@ class LLMEngine:
         engine_config: Optional[EngineConfig] = None,
         random_weights_seed: Optional[int] = None,
         ops=None,
+        config_dict: Optional[dict] = None,
     ):
         """``engine_config`` sizes the paged engine; by default it is derived from the
         inference configuration: ``max_batch_size`` live requests of
         ``max_length_of_generated_sequences`` tokens each (the reference's meaning of
         that option: the longest sequence, prompt included, yalis/engine.py:353-368).
         ``random_weights_seed``: ignore the folder's weights and make random ones
-        (config.json is still read)."""
+        (config.json is still read).  ``config_dict``: the configuration itself instead of a
+        folder's config.json (``model_config`` may then be None: see ``from_random``)."""
         self.model_config = model_config
         self.inference_config = inference_config
         dev = "cuda:0" if device == "cuda" else device
-        raw = read_config_json(model_config.model_path)
+        if config_dict is not None:
+            raw = dict(config_dict)
+            if random_weights_seed is None:
+                raise ValueError("a configuration without a folder has no weights: give random_weights_seed")
+        else:
+            raw = read_config_json(model_config.model_path)
         if engine_config is None:
             max_len = min(inference_config.max_length, int(raw.get("max_position_embeddings", inference_config.max_length)))
             engine_config = EngineConfig(
                 max_num_seqs=inference_config.max_batch_size,
                 max_model_len=max_len,
                 max_num_batched_tokens=max(2048, inference_config.max_batch_size),
-                dtype=model_config.dtype,
+                dtype=model_config.dtype if model_config is not None else "bfloat16",
                 device=dev,
             )
         self.engine_config = engine_config
         if random_weights_seed is None:
-            self.runner = load_runner(model_config.model_path, engine_config, ops=ops)
+            self.runner = load_runner(model_config.model_path, engine_config, ops=ops, progress=logger.debug)
         else:
             self.runner = random_runner(raw, engine_config, random_weights_seed, ops=ops)
+        # the reference reports memory at the same two places (yalis/engine.py:214, 250); here the
+        # pool is made together with the model's runner
+        logger.info("Memory Stats after Initializing Model and KV Cache - (allocated, reserved) GiB = (%.2f, %.2f)", *gpu_memory_info())
         self.model = self.runner.model
         self.sampler = Sampler(self.runner.rt.ops, engine_config.device)
         self.eos_token_ids = tuple(self.model.spec.eos_token_ids)
-        self.tokenizer = self._load_tokenizer(model_config.model_path)
+        self.tokenizer = self._load_tokenizer(model_config.model_path) if model_config is not None else None
         self.last_scheduler: Optional[Scheduler] = None
         self.last_timers: Optional[Timers] = None
+        self._next_request_id = 0  # request ids never repeat over the engine's life
+
+    @classmethod
+    def from_random(cls, config_dict: dict, inference_config: InferenceConfig, precision: str = "bf16", seed: int = 0,
+                    device: str = "cuda", engine_config: Optional[EngineConfig] = None, ops=None) -> "LLMEngine":
+        """An engine over random weights of the architecture and sizes that ``config_dict``
+        (the keys of a config.json) names; no folder is read or written."""
+        from ..config.runtime import canonical_dtype
+
+        if engine_config is None:
+            max_len = min(inference_config.max_length, int(config_dict.get("max_position_embeddings", inference_config.max_length)))
+            engine_config = EngineConfig(
+                max_num_seqs=inference_config.max_batch_size, max_model_len=max_len,
+                max_num_batched_tokens=max(2048, inference_config.max_batch_size),
+                dtype=canonical_dtype(precision), device="cuda:0" if device == "cuda" else device,
+            )
+        return cls(None, inference_config, device=device, engine_config=engine_config, random_weights_seed=seed, ops=ops,
+                   config_dict=config_dict)
 
     # --------------------------------------------------------------- tokenizer
     @staticmethod
@@ -90,7 +121,13 @@ class LLMEngine:
             if self.tokenizer is None:
                 raise ValueError("text prompts need a tokenizer in the model folder; give lists of token ids instead")
             return [self.tokenizer(p)["input_ids"] for p in prompts]
-        return [[int(t) for t in p] for p in prompts]
+        ids = [[int(t) for t in p] for p in prompts]
+        vocab = self.model.spec.vocab_size
+        for i, p in enumerate(ids):
+            bad = [t for t in p if not 0 <= t < vocab]
+            if bad:
+                raise ValueError(f"prompt {i}: token id {bad[0]} is outside the vocabulary of {vocab}")
+        return ids
 
     # ----------------------------------------------------------------- generate
     @torch.inference_mode()
@@ -122,7 +159,7 @@ class LLMEngine:
         if len(ids) > ic.max_batch_size:
             # yalis/engine.py:347-352
             raise ValueError(f"Batch size {len(ids)} exceeds max_batch_size {ic.max_batch_size}")
-        sched = Scheduler(self.runner, self.eos_token_ids)
+        sched = Scheduler(self.runner, self.eos_token_ids, first_request_id=self._next_request_id)
         self.last_scheduler = sched
         reqs: List[Request] = []
         for i, p in enumerate(ids):
@@ -161,6 +198,7 @@ class LLMEngine:
                 torch.cuda.nvtx.range_pop()
             timers.stop(name)
 
+        self._next_request_id = sched.next_request_id
         sync()
         t0 = time.perf_counter()
         m0 = mark()
@@ -168,6 +206,22 @@ class LLMEngine:
         first_token_at: Dict[int, object] = {}
         decode_steps = 0
         decode_spans = []  # (mark before, mark after, steps)
+        steps_ahead = 0
+        try:
+            steps_ahead = self._run(sched, get_logits, enable_nvtx, mark, open_range, close_range, first_token_at, decode_spans)
+        except BaseException:
+            # whatever stopped the loop (a bad input, an interrupt), the engine stays usable:
+            # every request of this call gives its pages and slot back
+            sched.abort_all()
+            raise
+        timers.stop("generate")
+        sync()
+        total = time.perf_counter() - t0
+        return self._finish(sched, reqs, ids, total, tokenize_ms, m0, seconds, first_token_at, decode_spans, steps_ahead,
+                            report_throughput, get_logits)
+
+    def _run(self, sched, get_logits, enable_nvtx, mark, open_range, close_range, first_token_at, decode_spans) -> int:
+        """The step loop of ``generate``; returns how many steps were launched ahead."""
         steps_ahead = 0
         while sched.has_work():
             before = mark()
@@ -226,9 +280,11 @@ class LLMEngine:
                     at += len(p)
                 continue
             sched.update(plan, toks.tolist() if toks is not None else [])
-        timers.stop("generate")
-        sync()
-        total = time.perf_counter() - t0
+        return steps_ahead
+
+    def _finish(self, sched, reqs, ids, total, tokenize_ms, m0, seconds, first_token_at, decode_spans, steps_ahead,
+                report_throughput, get_logits):
+        """Tokens, the metrics dictionary and (asked for) the logits of a finished call."""
         decode_steps = sum(n for _, _, n in decode_spans)
         decode_time = sum(seconds(a, b) for a, b, _ in decode_spans)
 
@@ -269,7 +325,26 @@ class LLMEngine:
         return out, metrics
 
     def reset_kv_cache(self, max_batch_size: Optional[int] = None) -> None:
-        """yalis/engine.py:280-304 rebuilds the caches; pages here are given back when
-        requests end, so there is nothing to rebuild unless the batch limit changes."""
-        if max_batch_size is not None and max_batch_size != self.inference_config.max_batch_size:
-            raise ValueError("the number of live requests is fixed when the engine is built")
+        """Rebuild the cache for ``max_batch_size`` live requests, as yalis/engine.py:280-304
+        does: a new pool of pages (sized as before per request), new block tables and state
+        slots, captured decode graphs dropped; the weights stay.  Without an argument, or with
+        the current size, only what requests hold is given back (nothing should be live between
+        calls of ``generate``)."""
+        runner = self.runner
+        for rid in list(runner.cached):
+            runner.release(rid)
+        if max_batch_size is None or max_batch_size == runner.config.max_num_seqs:
+            return
+        if max_batch_size <= 0:
+            raise ValueError("max_batch_size must be a positive integer.")
+        import dataclasses
+
+        old = runner.config
+        pages = None if old.num_pages is None else max(1, old.num_pages * max_batch_size // old.max_num_seqs)
+        new_config = dataclasses.replace(old, max_num_seqs=max_batch_size, num_pages=pages)
+        self.runner = None
+        del runner  # the old pool is freed before the new one is made
+        self.runner = ModelRunner(self.model, new_config)
+        self.engine_config = new_config
+        self.inference_config.max_batch_size = max_batch_size
+        logger.info("Memory Stats after KV Cache Init - (allocated, reserved) GiB = (%.2f, %.2f)", *gpu_memory_info())

@@ -61,21 +61,43 @@ class Scheduled:
 
 
 class Scheduler:
-    def __init__(self, runner: ModelRunner, eos_token_ids: Sequence[int] = ()):
+    def __init__(self, runner: ModelRunner, eos_token_ids: Sequence[int] = (), first_request_id: int = 0):
+        """``first_request_id``: where this scheduler's request ids start (a caller that makes a
+        scheduler per call over one runner passes ``next_request_id`` of the one before, so that
+        an id never names two requests of the runner)."""
         self.runner = runner
         self.cfg = runner.config
         self.eos = set(eos_token_ids)
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []
         self.finished: List[Request] = []
-        self._next_rid = 0
+        self._next_rid = int(first_request_id)
         self.n_preemptions = 0
+
+    @property
+    def next_request_id(self) -> int:
+        return self._next_rid
+
+    def abort_all(self) -> None:
+        """Give back what every request of this scheduler holds (after a failure mid-way):
+        running requests release their pages and slot, waiting ones are dropped."""
+        for req in list(self.running):
+            if self.runner.is_live(req.rid):
+                self.runner.release(req.rid)
+            req.state = FINISHED
+            req.finish_reason = "aborted"
+        self.running.clear()
+        self.waiting.clear()
 
     # ------------------------------------------------------------------- intake
     def add(self, prompt: Sequence[int], params: SamplingParams) -> Request:
         prompt = [int(t) for t in prompt]
         if not prompt:
             raise ValueError("a prompt needs at least one token")
+        vocab = self.runner.model.spec.vocab_size
+        for t in prompt:
+            if not 0 <= t < vocab:
+                raise ValueError(f"token id {t} is outside the vocabulary of {vocab}")
         if len(prompt) >= self.cfg.max_model_len:
             raise ValueError(
                 f"prompt of {len(prompt)} tokens leaves no room to generate within max_model_len={self.cfg.max_model_len}"

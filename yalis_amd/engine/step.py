@@ -286,7 +286,10 @@ class ModelRunner:
             self._feed_tokens(ints, layout, len(spans), token_source, token_index is not None)
             ctx = StepContext(hb, self._views(ints, layout), self.sites, self.rt)
             ops = self.rt.ops
-            ops.reserve_workspaces(hb.n_seqs)
+            # every weight matrix a part holds, as (rows, columns): the products of the step
+            products = sorted({tuple(t.shape) for p in self.model.all_parts() for t in vars(p).values()
+                               if isinstance(t, torch.Tensor) and t.dim() == 2})
+            ops.reserve_workspaces(hb.n_seqs, products)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):

@@ -26,7 +26,9 @@ DEFAULT_PROMPTS = [
 
 def parse_args(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--model", "--model-path", dest="model_path", required=True, help="folder with config.json, model.safetensors (and a tokenizer for text prompts)")
+    ap.add_argument("--model", "--model-path", dest="model_path", default=None, help="folder with config.json, model.safetensors (and a tokenizer for text prompts)")
+    ap.add_argument("--random", dest="random_shape", default=None, metavar="SHAPE",
+                    help="no folder: random weights (seed: --random-weights-seed, default 0) of a named shape: 8b, 3b, 70b, tiny-a, tiny-b")
     ap.add_argument("--model-name", default=None)
     ap.add_argument("--precision", "--dtype", dest="precision", default="bf16", choices=["bf16", "fp32", "bfloat16", "float32"])
     ap.add_argument("--prompt", action="append", default=[], help="a text prompt (repeatable; needs a tokenizer)")
@@ -50,7 +52,10 @@ def parse_args(argv=None):
     ap.add_argument("--page-size", type=int, default=64)
     ap.add_argument("--num-pages", type=int, default=None)
     ap.add_argument("--max-num-batched-tokens", "--max-batched-tokens", dest="max_num_batched_tokens", type=int, default=2048)
-    return ap.parse_args(argv)
+    args = ap.parse_args(argv)
+    if (args.model_path is None) == (args.random_shape is None):
+        ap.error("give either --model DIR or --random SHAPE")
+    return args
 
 
 def main(argv=None) -> int:
@@ -59,7 +64,8 @@ def main(argv=None) -> int:
     from yalis_amd.config.reader import read_config_json
     from yalis_amd.config.runtime import EngineConfig
 
-    model_config = ModelConfig(model_name=args.model_name, model_path=args.model_path, precision=args.precision)
+    from yalis_amd.config.runtime import canonical_dtype
+
     inference_config = InferenceConfig(
         max_batch_size=args.max_batch_size,
         max_length_of_generated_sequences=args.max_length_of_generated_sequences,
@@ -68,16 +74,28 @@ def main(argv=None) -> int:
         temperature=args.temperature,
         seed=args.seed,
     )
-    raw = read_config_json(args.model_path)
+    if args.random_shape is not None:
+        from yalis_amd.models.presets import shape
+
+        label, raw = shape(args.random_shape)
+        model_config = None
+        print_rank0(f"Model = random weights of the {label} shape")
+    else:
+        model_config = ModelConfig(model_name=args.model_name, model_path=args.model_path, precision=args.precision)
+        raw = read_config_json(args.model_path)
     engine_config = EngineConfig(
         page_size=args.page_size,
         num_pages=args.num_pages,
         max_num_seqs=args.max_batch_size,
         max_model_len=min(args.max_length_of_generated_sequences, int(raw.get("max_position_embeddings", 1 << 30))),
         max_num_batched_tokens=args.max_num_batched_tokens,
-        dtype=model_config.dtype,
+        dtype=canonical_dtype(args.precision),
     )
-    engine = LLMEngine(model_config, inference_config, engine_config=engine_config, random_weights_seed=args.random_weights_seed)
+    if model_config is None:
+        engine = LLMEngine.from_random(raw, inference_config, precision=args.precision, seed=args.random_weights_seed or 0,
+                                       engine_config=engine_config)
+    else:
+        engine = LLMEngine(model_config, inference_config, engine_config=engine_config, random_weights_seed=args.random_weights_seed)
 
     prompts: List = []
     if args.prompt_ids:
@@ -94,6 +112,11 @@ def main(argv=None) -> int:
         prompts = [[int(t) for t in ln.split(",")] for ln in lines] if as_ids else lines
     elif args.prompt:
         prompts = list(args.prompt)
+    elif engine.tokenizer is None:
+        # nothing to tokenize text with: a few seeded random prompts instead of the built-in texts
+        g = torch.Generator().manual_seed(args.seed)
+        vocab = engine.model.spec.vocab_size
+        prompts = [torch.randint(0, vocab, (16,), generator=g).tolist() for _ in range(min(4, args.max_batch_size))]
     else:
         prompts = DEFAULT_PROMPTS[: args.max_batch_size]
     if args.chat and prompts and isinstance(prompts[0], str):

@@ -59,6 +59,7 @@ _SIGNATURES = {
         _c_int,
     ),
     "yk_gemm_skinny_splits": ([_c_int, _c_int, _c_int, _c_int], _c_int),
+    "yk_gemm_skinny_force": ([_c_int, _c_int, _c_int], _c_int),
     "yk_gemm_mfma_skinny": (
         [_vp, _vp, _vp, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
         _c_int,
@@ -73,7 +74,7 @@ _SIGNATURES = {
     "yk_attn_tokens_per_tile": ([_c_int, _c_int], _c_int),
     "yk_attn_mfma_workspace": ([_c_int, _c_int, _c_int, _c_int, _c_int], _c_size_t),
     "yk_attn_mfma_prefill": (
-        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _vp],
+        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _c_int, _vp],
         _c_int,
     ),
     "yk_attn_mfma": (
@@ -106,7 +107,7 @@ _LATER_SIGNATURES = {
         "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
     },
 }
-_ABI = 10
+_ABI = 11
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
 # above it the vendor library does.
@@ -220,6 +221,9 @@ class HipOps:
         self._workspace: Optional[torch.Tensor] = None  # attention splits, argmax parts
         self._gemm_workspace: Optional[torch.Tensor] = None  # K slices of products
         self._mm_f32: Optional[bool] = None  # see _library_f32_out
+        # page ids a workgroup of the long-span attention keeps in LDS (more: looked up in the
+        # block table one by one); tests lower it to walk that path with short tables
+        self.long_span_pages_in_lds = 2048
 
     # ------------------------------------------------------------------ helpers
     @staticmethod
@@ -250,22 +254,42 @@ class HipOps:
         if rc != 0:
             raise KernelError((lib or self.lib).yk_last_error().decode())
 
+    def _grown(self, have: Optional[torch.Tensor], floats: int) -> torch.Tensor:
+        if have is not None and have.numel() >= floats:
+            return have
+        if have is not None and torch.cuda.is_current_stream_capturing():
+            # kernels already recorded hold the old buffer's address
+            raise KernelError(f"a scratch buffer would have to grow to {floats} floats while a graph is being captured; "
+                              "reserve_workspaces() before the capture must ask for more")
+        return torch.empty(max(floats, 1 << 22), dtype=torch.float32, device=self.device)
+
     def _ws(self, floats: int) -> torch.Tensor:
         """Float32 scratch that grows and is reused (stream order keeps uses apart)."""
-        if self._workspace is None or self._workspace.numel() < floats:
-            self._workspace = torch.empty(max(floats, 1 << 22), dtype=torch.float32, device=self.device)
+        self._workspace = self._grown(self._workspace, floats)
         return self._workspace
 
     def _gemm_ws(self, floats: int) -> torch.Tensor:
-        if self._gemm_workspace is None or self._gemm_workspace.numel() < floats:
-            self._gemm_workspace = torch.empty(max(floats, 1 << 22), dtype=torch.float32, device=self.device)
+        self._gemm_workspace = self._grown(self._gemm_workspace, floats)
         return self._gemm_workspace
 
-    def reserve_workspaces(self, rows: int) -> None:
-        """Make the scratch buffers large enough for steps of ``rows`` tokens before a
-        graph is captured (a buffer must not be replaced while a capture is running)."""
+    def reserve_workspaces(self, rows: int, products=()) -> None:
+        """Make the scratch buffers large enough for steps of ``rows`` tokens before a graph is
+        captured (a buffer must not be replaced while a capture is running: that raises).
+        ``products``: the (n, k) of the weight matrices the step multiplies ``rows`` rows by; the
+        unreduced K slices of each take slices x rows x n floats."""
+        need = 1 << 24
+        if rows <= SKINNY_MAX_ROWS:
+            for n, k in products:
+                if k >= 8 and k % 8 == 0:
+                    need = max(need, self._ask("yk_gemm_skinny_splits", rows, n, k, 0) * rows * n)
         self._ws(1 << 24)
-        self._gemm_ws(1 << 24)
+        self._gemm_ws(need)
+
+    def force_skinny_plan(self, chunk: int = 0, waves: int = 0, slices: int = 0) -> None:
+        """For tests and measurements: force the few-row product's chunk length (128 / 256), waves a
+        workgroup and number of K slices (0: the library decides); call without arguments to clear."""
+        self._check(self.lib.yk_gemm_skinny_force(int(chunk), int(waves), int(slices)))
+        self._answers = {k: v for k, v in self._answers.items() if k[0] not in ("yk_gemm_skinny_splits", "yk_gemm_skinny_from_attention_ok")}
 
     def workspaces(self):
         """The scratch buffers in use, for whoever must keep them alive (a captured graph)."""
@@ -435,7 +459,7 @@ class HipOps:
         if rc < 0:
             raise KernelError(self.lib.yk_last_error().decode())
         if keep:
-            return SplitSum(ws[: splits * m * n].view(splits, m, n), out_dtype)
+            return SplitSum(ws[: rc * m * n].view(rc, m, n), out_dtype)  # rc: the slices the launch wrote
         return y
 
     def _library_f32_out(self) -> bool:
@@ -517,7 +541,7 @@ class HipOps:
         if rc < 0:
             raise KernelError(self.lib.yk_last_error().decode())
         if keep:
-            return SplitSum(ws[: splits * m * n].view(splits, m, n), out_dtype)
+            return SplitSum(ws[: rc * m * n].view(rc, m, n), out_dtype)  # rc: the slices the launch wrote
         return y
 
     # ------------------------------------------------- rotary + append to the cache
@@ -637,7 +661,7 @@ class HipOps:
                     qkv.data_ptr(), qkv.stride(0), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                     long_tiles.data_ptr(), n_long, bt.data_ptr(), bt.shape[1], page_size, head_dim,
                     n_heads, n_kv, float(scale), int(window), long_splits, int(long_col_tiles), _ptr(ws),
-                    0 if ws is None else ws.numel(),
+                    0 if ws is None else ws.numel(), int(self.long_span_pages_in_lds),
                     self._stream(),
                 )
             )

@@ -1,7 +1,7 @@
 """Loading a model's tensors by name.
 
 The parts of a model declare what they need (``TensorSpec`` by checkpoint name);
-``load_tensors`` reads exactly those from the folder and fails with ONE error that
+``open_tensors`` reads exactly those from the folder and fails with ONE error that
 lists every missing tensor, every unexpected tensor and every wrong shape (the
 reference gets the same from ``load_state_dict(strict=True)``,
 yalis/model_loading.py:201-249).
@@ -9,7 +9,11 @@ yalis/model_loading.py:201-249).
 Precision rule: a floating tensor stored in 16 bits is kept in bfloat16, a tensor
 stored in 32 bits stays in 32 bits (such tensors are stored wide because they need
 it), integer tables become int32.  In the 32-bit mode of the engine every floating
-tensor is widened to float32 (exact).
+tensor is widened to float32 (exact).  A checkpoint stored in float16 is refused by the
+bfloat16 engine: rounding it to bfloat16 would silently drop three bits of every weight (the
+reference runs such checkpoints in float16, a precision this engine does not have); the
+float32 engine takes it.  Matrices stored in 32 bits stay so in the bfloat16 engine, which
+then runs their products on the float32 kernels: that is said once, loudly, when it happens.
 """
 from __future__ import annotations
 
@@ -18,7 +22,10 @@ from typing import Callable, Dict, Mapping, Optional, Tuple
 
 import torch
 
+from ..utils.logger import get_logger
 from .safetensors_io import TensorEntry, index_folder, read_tensor
+
+logger = get_logger("weights")
 
 
 @dataclass(frozen=True)
@@ -73,7 +80,7 @@ def target_dtype(storage_tag: str, kind: str, engine_dtype: str) -> torch.dtype:
     return torch.bfloat16
 
 
-def check_against(entries: Dict[str, TensorEntry], wanted: Dict[str, TensorSpec], where: str) -> None:
+def check_against(entries: Dict[str, TensorEntry], wanted: Dict[str, TensorSpec], where: str, engine_dtype: Optional[str] = None) -> None:
     missing = [n for n in wanted if n not in entries]
     unexpected = [
         n for n in entries if n not in wanted and not n.endswith(IGNORED_SUFFIXES)
@@ -90,6 +97,8 @@ def check_against(entries: Dict[str, TensorEntry], wanted: Dict[str, TensorSpec]
             ok = tag in (_FLOAT_TAGS if s.kind == "float" else _INT_TAGS)
             if not ok:
                 wrong_kind.append((n, tag, s.kind))
+            elif tag == "F16" and engine_dtype == "bfloat16":
+                wrong_kind.append((n, tag, "bfloat16 or float32 (this engine has no float16; run it with precision fp32 or convert the checkpoint)"))
     if missing or unexpected or wrong_shape or wrong_kind:
         raise WeightsError(where, sorted(missing), sorted(unexpected), wrong_shape, wrong_kind)
 
@@ -134,7 +143,13 @@ def open_tensors(
     """Check the folder against ``wanted`` (the one error lists everything that is wrong)
     and return a source that reads each tensor onto ``device`` when it is asked for."""
     entries = index_folder(model_dir)
-    check_against(entries, wanted, model_dir)
+    check_against(entries, wanted, model_dir, engine_dtype)
+    if engine_dtype == "bfloat16":
+        wide = [n for n, sp in wanted.items() if sp.kind == "float" and len(sp.shape) >= 2 and entries[n].dtype in ("F32", "F64")]
+        if wide:
+            logger.warning(
+                "%d matrices of %s are stored in 32 bits and stay so: the bfloat16 engine runs their products on its "
+                "float32 kernels (twice the memory, far slower than the matrix cores); first: %s", len(wide), model_dir, wide[0])
     done = [0]
 
     def make(name: str) -> torch.Tensor:
@@ -147,25 +162,3 @@ def open_tensors(
         return t
 
     return TensorSource(uses, make)
-
-
-def load_tensors(
-    model_dir: str,
-    wanted: Dict[str, TensorSpec],
-    engine_dtype: str,
-    device: str,
-    progress: Optional[Callable[[str], None]] = None,
-) -> Dict[str, torch.Tensor]:
-    """Read ``wanted`` from the folder onto ``device``; see the module text for
-    the precision rule and the error."""
-    entries = index_folder(model_dir)
-    check_against(entries, wanted, model_dir)
-    out: Dict[str, torch.Tensor] = {}
-    for i, (name, spec) in enumerate(wanted.items()):
-        e = entries[name]
-        t = read_tensor(e)
-        dt = target_dtype(e.dtype, spec.kind, engine_dtype)
-        out[name] = t.to(device=device, dtype=dt).contiguous()
-        if progress is not None and i % 32 == 0:
-            progress(f"loaded {i + 1}/{len(wanted)} tensors")
-    return out
