@@ -11,6 +11,15 @@ function over the paged cache, greedy sampling.  As in ``LLMEngine.generate``, s
 no decision of the scheduler are launched one behind the other, each feeding on the tokens the
 step before left on the device; the tokens of all timed steps are on the host when the clock
 stops.
+
+Beside the headline the one JSON line holds: ``roofline`` (the bytes a decode step has to
+read, every weight once and the cache of the live requests, over its time, against 8 TB/s);
+``prefill`` (2,048 tokens, the mean of three timed runs, with its fraction of 2.5 PFLOP/s);
+``points``: decode at batch 1 and 64 with the same roofline fraction each, and mixed steps at
+the Llama-3.2-3B shape (32 decode streams beside 480-token portions of 4,096-token prompts)
+with their bound max(bytes / 8 TB/s, flops / 2.5 PFLOP/s); ``breakdown``: the time of a
+decode step and of the prefill by kind of work (products, attention, output head, norms),
+each with the fraction of the peak that bounds it.
 """
 import argparse
 import json
@@ -117,6 +126,231 @@ def sampling_times(vocab: int, batch: int) -> int:
     return 0
 
 
+class Shape:
+    """The sizes of a configuration that the byte and flop counts need."""
+
+    def __init__(self, cfg: dict):
+        self.c, self.h, self.g, self.d = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+        self.inter, self.vocab, self.layers = cfg["intermediate_size"], cfg["vocab_size"], cfg["num_hidden_layers"]
+        self.layer_params = self.c * (self.h + 2 * self.g) * self.d + self.h * self.d * self.c + 3 * self.c * self.inter
+        # every weight a decode step reads once: the layers, the norms, the output head (the
+        # embedding table itself when tied; of a separate table only a row per token is read)
+        self.weight_bytes = 2 * (self.layers * (self.layer_params + 2 * self.c) + self.c + self.vocab * self.c)
+        self.kv_bytes_per_token = self.layers * 2 * self.g * self.d * 2
+
+    def decode_bytes(self, batch: int, mean_ctx_tokens: float) -> float:
+        """What a decode step has to read: every weight once, the cache of the live requests."""
+        return self.weight_bytes + batch * self.c * 2 + mean_ctx_tokens * self.kv_bytes_per_token
+
+    def prefill_flops(self, t: int) -> float:
+        return self.layers * (2 * t * self.layer_params + 2 * self.h * self.d * t * t) + 2 * self.vocab * self.c
+
+
+def make_runner(cfg: dict, max_batch: int, ctx_cap: int, graphs: bool = True, page: int = 64):
+    from yalis_amd.config.runtime import EngineConfig
+    from yalis_amd.engine.factory import random_runner
+
+    pages_per_req = -(-ctx_cap // page)
+    engine = EngineConfig(
+        page_size=page, num_pages=pages_per_req * max_batch, max_num_seqs=max_batch,
+        max_model_len=min(cfg["max_position_embeddings"], pages_per_req * page),
+        max_num_batched_tokens=8192, dtype="bfloat16", decode_graphs=graphs,
+    )
+    return random_runner(cfg, engine, seed=0)
+
+
+def decode_run(runner, vocab: int, gen, batch: int, prompt_len: int, steps: int, warmup: int):
+    """Prefill ``batch`` prompts, then time ``steps`` decode steps launched one behind the other.
+    Returns (seconds, mean cached tokens read per step)."""
+    import torch
+
+    from yalis_amd.engine.step import StepEntry
+
+    ops = runner.rt.ops
+    toks = []
+    for r in range(batch):
+        assert runner.admit(r)
+        prompt = torch.randint(0, vocab, (prompt_len,), generator=gen).tolist()
+        assert runner.reserve(r, len(prompt))
+        toks.append(ops.argmax(runner.step([StepEntry(r, prompt, [len(prompt) - 1])])).tolist()[0])
+    for _ in range(warmup):
+        for r in range(batch):
+            assert runner.reserve(r, 1)
+        toks = ops.argmax(runner.step([StepEntry(r, [toks[r]], [0]) for r in range(batch)])).tolist()
+    entries = [StepEntry(r, [0], [0]) for r in range(batch)]
+    last = torch.tensor(toks, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ctx_sum, run = 0, []
+    for r in range(batch):
+        assert runner.reserve(r, steps)
+    for _ in range(steps):
+        ctx_sum += sum(runner.cached[r] + 1 for r in range(batch))
+        last = ops.argmax(runner.step(entries, token_source=last))
+        run.append(last)
+    torch.stack(run).tolist()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    for r in range(batch):
+        runner.release(r)
+    return dt, ctx_sum / steps
+
+
+def prefill_run(runner, vocab: int, gen, t: int, runs: int = 4):
+    """One request of ``t`` tokens, whole, ``runs`` times (the first warms up); the mean of the rest, in seconds."""
+    import torch
+
+    from yalis_amd.engine.step import StepEntry
+
+    ops = runner.rt.ops
+    prompt = torch.randint(0, vocab, (t,), generator=gen).tolist()
+    times = []
+    for i in range(runs):
+        assert runner.admit(1000 + i) and runner.reserve(1000 + i, t)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ops.argmax(runner.step([StepEntry(1000 + i, prompt, [t - 1])])).tolist()
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        runner.release(1000 + i)
+    return sum(times[1:]) / len(times[1:]), times
+
+
+def mixed_run(runner, shape: Shape, gen, prompt_len: int, portion: int, n_dec: int = 32, plen: int = 4096):
+    """``n_dec`` requests decode while ``plen``-token prompts arrive in portions: every step holds
+    ``n_dec`` single tokens and one portion (the last portion's row is sampled too).  The rows of
+    a step's products are the step's tokens: 480 + 32 = 512 rows fill the vendor library's tiles,
+    512 + 32 = 544 rows cost a fifth tile row for a quarter of its work.  Returns (ms a step,
+    the bound max(bytes / HBM, flops / matrix cores) in ms, steps timed)."""
+    import torch
+
+    from yalis_amd.engine.step import StepEntry
+
+    ops = runner.rt.ops
+    toks = []
+    for r in range(n_dec):
+        assert runner.admit(r)
+        prompt = torch.randint(0, shape.vocab, (prompt_len,), generator=gen).tolist()
+        assert runner.reserve(r, len(prompt))
+        toks.append(ops.argmax(runner.step([StepEntry(r, prompt, [len(prompt) - 1])])).tolist()[0])
+    prompt = torch.randint(0, shape.vocab, (plen,), generator=gen).tolist()
+    times, kv_tokens = [], []
+    for rid in (100, 101, 102):  # the first prompt warms up
+        assert runner.admit(rid)
+        for c0 in range(0, plen - portion + 1, portion):
+            for r in range(n_dec):
+                assert runner.reserve(r, 1)
+            assert runner.reserve(rid, portion)
+            last = c0 + 2 * portion > plen
+            entries = [StepEntry(r, [toks[r]], [0]) for r in range(n_dec)]
+            entries.append(StepEntry(rid, prompt[c0 : c0 + portion], [portion - 1] if last else []))
+            ctx_tokens = sum(runner.cached[r] + 1 for r in range(n_dec)) + c0 + portion
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            out = ops.argmax(runner.step(entries)).tolist()
+            torch.cuda.synchronize()
+            if rid != 100:
+                times.append(time.perf_counter() - t0)
+                kv_tokens.append(ctx_tokens)
+            toks = out[:n_dec]
+        runner.release(rid)
+    for r in range(n_dec):
+        runner.release(r)
+    ms = 1e3 * sum(times) / len(times)
+    n_tok = n_dec + portion
+    step_b = shape.weight_bytes + sum(kv_tokens) / len(kv_tokens) * shape.kv_bytes_per_token
+    # products over all tokens of the step; attention of the portion against the prompt so far
+    step_f = shape.layers * (2 * n_tok * shape.layer_params + 4 * shape.h * shape.d * portion * (plen / 2)) + 2 * (n_dec + 1 / 8) * shape.vocab * shape.c
+    bound_ms = 1e3 * max(step_b / (HBM_GBPS * 1e9), step_f / BF16_FLOPS)
+    return ms, bound_ms, len(times)
+
+
+def breakdown(runner, shape: Shape, gen, batch: int, prompt_len: int, prefill_len: int):
+    """Where a decode step's and a prefill's time goes, by kind of work, from device events
+    around every call into the kernel library (steps launched kernel by kernel for this: the
+    replayed graph of a decode step cannot be timed from inside).  Each kind comes with what
+    bounds it: products and the output head the bytes of their weights over the memory
+    bandwidth (decode) or their flops over the matrix cores' rate (prefill), attention the bytes
+    of the cached keys and values (decode) or its flops (prefill)."""
+    import torch
+
+    from yalis_amd.engine.step import StepEntry
+
+    ops = runner.rt.ops
+    kinds = {"linear": "products", "gate_up_act": "products", "gemm_mfma_skinny": None, "gemm_fma": None,
+             "attention": "attention", "rope_append": "attention", "add_rmsnorm": "norms", "gather_add_rmsnorm": "norms",
+             "gated_act": "activation", "embed": "other", "argmax": "other"}
+    spans, depth, head_rows = [], [0], shape.vocab
+
+    def timed(name, fn, kind):
+        def call(*a, **kw):
+            if depth[0]:  # a call made by a timed call belongs to it
+                return fn(*a, **kw)
+            k = kind
+            if name == "linear" and a[1].shape[0] == head_rows:
+                k = "head"
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            depth[0] += 1
+            start.record()
+            try:
+                return fn(*a, **kw)
+            finally:
+                stop.record()
+                depth[0] -= 1
+                spans.append((k, start, stop))
+        return call
+
+    saved = {}
+    for name, kind in kinds.items():
+        if kind is not None and hasattr(ops, name):
+            saved[name] = getattr(ops, name)
+            setattr(ops, name, timed(name, saved[name], kind))
+    graphs, runner.use_graphs = runner.use_graphs, False
+    out = {}
+    try:
+        toks = []
+        for r in range(batch):
+            assert runner.admit(r)
+            prompt = torch.randint(0, shape.vocab, (prompt_len,), generator=gen).tolist()
+            assert runner.reserve(r, len(prompt) + 8)
+            toks.append(ops.argmax(runner.step([StepEntry(r, prompt, [len(prompt) - 1])])).tolist()[0])
+        sums, n_steps = {}, 4
+        for i in range(n_steps + 2):
+            spans.clear()
+            toks = ops.argmax(runner.step([StepEntry(r, [toks[r]], [0]) for r in range(batch)])).tolist()
+            torch.cuda.synchronize()
+            if i >= 2:
+                for k, a, b in spans:
+                    sums[k] = sums.get(k, 0.0) + a.elapsed_time(b) * 1e3 / n_steps
+        ctx = sum(runner.cached[r] for r in range(batch))
+        for r in range(batch):
+            runner.release(r)
+        bytes_of = {"products": 2 * shape.layers * shape.layer_params, "attention": ctx * shape.kv_bytes_per_token, "head": 2 * shape.vocab * shape.c}
+        out["decode_us"] = {k: round(v, 1) for k, v in sorted(sums.items())}
+        out["decode_frac_of_hbm"] = {k: round(bytes_of[k] / (sums[k] * 1e-6) / (HBM_GBPS * 1e9), 3) for k in bytes_of if sums.get(k)}
+        # prefill
+        t = prefill_len
+        prompt = torch.randint(0, shape.vocab, (t,), generator=gen).tolist()
+        sums = {}
+        for i in range(3):
+            spans.clear()
+            assert runner.admit(2000 + i) and runner.reserve(2000 + i, t)
+            ops.argmax(runner.step([StepEntry(2000 + i, prompt, [t - 1])])).tolist()
+            torch.cuda.synchronize()
+            runner.release(2000 + i)
+            if i >= 1:
+                for k, a, b in spans:
+                    sums[k] = sums.get(k, 0.0) + a.elapsed_time(b) / 2
+        flops_of = {"products": 2 * t * shape.layers * shape.layer_params, "attention": 2 * shape.h * shape.d * t * t * shape.layers}
+        out["prefill_ms"] = {k: round(v, 3) for k, v in sorted(sums.items())}
+        out["prefill_frac_of_mfma"] = {k: round(flops_of[k] / (sums[k] * 1e-3) / BF16_FLOPS, 3) for k in flops_of if sums.get(k)}
+    finally:
+        runner.use_graphs = graphs
+        for name, fn in saved.items():
+            setattr(ops, name, fn)
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -126,7 +360,7 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=1024)
     ap.add_argument("--prefill-len", type=int, default=2048)
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    ap.add_argument("--no-points", action="store_true", help="the headline decode measurement only (no prefill, batch 1 / 64, breakdown, mixed steps)")
     ap.add_argument("--only-prefill", action="store_true", help="measure the prefill only (for profiling)")
     ap.add_argument("--mixed", action="store_true", help="measure mixed steps instead: 32 decode streams beside portions of 4,096-token prompts")
     ap.add_argument("--portion", type=int, default=480, help="tokens of a prompt portion in --mixed steps (with the 32 decoded tokens: 512 rows, as the scheduler cuts under a budget of 512)")
@@ -146,155 +380,41 @@ def main() -> int:
     if args.sample:
         return sampling_times(SHAPES[args.shape][1]["vocab_size"], args.batch)
 
-    from yalis_amd.config.runtime import EngineConfig
-    from yalis_amd.engine.factory import random_runner
-    from yalis_amd.engine.step import StepEntry
-
     shape_name, shape_cfg = SHAPES[args.shape]
     cfg = dict(shape_cfg)
     full_layers = cfg["num_hidden_layers"]
     if args.layers is not None:
         cfg["num_hidden_layers"] = args.layers
-    layers = cfg["num_hidden_layers"]
-    page = 64
-    max_batch = max(args.batch, 1 if args.no_points else 64)
-    total_steps = args.steps + args.warmup + 8
-    ctx_cap = max(args.prompt_len + total_steps + 1, args.prefill_len)
-    if args.mixed:
-        max_batch, ctx_cap = 34, 4096 + 64
-    pages_per_req = -(-ctx_cap // page)
-    engine = EngineConfig(
-        page_size=page,
-        num_pages=pages_per_req * max_batch,
-        max_num_seqs=max_batch,
-        max_model_len=min(cfg["max_position_embeddings"], pages_per_req * page),
-        max_num_batched_tokens=8192,
-        dtype="bfloat16",
-        decode_graphs=not args.no_graphs,
-    )
-    runner = random_runner(cfg, engine, seed=0)
-    ops = runner.rt.ops
-    vocab = cfg["vocab_size"]
+    shape = Shape(cfg)
     gen = torch.Generator().manual_seed(0)
 
-    def decode_run(batch: int, steps: int, warmup: int):
-        """Prefill ``batch`` prompts, then time ``steps`` decode steps."""
-        for r in range(batch):
-            assert runner.admit(r)
-            prompt = torch.randint(0, vocab, (args.prompt_len,), generator=gen).tolist()
-            assert runner.reserve(r, len(prompt))
-            logits = runner.step([StepEntry(r, prompt, [len(prompt) - 1])])
-            first = ops.argmax(logits).tolist()
-            if r == 0:
-                toks = []
-            toks.append(first[0])
-
-        def one_step(toks):
-            for r in range(batch):
-                assert runner.reserve(r, 1)
-            logits = runner.step([StepEntry(r, [toks[r]], [0]) for r in range(batch)])
-            return ops.argmax(logits).tolist()
-
-        for _ in range(warmup):
-            toks = one_step(toks)
-        entries = [StepEntry(r, [0], [0]) for r in range(batch)]
-        last = torch.tensor(toks, dtype=torch.int32, device="cuda")
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        ctx_sum = 0
-        run = []
-        for r in range(batch):
-            assert runner.reserve(r, steps)
-        for _ in range(steps):
-            ctx_sum += sum(runner.cached[r] + 1 for r in range(batch))
-            last = ops.argmax(runner.step(entries, token_source=last))
-            run.append(last)
-        toks = torch.stack(run).tolist()[-1]
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        for r in range(batch):
-            runner.release(r)
-        return dt, ctx_sum / steps  # seconds, mean cached tokens read per step
-
-    c, h, g, d, inter = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["intermediate_size"]
-    layer_params = c * (h + 2 * g) * d + h * d * c + 3 * c * inter
-    # every weight a decode step reads once: the layers, the final norm, the output head (the
-    # embedding table itself when tied; of a separate table only a row per token is read)
-    weight_bytes = 2 * (layers * (layer_params + 2 * c) + c + vocab * c)
-
-    def step_bytes(batch, mean_ctx_tokens):
-        kv = mean_ctx_tokens * layers * 2 * g * d * 2
-        return weight_bytes + batch * c * 2 + kv
-
     if args.mixed:
-        # 32 requests decode while 4,096-token prompts arrive in portions: every step holds 32
-        # single tokens and one portion (the last portion's row is sampled too).  The rows of a
-        # step's products are the step's tokens: 480 + 32 = 512 rows fill the vendor library's
-        # tiles, 512 + 32 = 544 rows cost a fifth tile row for a quarter of its work.
-        n_dec, portion, plen = 32, args.portion, 4096
-        toks = []
-        for r in range(n_dec):
-            assert runner.admit(r)
-            prompt = torch.randint(0, vocab, (args.prompt_len,), generator=gen).tolist()
-            assert runner.reserve(r, len(prompt))
-            toks.append(ops.argmax(runner.step([StepEntry(r, prompt, [len(prompt) - 1])])).tolist()[0])
-        prompt = torch.randint(0, vocab, (plen,), generator=gen).tolist()
-        times, kv_tokens = [], []
-        for rid in (100, 101, 102):  # the first prompt warms up
-            assert runner.admit(rid)
-            for c0 in range(0, plen - portion + 1, portion):
-                for r in range(n_dec):
-                    assert runner.reserve(r, 1)
-                assert runner.reserve(rid, portion)
-                last = c0 + 2 * portion > plen
-                entries = [StepEntry(r, [toks[r]], [0]) for r in range(n_dec)]
-                entries.append(StepEntry(rid, prompt[c0 : c0 + portion], [portion - 1] if last else []))
-                ctx_tokens = sum(runner.cached[r] + 1 for r in range(n_dec)) + c0 + portion
-                torch.cuda.synchronize()
-                t0 = time.perf_counter()
-                out = ops.argmax(runner.step(entries)).tolist()
-                torch.cuda.synchronize()
-                if rid != 100:
-                    times.append(time.perf_counter() - t0)
-                    kv_tokens.append(ctx_tokens)
-                toks = out[:n_dec]
-            runner.release(rid)
-        ms = 1e3 * sum(times) / len(times)
-        n_tok = n_dec + portion
-        mean_kv = sum(kv_tokens) / len(kv_tokens)
-        step_b = weight_bytes + mean_kv * layers * 2 * g * d * 2
-        # products over all tokens of the step; attention of the portion against the prompt so far
-        step_f = layers * (2 * n_tok * layer_params + 4 * h * d * portion * (plen / 2)) + 2 * (n_dec + 1 / 8) * vocab * c
-        bound_ms = 1e3 * max(step_b / (HBM_GBPS * 1e9), step_f / BF16_FLOPS)
+        runner = make_runner(cfg, 34, 4096 + 64, graphs=not args.no_graphs)
+        ms, bound_ms, n = mixed_run(runner, shape, gen, args.prompt_len, args.portion)
         print(json.dumps({
-            "metric": f"mixed steps ({shape_name} shape): {n_dec} decode streams beside {portion}-token portions of {plen:,}-token prompts",
-            "ms_per_step": round(ms, 3), "decode_tokens_per_s": round(n_dec / ms * 1e3, 1), "prefill_tokens_per_s": round(portion / ms * 1e3, 1),
-            "steps": len(times), "dtype": "bf16", "n_gpus": 1,
+            "metric": f"mixed steps ({shape_name} shape): 32 decode streams beside {args.portion}-token portions of 4,096-token prompts",
+            "ms_per_step": round(ms, 3), "decode_tokens_per_s": round(32 / ms * 1e3, 1), "prefill_tokens_per_s": round(args.portion / ms * 1e3, 1),
+            "steps": n, "dtype": "bf16", "n_gpus": 1,
             "roofline": {"bound": "max(hbm, mfma)", "bound_ms": round(bound_ms, 3), "frac": round(bound_ms / ms, 4)},
         }))
         return 0
 
+    max_batch = max(args.batch, 1 if args.no_points else 64)
+    total_steps = args.steps + args.warmup + 8
+    runner = make_runner(cfg, max_batch, max(args.prompt_len + total_steps + 1, args.prefill_len), graphs=not args.no_graphs)
+
     if args.only_prefill:
-        t = args.prefill_len
-        prompt = torch.randint(0, vocab, (t,), generator=gen).tolist()
-        for i in range(3):
-            assert runner.admit(1000 + i) and runner.reserve(1000 + i, t)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            ops.argmax(runner.step([StepEntry(1000 + i, prompt, [t - 1])])).tolist()
-            torch.cuda.synchronize()
-            print(f"prefill {t} tokens: {1e3 * (time.perf_counter() - t0):.3f} ms")
-            runner.release(1000 + i)
+        _, times = prefill_run(runner, shape.vocab, gen, args.prefill_len, runs=3)
+        for x in times:
+            print(f"prefill {args.prefill_len} tokens: {1e3 * x:.3f} ms")
         return 0
 
-    dt, mean_ctx = decode_run(args.batch, args.steps, args.warmup)
+    dt, mean_ctx = decode_run(runner, shape.vocab, gen, args.batch, args.prompt_len, args.steps, args.warmup)
     ms_per_step = 1e3 * dt / args.steps
-    value = args.batch * args.steps / dt
-    achieved = step_bytes(args.batch, mean_ctx) / (dt / args.steps) / 1e9
-
+    achieved = shape.decode_bytes(args.batch, mean_ctx) / (dt / args.steps) / 1e9
     result = {
         "metric": f"decode tok/s ({shape_name} shape, batch {args.batch}, {args.prompt_len:,}-token prompts)",
-        "value": round(value, 2),
+        "value": round(args.batch * args.steps / dt, 2),
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,
@@ -307,57 +427,49 @@ def main() -> int:
         "data": "synthetic: random N(0,0.02) bf16 weights, seeded uniform-random token ids",
         "config": {
             "model": f"{shape_name} shape",
-            "layers": layers,
+            "layers": shape.layers,
             "layers_of_full_model": full_layers,
-            "hidden_size": c,
-            "num_attention_heads": h,
-            "num_key_value_heads": g,
-            "head_dim": d,
-            "intermediate_size": inter,
-            "vocab_size": vocab,
+            "hidden_size": shape.c,
+            "num_attention_heads": shape.h,
+            "num_key_value_heads": shape.g,
+            "head_dim": shape.d,
+            "intermediate_size": shape.inter,
+            "vocab_size": shape.vocab,
             "global_batch": args.batch,
             "seq_len": args.prompt_len,
             "context": cfg["max_position_embeddings"],
-            "page_size": page,
+            "page_size": 64,
             "parallelism": "single GPU",
         },
-        "roofline": {
-            "bound": "hbm",
-            "achieved": round(achieved, 1),
-            "peak": HBM_GBPS,
-            "unit": "GB/s",
-            "frac": round(achieved / HBM_GBPS, 4),
-        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_GBPS, 4)},
     }
 
     if not args.no_points:
-        # prefill of one request of 2,048 tokens, whole
         t = args.prefill_len
-        prompt = torch.randint(0, vocab, (t,), generator=gen).tolist()
-        times = []
-        for i in range(3):
-            assert runner.admit(1000 + i)
-            assert runner.reserve(1000 + i, t)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            logits = runner.step([StepEntry(1000 + i, prompt, [t - 1])])
-            ops.argmax(logits).tolist()
-            torch.cuda.synchronize()
-            times.append(time.perf_counter() - t0)
-            runner.release(1000 + i)
-        pf = min(times[1:])
-        flops = layers * (2 * t * layer_params + 2 * h * d * t * t) + 2 * vocab * c
-        result["prefill"] = {
-            "value": round(t / pf, 1),
-            "tokens": t,
-            "ms": round(1e3 * pf, 3),
-            "frac": round(flops / pf / BF16_FLOPS, 4),
-        }
+        pf, _ = prefill_run(runner, shape.vocab, gen, t, runs=4)  # the mean of three timed runs
+        result["prefill"] = {"value": round(t / pf, 1), "tokens": t, "ms": round(1e3 * pf, 3),
+                             "frac": round(shape.prefill_flops(t) / pf / BF16_FLOPS, 4)}
         points = {}
         for b, name in ((1, "decode_b1"), (64, "decode_b64")):
             steps = max(8, args.steps // 2)
-            dtb, _ = decode_run(b, steps, 2)
+            dtb, ctx_b = decode_run(runner, shape.vocab, gen, b, args.prompt_len, steps, 2)
             points[name] = round(b * steps / dtb, 2)
+            # the same roofline as the headline: bytes the step has to read / its time / 8 TB/s
+            points[name + "_frac"] = round(shape.decode_bytes(b, ctx_b) / (dtb / steps) / (HBM_GBPS * 1e9), 4)
+        result["breakdown"] = breakdown(runner, shape, gen, args.batch, args.prompt_len, t)
+        del runner
+        torch.cuda.empty_cache()
+        # mixed steps at the Llama-3.2-3B shape: 32 decode streams beside 480-token portions of
+        # 4,096-token prompts (only with the headline's own shape and all its layers)
+        if args.shape == "8b" and args.layers is None:
+            name3, cfg3 = SHAPES["3b"]
+            shape3 = Shape(cfg3)
+            ms3, bound3, _ = mixed_run(make_runner(dict(cfg3), 34, 4096 + 64), shape3, gen, args.prompt_len, 480)
+            points["mixed_3b_ms_per_step"] = round(ms3, 3)
+            points["mixed_3b_decode_tok_s"] = round(32 / ms3 * 1e3, 1)
+            points["mixed_3b_prefill_tok_s"] = round(480 / ms3 * 1e3, 1)
+            points["mixed_3b_bound_ms"] = round(bound3, 3)  # max(bytes / 8 TB/s, flops / 2.5 PFLOP/s)
+            points["mixed_3b_frac"] = round(bound3 / ms3, 4)
         result["points"] = points
 
     print(json.dumps(result))
