@@ -39,8 +39,16 @@ def _rmsnorm(x, weight, eps, unit_offset):
     return x * torch.rsqrt(ms + eps) * w
 
 
-def linear(x, w, out_dtype, partial_ok=False):
-    return (x.to(torch.float32) @ w.to(torch.float32).T).to(out_dtype)
+def rmsnorm(x, weight, eps, unit_offset, out_dtype):
+    """The norm of rows that are no residual stream."""
+    return _rmsnorm(x.to(torch.float32), weight, eps, unit_offset).to(out_dtype)
+
+
+def linear(x, w, out_dtype, partial_ok=False, bias=None):
+    y = (x.to(torch.float32) @ w.to(torch.float32).T).to(out_dtype)
+    if bias is not None:  # the product is rounded first, then the bias is added and the sum rounded
+        y = (y.to(torch.float32) + bias.to(torch.float32)).to(out_dtype)
+    return y
 
 
 def rope_append(qkv, n_heads, n_kv, head_dim, positions, cos, sin, rotary_dim, interleaved,
@@ -155,6 +163,7 @@ class RefOps:
     embed = staticmethod(embed)
     add_rmsnorm = staticmethod(add_rmsnorm)
     gather_add_rmsnorm = staticmethod(gather_add_rmsnorm)
+    rmsnorm = staticmethod(rmsnorm)
     linear = staticmethod(linear)
     rope_append = staticmethod(rope_append)
     attention = staticmethod(attention)

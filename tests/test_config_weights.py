@@ -85,11 +85,12 @@ def test_registry(tmp_path):
 def test_spec_has_every_constant_as_data():
     _, _, spec = spec_from_config(TINY_B)
     assert len(spec.layers) == 3 and [e.layer for e in spec.run_order] == [0, 1, 2]
-    m = spec.layers[1].mixer.params
+    assert list(spec.layers[1].parts) == ["mixer_norm", "mixer", "feed_forward_norm", "feed_forward"] and spec.layers[1].block == "prenorm"
+    m = spec.layers[1].part("mixer").params
     assert (m["num_heads"], m["num_kv_heads"], m["head_dim"], m["window"]) == (4, 1, 32, None)
     assert abs(m["scale"] - 32**-0.5) < 1e-12
     assert m["position"].params["theta"] == 500000.0 and m["position"].params["scaling"]["factor"] == 8.0
-    assert spec.layers[1].mixer_norm.params["eps"] == 1e-6
+    assert spec.layers[1].part("mixer_norm").params["eps"] == 1e-6 and spec.layers[1].part("post_mixer_norm") is None
     assert spec.head.params["tied_to"] == "model.embed_tokens.weight"
 
 

@@ -19,7 +19,8 @@ from yalis_amd.config.runtime import EngineConfig
 from yalis_amd.config.specs import LayerSpec, ModelSpec, PartSpec, RunEntry
 from yalis_amd.engine.factory import build_model, tensor_specs_for
 from yalis_amd.engine.step import ModelRunner
-from yalis_amd.parts import FeedForward, Mixer, Position, StateNeed, register_feed_forward, register_mixer, register_position
+from yalis_amd.parts import (Block, FeedForward, KVNeed, Mixer, Position, Rotation, StateNeed, register_block, register_feed_forward,
+                             register_mixer, register_position)
 from yalis_amd.weights.loader import TensorSpec
 from yalis_amd.weights.random_init import random_tensors
 
@@ -110,16 +111,18 @@ class RoutedFeedForward(FeedForward):
 # ------------------------------------------------------ a position encoding of its own
 @register_position("toy_sqrt_rotary")
 class SqrtRotary(Position):
-    """Rotation by angles sqrt(position) * theta^(-2i/d): offers what the attention part
-    reads of a position encoding (cos, sin, rotary_dim, interleaved)."""
+    """Rotation by angles sqrt(position) * theta^(-2i/d): offers the attention part a
+    ``Rotation`` of its own making."""
 
     def __init__(self, params, rt):
         super().__init__(params, rt)
         self.rotary_dim = params["rotary_dim"]
-        self.interleaved = False
         inv = 1.0 / (params["theta"] ** (torch.arange(0, self.rotary_dim, 2, dtype=torch.float32) / self.rotary_dim))
         angle = torch.outer(torch.sqrt(torch.arange(rt.max_positions, dtype=torch.float32)), inv)
         self.cos, self.sin = torch.cos(angle).to(rt.device), torch.sin(angle).to(rt.device)
+
+    def rotation(self):
+        return Rotation(self.cos, self.sin, self.rotary_dim, interleaved=False)
 
 
 # ----------------------------------------------------------------- a toy architecture
@@ -159,7 +162,8 @@ def build_toy_spec(c: ToyConfig) -> ModelSpec:
 
     def layer(i, mixer, feed_forward=None):
         p = f"toy.{i}"
-        return LayerSpec(p, "prenorm", mixer, feed_forward or ffn(p + ".ff"), norm(p + ".n1"), norm(p + ".n2"))
+        return LayerSpec.of(p, "prenorm", mixer_norm=norm(p + ".n1"), mixer=mixer, feed_forward_norm=norm(p + ".n2"),
+                            feed_forward=feed_forward or ffn(p + ".ff"))
 
     routed = PartSpec("toy_routed", {"prefix": "toy.1.ff", "hidden_size": c.hidden, "inner_size": c.inter // 2, "experts": c.experts})
     sqrt_rotary = PartSpec("toy_sqrt_rotary", {"rotary_dim": c.head_dim, "theta": c.theta})

@@ -182,33 +182,35 @@ class CacheMemory:
 
     def __init__(self, model, page_size: int, num_pages: Sequence[int], num_slots: int, dtype: torch.dtype, device: str):
         self.page_size = page_size
-        self.pages: List[torch.Tensor] = []
+        # per group: keys [entries, pages, kv_heads, page_size * head_dim] and values
+        # [entries, pages, kv_heads, page_size * value_dim] (None for a group that keeps keys only)
+        self.keys: List[torch.Tensor] = []
+        self.values: List[Optional[torch.Tensor]] = []
         for g, grp in enumerate(model.cache_groups):
             n = grp.need
-            self.pages.append(
-                torch.zeros(
-                    (len(grp.entries), 2, num_pages[g], n.num_kv_heads, page_size * n.head_dim),
-                    dtype=dtype,
-                    device=device,
-                )
-            )
+            shape = (len(grp.entries), num_pages[g], n.num_kv_heads)
+            self.keys.append(torch.zeros((*shape, page_size * n.head_dim), dtype=dtype, device=device))
+            self.values.append(torch.zeros((*shape, page_size * n.v_dim), dtype=dtype, device=device) if n.v_dim else None)
+        self._state_needs = list(model.state_needs)
         self.states: List[torch.Tensor] = [
-            torch.zeros((num_slots, *s.shape), dtype=s.dtype, device=device) for s in model.state_needs
+            torch.full((num_slots, *s.shape), s.fill, dtype=s.dtype, device=device) for s in self._state_needs
         ]
         self._needs = [grp.need for grp in model.cache_groups]
 
     def kv(self, group: int, index: int):
-        """(keys [pages, kv_heads, page_size, head_dim], values [pages, kv_heads,
-        head_dim, page_size]) of one run entry."""
-        t = self.pages[group][index]
+        """(keys [pages, kv_heads, page_size, head_dim], values [pages, kv_heads, value_dim,
+        page_size] or None where the group keeps no values) of one run entry."""
         n = self._needs[group]
-        k = t[0].view(-1, n.num_kv_heads, self.page_size, n.head_dim)
-        v = t[1].view(-1, n.num_kv_heads, n.head_dim, self.page_size)
+        k = self.keys[group][index].view(-1, n.num_kv_heads, self.page_size, n.head_dim)
+        v = self.values[group]
+        if v is not None:
+            v = v[index].view(-1, n.num_kv_heads, n.v_dim, self.page_size)
         return k, v
 
     def clear_state(self, slot: int) -> None:
-        for s in self.states:
-            s[slot].zero_()
+        """A request's rows of every state tensor, as a new request finds them."""
+        for s, need in zip(self.states, self._state_needs):
+            s[slot].fill_(need.fill)
 
     def bytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in self.pages + self.states)
+        return sum(t.numel() * t.element_size() for t in self.keys + [v for v in self.values if v is not None] + self.states)

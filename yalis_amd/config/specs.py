@@ -26,18 +26,28 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer: a block arrangement around a mixer and a feed-forward.
+    """One layer: a block arrangement and the parts it is built from, by role.
 
-    ``prefix`` is the layer's tensor-name prefix (``model.layers.3``); each part
-    gets its own prefix below it through its params (``prefix`` key).
+    ``block`` is the block-arrangement registry key; the arrangement says which roles it
+    knows, of which family each is (mixer, feed-forward, norm) and which it can do without
+    (``Block.roles``).  The pre-norm block of Llama has the roles ``mixer_norm``, ``mixer``,
+    ``feed_forward_norm`` and ``feed_forward``; another arrangement may have post-norms, a
+    single norm, or no feed-forward at all.  ``prefix`` is the layer's tensor-name prefix
+    (``model.layers.3``); each part gets its own prefix below it through its params.
     """
 
     prefix: str
     block: str  # block-arrangement registry key, e.g. "prenorm"
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    parts: Mapping[str, PartSpec] = field(default_factory=dict)  # role -> part
+
+    @classmethod
+    def of(cls, prefix: str, block: str, **parts: Optional[PartSpec]) -> "LayerSpec":
+        """``LayerSpec.of("layers.0", "prenorm", mixer=..., feed_forward=..., ...)``; roles
+        given as None are left out."""
+        return cls(prefix, block, {role: part for role, part in parts.items() if part is not None})
+
+    def part(self, role: str) -> Optional[PartSpec]:
+        return self.parts.get(role)
 
 
 @dataclass(frozen=True)

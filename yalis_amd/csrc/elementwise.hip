@@ -121,6 +121,8 @@ __device__ __forceinline__ size_t table_row(const int32_t* __restrict__ ids, siz
 //       n_splits > 1: delta holds the unreduced K slices of a product, float32)
 //   residual[src] = v                                  (only when rows is null)
 //   out[r] = v * rsqrt(mean(v^2) + eps) * (weight [+ 1])
+// Without a residual (null) v is the delta alone and nothing is written back: the plain norm
+// of rows that are no residual stream (a branch's output, queries, keys).
 // With table_ids the residual stream starts here: `delta` is an embedding table, v =
 // table[table_ids[src]] (the residual is not read, and written as in the plain form).
 // General form: any width, two passes over the row.
@@ -133,16 +135,17 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
   __shared__ float scratch[17];
   const int r = blockIdx.x;
   const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
-  float* res = residual + src * width;
+  float* res = residual ? residual + src * width : nullptr;
+  const bool fresh = table_ids != nullptr || res == nullptr;  // nothing is read from a residual
   const TD* del = delta ? delta + (table_ids ? table_row(table_ids, src, table_rows) : src) * width : nullptr;
   float ss = 0.f;
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
-    float v = table_ids ? 0.f : res[c];
+    float v = fresh ? 0.f : res[c];
     if (del) {
       float d = 0.f;
       for (int s = 0; s < n_splits; ++s) d += to_f32<TD>(del[s * split_stride + c]);
       v += as_output(d, round_sum);
-      if (!rows) res[c] = v;
+      if (!rows && res) res[c] = v;
     }
     ss += v * v;
   }
@@ -150,8 +153,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
   const float inv = rsqrtf(ss / static_cast<float>(width) + eps);
   TO* o = out + static_cast<size_t>(r) * width;
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
-    float v = res[c];
-    if (del && rows) {  // not written back in the gathered form
+    float v = res ? res[c] : 0.f;
+    if (del && (rows || !res)) {  // not written back in the gathered form, nor without a residual
       float d = 0.f;
       for (int s = 0; s < n_splits; ++s) d += to_f32<TD>(del[s * split_stride + c]);
       v += as_output(d, round_sum);
@@ -174,7 +177,8 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(
   __shared__ float scratch[17];
   const int r = blockIdx.x;
   const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
-  float* res = residual + src * width;
+  float* res = residual ? residual + src * width : nullptr;
+  const bool fresh = table_ids != nullptr || res == nullptr;  // nothing is read from a residual
   const TD* del = delta ? delta + (table_ids ? table_row(table_ids, src, table_rows) : src) * width : nullptr;
   float4 v[NORM_IT], w[NORM_IT], ds[NORM_IT];
   float ss = 0.f;
@@ -182,7 +186,7 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(
   for (int it = 0; it < NORM_IT; ++it) {
     const int c = (threadIdx.x + it * blockDim.x) * 4;
     if (c < width) {
-      v[it] = table_ids ? make_float4(0.f, 0.f, 0.f, 0.f) : load4<float>(res + c);
+      v[it] = fresh ? make_float4(0.f, 0.f, 0.f, 0.f) : load4<float>(res + c);
       w[it] = load4<TW>(weight + c);
     }
   }
@@ -226,7 +230,7 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(
   for (int it = 0; it < NORM_IT; ++it) {
     const int c = (threadIdx.x + it * blockDim.x) * 4;
     if (c < width) {
-      if (del && !rows) store4<float>(res + c, v[it]);
+      if (del && !rows && res) store4<float>(res + c, v[it]);
       ss += v[it].x * v[it].x + v[it].y * v[it].y + v[it].z * v[it].z + v[it].w * v[it].w;
     }
   }
@@ -289,6 +293,7 @@ extern "C" int yk_add_rmsnorm(float* residual, const void* delta, int delta_dtyp
                               int out_dtype, int n_rows, int n_residual_rows, int width, float eps,
                               int unit_offset, const int32_t* table_ids, int table_rows, hipStream_t stream) {
   YK_REQUIRE(n_rows >= 0 && width > 0 && n_residual_rows >= 0, "add_rmsnorm: bad sizes");
+  YK_REQUIRE(residual || (delta && !table_ids), "add_rmsnorm: without a residual there must be rows to normalise");
   YK_REQUIRE(!table_ids || (delta && n_splits == 1 && !rows && table_rows > 0 && !round_sum),
              "add_rmsnorm: an embedding table comes whole, with one id per row of the residual");
   YK_REQUIRE(eps >= 0.f, "add_rmsnorm: eps must not be negative");
@@ -689,4 +694,37 @@ extern "C" int yk_gated_act(const void* gu, int src_dtype, int n_splits, int rou
   if (src_dtype == YK_F32 && out_dtype == YK_BF16) return launch_gated_act<float, bf16_t>(gu, n_splits, round_sum, out, n_rows, inter, act, group, stream);
   if (src_dtype == YK_BF16 && out_dtype == YK_BF16) return launch_gated_act<bf16_t, bf16_t>(gu, n_splits, round_sum, out, n_rows, inter, act, group, stream);
   return yk_fail("gated_act: unsupported dtype combination");
+}
+
+// ------------------------------------------------------------------------------- bias
+// y[m, :] += bias (float32 sum, rounded once to y's dtype).  Llama has no biases; parts
+// offer them as an option, and this is all that option costs the kernel library.
+template <typename TY, typename TB>
+__global__ void add_bias_kernel(TY* __restrict__ y, const TB* __restrict__ bias, size_t total, int cols, int ldy) {
+  for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    const size_t m = i / cols;
+    const int n = static_cast<int>(i % cols);
+    TY* p = y + m * ldy + n;
+    *p = from_f32<TY>(to_f32<TY>(*p) + to_f32<TB>(bias[n]));
+  }
+}
+
+extern "C" int yk_add_bias(void* y, int y_dtype, const void* bias, int bias_dtype, int rows, int cols, int ldy,
+                           hipStream_t stream) {
+  YK_REQUIRE(rows >= 0 && cols > 0 && ldy >= cols, "add_bias: bad sizes");
+  if (rows == 0) return 0;
+  const size_t total = static_cast<size_t>(rows) * cols;
+  const int grid = static_cast<int>(std::min<size_t>((total + 255) / 256, 65535));
+#define YK_CASE(YD, TY, BD, TB)                                                              \
+  if (y_dtype == YD && bias_dtype == BD) {                                                  \
+    add_bias_kernel<TY, TB><<<grid, 256, 0, stream>>>(static_cast<TY*>(y), static_cast<const TB*>(bias), total, cols, ldy); \
+    return yk_check_launch("add_bias");                                                     \
+  }
+  YK_CASE(YK_F32, float, YK_F32, float)
+  YK_CASE(YK_F32, float, YK_BF16, bf16_t)
+  YK_CASE(YK_BF16, bf16_t, YK_F32, float)
+  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t)
+#undef YK_CASE
+  return yk_fail("add_bias: unsupported dtype combination");
 }

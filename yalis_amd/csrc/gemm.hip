@@ -41,6 +41,9 @@ __global__ __launch_bounds__(256) void gemm_fma_kernel(const TX* __restrict__ x,
       ws[kk][r] = (n < N && k < K) ? to_f32<TW>(w[static_cast<size_t>(n) * ldw + k]) : 0.f;
     }
     __syncthreads();
+    // the K step's 16 products are summed on their own and then added to the running sum: a sum
+    // of K terms carries the rounding of about sqrt(K / 16) + 4 additions instead of sqrt(K)
+    float part[4][4] = {};
 #pragma unroll
     for (int kk = 0; kk < FK; ++kk) {
       float a[4], b[4];
@@ -51,8 +54,12 @@ __global__ __launch_bounds__(256) void gemm_fma_kernel(const TX* __restrict__ x,
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        for (int j = 0; j < 4; ++j) part[i][j] = fmaf(a[i], b[j], part[i][j]);
     }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] += part[i][j];
     __syncthreads();
   }
 #pragma unroll

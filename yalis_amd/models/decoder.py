@@ -13,7 +13,8 @@ from typing import Callable, Dict, List, Mapping, Optional, Tuple
 import torch
 
 from ..config.specs import ModelSpec
-from ..parts import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS
+from ..parts import BLOCKS, EMBEDDINGS, HEADS, NORMS
+from ..parts.base import FAMILIES
 from ..parts.base import KVNeed, Runtime, StateNeed
 from ..weights.loader import TensorSpec
 
@@ -55,14 +56,23 @@ class DecoderModel:
                 owns[e.layer] = True
         self.blocks = []
         for i, ls in enumerate(spec.layers):
-            mixer_params = dict(ls.mixer.params)
-            if not owns[i]:
-                mixer_params["projects_kv"] = False
-            mixer = MIXERS.get(ls.mixer.kind)(mixer_params, rt)
-            ffn = FEED_FORWARDS.get(ls.feed_forward.kind)(ls.feed_forward.params, rt)
-            n1 = NORMS.get(ls.mixer_norm.kind)(ls.mixer_norm.params, rt)
-            n2 = NORMS.get(ls.feed_forward_norm.kind)(ls.feed_forward_norm.params, rt)
-            self.blocks.append(BLOCKS.get(ls.block)(n1, mixer, n2, ffn))
+            arrangement = BLOCKS.get(ls.block)
+            unknown = [role for role in ls.parts if role not in arrangement.roles]
+            if unknown:
+                raise ValueError(f"layer {ls.prefix!r}: block {ls.block!r} has no roles {unknown}; it knows {sorted(arrangement.roles)}")
+            built = {}
+            for role, (family, required) in arrangement.roles.items():
+                part = ls.part(role)
+                if part is None:
+                    if required:
+                        raise ValueError(f"layer {ls.prefix!r}: block {ls.block!r} needs a part for the role {role!r}")
+                    built[role] = None
+                    continue
+                params = dict(part.params)
+                if family == "mixer" and not owns[i]:
+                    params["projects_kv"] = False
+                built[role] = FAMILIES[family].get(part.kind)(params, rt)
+            self.blocks.append(arrangement(**built))
 
         self.cache_groups, self.state_needs, self.sites = self._plan_memory()
         # a step may be replayed from a captured graph only if every part allows it
@@ -74,8 +84,8 @@ class DecoderModel:
         states: List[StateNeed] = []
         sites: List[SiteInfo] = []
         for i, e in enumerate(self.spec.run_order):
-            mixer = self.blocks[e.layer].mixer
-            need = mixer.kv_need()
+            mixer = getattr(self.blocks[e.layer], "mixer", None)
+            need = None if mixer is None else mixer.kv_need()
             group = index = None
             owns = False
             if need is not None:
@@ -100,7 +110,7 @@ class DecoderModel:
                     group, index = src.group, src.index_in_group
             elif e.cache_from is not None:
                 raise ValueError(f"run_order[{i}] names cache_from but its mixer keeps no cache")
-            sneed = mixer.state_need()
+            sneed = None if mixer is None else mixer.state_need()
             sidx = None
             if sneed is not None:
                 sidx = len(states)

@@ -214,13 +214,13 @@ def build_llama_spec(cfg: LlamaConfig) -> ModelSpec:
             },
         )
         layers.append(
-            LayerSpec(
-                prefix=p,
-                block="prenorm",
-                mixer=mixer,
-                feed_forward=ffn,
+            LayerSpec.of(
+                p,
+                "prenorm",
                 mixer_norm=norm(f"{p}.input_layernorm.weight"),
+                mixer=mixer,
                 feed_forward_norm=norm(f"{p}.post_attention_layernorm.weight"),
+                feed_forward=ffn,
             )
         )
     spec = ModelSpec(

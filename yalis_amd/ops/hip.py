@@ -53,6 +53,7 @@ _SIGNATURES = {
          _c_int, _c_int, _c_int, _vp, _vp, _vp, _c_int, _vp],
         _c_int,
     ),
+    "yk_add_bias": ([_vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_gated_act": ([_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_gemm_fma": (
         [_vp, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
@@ -107,7 +108,7 @@ _LATER_SIGNATURES = {
         "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
     },
 }
-_ABI = 11
+_ABI = 12
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
 # above it the vendor library does.
@@ -360,6 +361,30 @@ class HipOps:
         return residual, EmbeddedRows(self, token_ids, table)
 
     # ----------------------------------------------------------------------- norm
+    def rmsnorm(self, x, weight, eps, unit_offset, out_dtype):
+        """norm(x) * weight for rows ``x`` [N, width] that are no residual stream (a tensor, or a
+        ``SplitSum`` whose slices are summed on the way); nothing is written but the result."""
+        n_splits, round_sum, src = 1, 0, x
+        if isinstance(x, SplitAttention):
+            x = src = x.merge()
+        if isinstance(x, SplitSum):
+            n_splits, round_sum, src = x.n_splits, x.round_sum, x.tensor
+        else:
+            self._rows(x, "norm input")
+            if not x.is_contiguous():
+                raise KernelError("norm input must be contiguous")
+        n, width = x.shape
+        if weight.numel() != width:
+            raise KernelError(f"norm weight has {weight.numel()} elements, rows have {width}")
+        out = torch.empty((n, width), dtype=out_dtype, device=src.device)
+        self._check(
+            self.lib.yk_add_rmsnorm(
+                None, src.data_ptr(), _code(src.dtype), n_splits, round_sum, None, weight.data_ptr(), _code(weight.dtype),
+                out.data_ptr(), _code(out_dtype), n, n, width, float(eps), int(bool(unit_offset)), None, 0, self._stream(),
+            )
+        )
+        return out
+
     def _norm(self, residual, delta, rows, weight, eps, unit_offset, out_dtype, n_out):
         self._rows(residual, "residual")
         if residual.dtype != torch.float32 or not residual.is_contiguous():
@@ -401,9 +426,17 @@ class HipOps:
         return self._norm(residual, delta, rows, weight, eps, unit_offset, out_dtype, rows.numel())
 
     # --------------------------------------------------------------------- linear
-    def linear(self, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, partial_ok: bool = False):
-        """x [M, K] . w [N, K]^T -> [M, N].  With ``partial_ok`` the result may come as a
-        ``SplitSum`` for a consumer that adds the slices itself."""
+    def linear(self, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, partial_ok: bool = False, bias=None):
+        """x [M, K] . w [N, K]^T (+ bias [N]) -> [M, N].  With ``partial_ok`` (and no bias) the
+        result may come as a ``SplitSum`` for a consumer that adds the slices itself."""
+        if bias is not None:
+            y = self.linear(x, w, out_dtype, partial_ok=False)
+            if bias.numel() != y.shape[1] or not bias.is_contiguous():
+                raise KernelError(f"linear: bias has {bias.numel()} elements, the product {y.shape[1]} columns")
+            if y.shape[0]:
+                self._check(self.lib.yk_add_bias(y.data_ptr(), _code(y.dtype), bias.data_ptr(), _code(bias.dtype),
+                                                 y.shape[0], y.shape[1], y.stride(0), self._stream()))
+            return y
         if isinstance(x, SplitAttention):
             y = self._linear_from_attention(x, w, out_dtype, partial_ok)
             if y is not None:

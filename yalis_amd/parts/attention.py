@@ -9,8 +9,10 @@ group in one matrix (yalis/external/model.py:445-456); here the three checkpoint
 matrices are stacked [q; k; v], which is the same arithmetic.
 
 params: prefix, hidden_size, num_heads, num_kv_heads, head_dim, scale, window
-(None: every earlier key), position (a PartSpec or None), names (optional
-overrides of the four tensor names below the prefix).
+(None: every earlier key), position (a PartSpec or None; this mixer uses a position
+encoding's ``rotation()``), names (optional overrides of the tensor names below the
+prefix), bias (False; True: the four projections have biases ``*.bias`` beside their
+weights, which Llama's do not).
 """
 from __future__ import annotations
 
@@ -45,9 +47,14 @@ class Attention(Mixer):
         self.names = {k: f"{self.prefix}.{v}" for k, v in names.items()}
         # False when every run entry of this layer borrows another entry's cache
         self.projects_kv = bool(params.get("projects_kv", True))
+        self.bias = bool(params.get("bias", False))
         pos: PartSpec = params.get("position")
         self.position = None if pos is None else POSITIONS.get(pos.kind)(pos.params, rt)
-        if self.position is not None and self.position.rotary_dim > self.head_dim:
+        # what this mixer takes of a position encoding: a rotation of queries and keys
+        self.rotation = None if self.position is None else self.position.rotation()
+        if self.position is not None and self.rotation is None:
+            raise ValueError(f"{self.prefix}: position encoding {pos.kind!r} offers no rotation, which is all this mixer applies")
+        if self.rotation is not None and self.rotation.rotary_dim > self.head_dim:
             raise ValueError("rotary_dim exceeds head_dim")
         rt.ops.check_attention_sizes(self.n_heads, self.n_kv, self.head_dim, rt.page_size)
         self.tokens_per_tile = rt.ops.attention_tokens_per_tile(self.n_heads, self.n_kv)
@@ -65,12 +72,13 @@ class Attention(Mixer):
         if self.rotates_in_launch:
             from ..ops.hip import RopeInLaunch
 
-            p = self.position
+            p = self.rotation
             self.rope_in_launch = {
                 append: RopeInLaunch(None if p is None else p.cos, None if p is None else p.sin,
                                      0 if p is None else p.rotary_dim, False if p is None else p.interleaved, append)
                 for append in (False, True)
             }
+        self.b_qkv = self.b_q = self.b_o = None
 
     # ---- what it needs
     def tensor_specs(self) -> Dict[str, TensorSpec]:
@@ -83,7 +91,14 @@ class Attention(Mixer):
         if self.projects_kv:
             specs[self.names["k"]] = TensorSpec((kd, self.hidden))
             specs[self.names["v"]] = TensorSpec((kd, self.hidden))
+        if self.bias:
+            for which, spec in list(specs.items()):
+                specs[self._bias_name(which)] = TensorSpec((spec.shape[0],), "float", ("normal", 0.02))
         return specs
+
+    @staticmethod
+    def _bias_name(weight_name: str) -> str:
+        return weight_name[: -len("weight")] + "bias" if weight_name.endswith("weight") else weight_name + ".bias"
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         q = tensors[self.names["q"]]
@@ -93,6 +108,14 @@ class Attention(Mixer):
         else:
             self.w_q = q
         self.w_o = tensors[self.names["o"]]
+        if self.bias:
+            b = lambda which: tensors[self._bias_name(self.names[which])]
+            if self.projects_kv:
+                self.b_qkv = torch.cat([b("q"), b("k"), b("v")]).contiguous()
+                self.b_q = self.b_qkv[: q.shape[0]]
+            else:
+                self.b_q = b("q")
+            self.b_o = b("o")
 
     def kv_need(self) -> KVNeed:
         return KVNeed(self.n_kv, self.head_dim, self.window)
@@ -134,17 +157,17 @@ class Attention(Mixer):
         if site.owns_cache:
             if not self.projects_kv:
                 raise RuntimeError(f"{self.prefix}: run entry owns a cache but the layer has no k/v projections")
-            qkv = ops.linear(h, self.w_qkv, self.rt.act_dtype, partial_ok=True)
+            qkv = self._project(h, self.w_qkv, self.b_qkv)
             n_kv_rows = self.n_kv
         else:
-            qkv = ops.linear(h, self.w_q, self.rt.act_dtype, partial_ok=True)
+            qkv = self._project(h, self.w_q, self.b_q)
             n_kv_rows = 0
         k_cache, v_cache = site.kv()
         memo_key = f"attention_long_col_tiles_{self.layout}"
         col_tiles = ctx.memo.get(memo_key)
         if col_tiles is None:
             col_tiles = ctx.memo[memo_key] = self.long_col_tiles(ctx.host)
-        pos = self.position
+        pos = self.rotation
         tiles = ctx.arrays[f"attention_tiles_{self.tokens_per_tile}_upto{self.long_tile}"]
         token_cols = ctx.arrays[f"attention_token_columns_{self.tokens_per_tile}_upto{self.long_tile}"]
         if ctx.max_qlen == 1 and self.rotates_in_launch:
@@ -154,7 +177,7 @@ class Attention(Mixer):
                 0 if self.window is None else int(self.window), ctx, site.group, tiles, token_cols=token_cols,
                 rope=self.rope_in_launch[bool(n_kv_rows)],
             )
-            return ops.linear(out, self.w_o, self.rt.act_dtype, partial_ok=True)
+            return self._project(out, self.w_o, self.b_o)
         q = ops.rope_append(
             qkv,
             self.n_heads,
@@ -187,4 +210,10 @@ class Attention(Mixer):
             long_col_tiles=col_tiles,
             token_cols=token_cols,
         )
-        return ops.linear(out, self.w_o, self.rt.act_dtype, partial_ok=True)
+        return self._project(out, self.w_o, self.b_o)
+
+    def _project(self, x, w, b):
+        """x . w^T (+ b); without a bias the product may come as unreduced K slices."""
+        if b is None:
+            return self.rt.ops.linear(x, w, self.rt.act_dtype, partial_ok=True)
+        return self.rt.ops.linear(x, w, self.rt.act_dtype, bias=b)

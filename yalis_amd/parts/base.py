@@ -36,20 +36,40 @@ class Runtime:
 @dataclass(frozen=True)
 class KVNeed:
     """A mixer's need for cached keys and values: per token ``num_kv_heads`` rows
-    of ``head_dim`` for keys and the same for values.  ``window`` = how many of the
-    latest tokens are ever read again (None: all of them)."""
+    of ``head_dim`` for keys and of ``value_dim`` for values (None: as wide as the keys;
+    0: no values are kept, the pages hold keys only, e.g. one compressed row per token).
+    ``window`` = how many of the latest tokens are ever read again (None: all of them)."""
 
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    value_dim: Optional[int] = None
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclass(frozen=True)
 class StateNeed:
-    """A mixer's need for per-request state of fixed size (zero at admission)."""
+    """A mixer's need for per-request state of fixed size; a request's row is filled with
+    ``fill`` at admission."""
 
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+    fill: float = 0.0
+
+
+@dataclass(frozen=True)
+class Rotation:
+    """What a rotary position encoding hands a mixer: float32 tables [positions,
+    rotary_dim / 2] on the device, how many leading elements of a head rotate, and how pairs
+    are formed (interleaved: (2i, 2i + 1); else (i, i + rotary_dim / 2))."""
+
+    cos: torch.Tensor
+    sin: torch.Tensor
+    rotary_dim: int
+    interleaved: bool = False
 
 
 class Part:
@@ -104,6 +124,12 @@ class Norm(Part):
     # ungathered rows (``ops.embedded_rows``) in its place
     takes_embedded_rows = False
 
+    def norm(self, x) -> torch.Tensor:
+        """norm(x) for an ``x`` [N, size] that is no residual stream: a branch's output before it
+        joins the residual (a post-norm), queries or keys.  ``x`` may be whatever a part's
+        ``forward`` returned; the result is in the activation dtype."""
+        raise NotImplementedError
+
     def add_norm(self, residual: torch.Tensor, delta: Optional[torch.Tensor]) -> torch.Tensor:
         """residual (float32, [N, size]) += delta in place when delta is given;
         returns norm(residual) in the activation dtype."""
@@ -115,13 +141,32 @@ class Norm(Part):
 
 
 class Position(Part):
-    """A position encoding applied to queries and keys inside a mixer."""
+    """A position encoding.  What a mixer may ask of it (a kind implements what it offers and
+    leaves the rest at None; a mixer raises for a kind that offers nothing it can use):
+
+    * ``rotation()`` -> ``Rotation``: rotate queries and keys by position-dependent angles;
+    * ``added_to_input(positions)`` -> [N, hidden] in the activation dtype: an encoding of the
+      tokens' absolute positions that a mixer adds to its input (learned or fixed tables).
+    """
+
+    def rotation(self) -> Optional["Rotation"]:
+        return None
+
+    def added_to_input(self, positions: torch.Tensor) -> Optional[torch.Tensor]:
+        return None
 
 
 class Block:
     """The arrangement of norms, mixer and feed-forward around the residual.
-    Built from four finished parts: (mixer_norm, mixer, feed_forward_norm,
-    feed_forward)."""
+
+    ``roles`` names the parts an arrangement is built from: role -> (family, required), the
+    family one of "mixer", "feed_forward", "norm".  The model builds every role a layer's
+    spec names through the family's registry and calls the arrangement with them as keyword
+    arguments (roles the spec leaves out, where not required, come as None).  ``mixer`` (a role
+    or None) is the part whose cache and state the model plans memory for."""
+
+    roles: Dict[str, Tuple[str, bool]] = {}
+    mixer = None
 
     # True when the block's first act is ``add_norm(residual, delta)`` of a norm that takes an
     # embedding's ungathered rows as ``delta`` (``Norm.takes_embedded_rows``): the model then
@@ -129,7 +174,8 @@ class Block:
     takes_embedded_rows = False
 
     def parts(self):
-        raise NotImplementedError
+        """The block's parts, in the order of ``roles`` (None for roles left out are skipped)."""
+        return tuple(p for p in (getattr(self, role, None) for role in self.roles) if p is not None)
 
     def forward(self, residual, delta, ctx, site):
         """residual: float32 [N, hidden], updated in place; delta: the previous
@@ -164,6 +210,9 @@ POSITIONS = _Registry("position encoding")
 BLOCKS = _Registry("block arrangement")
 EMBEDDINGS = _Registry("embedding")
 HEADS = _Registry("output head")
+
+# family name (``Block.roles``) -> registry
+FAMILIES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS}
 
 register_mixer = MIXERS.register
 register_feed_forward = FEED_FORWARDS.register

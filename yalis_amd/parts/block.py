@@ -16,6 +16,13 @@ from .base import Block, register_block
 
 @register_block("prenorm")
 class PreNormBlock(Block):
+    roles = {
+        "mixer_norm": ("norm", True),
+        "mixer": ("mixer", True),
+        "feed_forward_norm": ("norm", True),
+        "feed_forward": ("feed_forward", True),
+    }
+
     def __init__(self, mixer_norm, mixer, feed_forward_norm, feed_forward):
         self.mixer_norm = mixer_norm
         self.mixer = mixer
@@ -25,9 +32,6 @@ class PreNormBlock(Block):
     @property
     def takes_embedded_rows(self):
         return bool(getattr(self.mixer_norm, "takes_embedded_rows", False))
-
-    def parts(self):
-        return (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward)
 
     def forward(self, residual, delta, ctx, site):
         h = self.mixer_norm.add_norm(residual, delta)

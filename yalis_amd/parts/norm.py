@@ -37,6 +37,9 @@ class RMSNorm(Norm):
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.weight = tensors[self.name]
 
+    def norm(self, x):
+        return self.rt.ops.rmsnorm(x, self.weight, self.eps, self.unit_offset, self.rt.act_dtype)
+
     def add_norm(self, residual, delta):
         return self.rt.ops.add_rmsnorm(
             residual, delta, self.weight, self.eps, self.unit_offset, self.rt.act_dtype

@@ -17,7 +17,7 @@ import math
 
 import torch
 
-from .base import Position, Runtime, register_position
+from .base import Position, Rotation, Runtime, register_position
 
 
 def inverse_frequencies(rotary_dim: int, theta: float, scaling) -> torch.Tensor:
@@ -72,3 +72,6 @@ class Rotary(Position):
     @property
     def interleaved(self) -> bool:
         return self.pairing == "interleaved"
+
+    def rotation(self) -> Rotation:
+        return Rotation(self.cos, self.sin, self.rotary_dim, self.interleaved)
