@@ -209,7 +209,9 @@ def test_far_key_across_pages(backend, page):
     cfg = ALL["C"]
     weights = P.random_weights(cfg, seed=2)
     for n in ("q_proj", "k_proj"):
-        weights[f"model.layers.0.self_attn.{n}.weight"][:64] *= 30.0
+        # (12: the head looks at its far key, and float32 itself still carries the result: at 30
+        # the plain implementation in float32 is 2.3e-5 from its own float64 form, at 12 7e-6)
+        weights[f"model.layers.0.self_attn.{n}.weight"][:64] *= 12.0
     toks = C.make_requests(cfg, [300], seed=6)["r0"]
     toks[-1] = toks[3]
     want = C.plain_logits(cfg, weights, {"r0": toks}, dtype == "bfloat16")
