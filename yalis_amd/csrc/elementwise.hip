@@ -100,8 +100,8 @@ __device__ __forceinline__ void store4<float>(float* p, float4 v) {
 template <>
 __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float4 v) {
   uint2 raw;
-  raw.x = static_cast<uint32_t>(f32_to_bf16(v.x)) | (static_cast<uint32_t>(f32_to_bf16(v.y)) << 16);
-  raw.y = static_cast<uint32_t>(f32_to_bf16(v.z)) | (static_cast<uint32_t>(f32_to_bf16(v.w)) << 16);
+  raw.x = pack_bf16x2(v.x, v.y);
+  raw.y = pack_bf16x2(v.z, v.w);
   *reinterpret_cast<uint2*>(p) = raw;
 }
 
@@ -434,10 +434,8 @@ __device__ __forceinline__ void rope_rotate8(const uint4& a, const uint4& b, con
     const float a0 = __uint_as_float(aw[j] << 16), a1 = __uint_as_float(aw[j] & 0xffff0000u);
     const float b0 = __uint_as_float(bw[j] << 16), b1 = __uint_as_float(bw[j] & 0xffff0000u);
     const float c0 = c[2 * j], c1 = c[2 * j + 1], s0 = s[2 * j], s1 = s[2 * j + 1];
-    ra[j] = static_cast<uint32_t>(from_f32<bf16_t>(rot_first(a0, b0, c0, s0))) |
-            (static_cast<uint32_t>(from_f32<bf16_t>(rot_first(a1, b1, c1, s1))) << 16);
-    rb[j] = static_cast<uint32_t>(from_f32<bf16_t>(rot_second(a0, b0, c0, s0))) |
-            (static_cast<uint32_t>(from_f32<bf16_t>(rot_second(a1, b1, c1, s1))) << 16);
+    ra[j] = pack_bf16x2(rot_first(a0, b0, c0, s0), rot_first(a1, b1, c1, s1));
+    rb[j] = pack_bf16x2(rot_second(a0, b0, c0, s0), rot_second(a1, b1, c1, s1));
   }
   oa = make_uint4(ra[0], ra[1], ra[2], ra[3]);
   ob = make_uint4(rb[0], rb[1], rb[2], rb[3]);
@@ -652,8 +650,7 @@ __global__ void gated_act_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* _
   for (int k = 0; k < 4; ++k) {
     const float g0 = __uint_as_float(gw[k] << 16), g1 = __uint_as_float(gw[k] & 0xffff0000u);
     const float u0 = __uint_as_float(uw[k] << 16), u1 = __uint_as_float(uw[k] & 0xffff0000u);
-    o[k] = static_cast<uint32_t>(from_f32<bf16_t>(act_apply(g0, act) * u0)) |
-           (static_cast<uint32_t>(from_f32<bf16_t>(act_apply(g1, act) * u1)) << 16);
+    o[k] = pack_bf16x2(act_apply(g0, act) * u0, act_apply(g1, act) * u1);
   }
   *reinterpret_cast<uint4*>(out + n * inter + j) = make_uint4(o[0], o[1], o[2], o[3]);
 }
