@@ -232,7 +232,9 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
   constexpr int KS = D / 32;  // matrix-core steps over the head dimension
   constexpr int DT = D / 16;  // output tiles over the head dimension
   constexpr bool ROPE = SRC != 0;  // SRC 0: queries from `q`; 1, 2: rotary + append in here (rope_src_load8)
-  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, gq = lane / 16;
+  const int lane = threadIdx.x % 64, r = lane % 16, gq = lane / 16;
+  // (the same in every lane, and said so: what hangs on it then branches instead of masking lanes)
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
   const int t = blockIdx.x;
   const int seq = tiles[4 * t], tok0 = tiles[4 * t + 1], pos0 = tiles[4 * t + 3];
   const int ntok = ROPE ? 1 : tiles[4 * t + 2];
@@ -510,8 +512,7 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
           }
           tmax = fmaxf(tmax, s[u][sb][i]);
         }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    tmax = column_lanes_max(tmax);
     // the maximum was taken over the raw scores (the scale is positive); the scale joins the
     // subtraction of the maximum in one fused multiply-add
     const float m_new = fmaxf(m, tmax * scale_log2);
@@ -577,8 +578,7 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
 #undef ATT_LOAD_K_AT
 #undef ATT_LOAD_V_AT
 #undef ATT_PUT_NEW_K
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
+  l = column_lanes_sum(l);
 
   if (W > 1) {
     constexpr int WP = W > 1 ? W - 1 : 1;
@@ -661,7 +661,9 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
   constexpr int PP = D / 32;    // 16-byte pieces of keys (and of values) per thread and block
   __shared__ __attribute__((aligned(16))) bf16_t ks[64][KROW];
   __shared__ __attribute__((aligned(16))) bf16_t vs[D][VROW];
-  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, gq = lane / 16;
+  const int lane = threadIdx.x % 64, r = lane % 16, gq = lane / 16;
+  // (the same in every lane, and said so: what hangs on it then branches instead of masking lanes)
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
   // Workgroups start in the order of blockIdx.x: heads vary fastest, so that the tiles the
   // host put first (those with the most keys) start first on every head and the short ones
   // fill the gaps at the end; consecutive workgroups, which land on different dies, hold
@@ -760,14 +762,22 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
     }
   }
   const size_t page_elems = static_cast<size_t>(n_kv) * page_size * D;
+  // (tiled pages: the blocks are fetched in their order, so the column of the block table and
+  // the place within the page are stepped along instead of divided out for every block)
+  int pf_col = page_col(kb_lo * 64), pf_off = page_off(kb_lo * 64);
 #define PF_LOAD(KB)                                                                                \
   if (TILED) {                                                                                      \
-    const int key0 = (KB) * 64;                                                                     \
-    const size_t base = static_cast<size_t>(page_of(key0)) * page_elems + static_cast<size_t>(g) * page_size * D + \
-                        static_cast<size_t>(page_off(key0)) * D;                                    \
+    const int page = pages_in_lds ? pages_s[pf_col - first_col] : max(0, bt[pf_col]);               \
+    const size_t base = static_cast<size_t>(page) * page_elems + static_cast<size_t>(g) * page_size * D + \
+                        static_cast<size_t>(pf_off) * D;                                            \
     _Pragma("unroll") for (int p = 0; p < PP; ++p) {                                                \
       kreg[p] = *reinterpret_cast<const u32x4_t*>(k_cache + base + 8 * (threadIdx.x + 256 * p));    \
       vreg[p] = *reinterpret_cast<const u32x4_t*>(v_cache + base + 8 * (threadIdx.x + 256 * p));    \
+    }                                                                                               \
+    pf_off += 64;                                                                                   \
+    if (pf_off >= page_size) {                                                                      \
+      pf_off = 0;                                                                                   \
+      pf_col = min(pf_col + 1, last_page_col);                                                      \
     }                                                                                               \
   } else {                                                                                          \
     _Pragma("unroll") for (int p = 0; p < PP; ++p) {                                                \
@@ -784,7 +794,7 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
     }                                                                                               \
   }
 
-  if (kb_lo < kb_hi) PF_LOAD(kb_lo)
+  if (kb_lo < kb_hi) { PF_LOAD(kb_lo) }
   for (int kb = kb_lo; kb < kb_hi; ++kb) {
     __syncthreads();  // every wave is done with the previous block
 #pragma unroll
@@ -810,8 +820,9 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
       }
     }
     __syncthreads();
-    if (kb + 1 < kb_hi) PF_LOAD(kb + 1)  // in flight while this block is worked on
-    if (kb * 64 >= wave_hi) continue;  // nothing of this block is visible to this wave
+    if (kb + 1 < kb_hi) { PF_LOAD(kb + 1) }  // in flight while this block is worked on
+    const int key0 = kb * 64;
+    if (key0 >= wave_hi) continue;  // nothing of this block is visible to this wave
 
     f32x4_t s[CT][2][2];
 #pragma unroll
@@ -829,9 +840,9 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
             s[c][u][sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[c][ks_].v, s[c][u][sb], 0, 0, 0);
         }
       }
-    // a block that every column sees whole needs no mask (columns that stand for nothing
+    // keys that every column sees whole need no mask (columns that stand for nothing
     // compute on zeros and are never stored)
-    const bool whole = kb * 64 + 63 <= (tile_pos0 + wave_tok0) && (window == 0 || kb * 64 >= max(0, wave_hi - window));
+    const bool whole = key0 + 63 <= (tile_pos0 + wave_tok0) && (window == 0 || key0 >= max(0, wave_hi - window));
     AFrag8 pf[CT][2];
     float alpha[CT];
     bool grew = false;  // some column's maximum rose: only then the running sums need rescaling
@@ -839,22 +850,26 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
     for (int c = 0; c < CT; ++c) {
       // the maximum is taken over the raw scores (the scale is positive), and the scale
       // joins the subtraction of the maximum in one fused multiply-add
+      if (!whole) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int key = key0 + 32 * u + 8 * gq + 4 * sb + i;
+              const bool ok = col_ok[c] && key <= pos_c[c] && key >= lo_c[c];
+              s[c][u][sb][i] = ok ? s[c][u][sb][i] : -INFINITY;
+            }
+      }
       float tmax = -INFINITY;
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
         for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            if (!whole) {
-              const int key = kb * 64 + 32 * u + 8 * gq + 4 * sb + i;
-              const bool ok = col_ok[c] && key <= pos_c[c] && key >= lo_c[c];
-              if (!ok) s[c][u][sb][i] = -INFINITY;
-            }
-            tmax = fmaxf(tmax, s[c][u][sb][i]);
-          }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+          for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, s[c][u][sb][i]);
+      tmax = column_lanes_max(tmax);
       const float m_new = fmaxf(m[c], tmax * scale_log2);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
       grew = grew || m_new > m[c];
@@ -875,13 +890,15 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
       l[c] = l[c] * alpha[c] + psum;
       m[c] = m_new;
     }
-    grew = __any(grew);
+    if (__any(grew)) {
+      asm volatile("" ::: "memory");  // (a branch, not a multiplication and a select per element)
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      if (grew) {
+      for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int c = 0; c < CT; ++c) acc[c][dt] *= alpha[c];
-      }
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         AFrag8 a;
@@ -896,8 +913,7 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
 #pragma unroll
   for (int c = 0; c < CT; ++c) {
     float lc = l[c];
-    lc += __shfl_xor(lc, 16, 64);
-    lc += __shfl_xor(lc, 32, 64);
+    lc = column_lanes_sum(lc);
     if (n_splits > 1) {
       // partial result of this split, a group of 16 columns per wave (and column tile)
       const size_t group = (static_cast<size_t>(t) * 4 * CT + wave * CT + c) * n_y + by;
@@ -1009,17 +1025,15 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
   float* ws_ml = workspace ? workspace + (need / (head_dim + 2)) * head_dim : nullptr;
   const float scale_log2 = scale * 1.4426950408889634f;
   dim3 grid(n_tiles * n_kv * chunks, n_splits), block(256);
+#define YK_PF_ARGS                                                                                           \
+  static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),     \
+      static_cast<const bf16_t*>(v_cache), tiles, block_table, table_width, page_size, n_heads, n_kv, hpt,     \
+      chunks, scale_log2, window, n_splits, ws_o, ws_ml, pages_lds_limit
 #define YK_PF(DD, BIP)                                                                                       \
-  if (col_tiles == 1)                                                                                        \
-    attn_mfma_prefill_kernel<DD, BIP, 1><<<grid, block, 0, stream>>>(                                            \
-      static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),   \
-      static_cast<const bf16_t*>(v_cache), tiles, block_table, table_width, page_size, n_heads, n_kv, hpt, chunks, \
-      scale_log2, window, n_splits, ws_o, ws_ml, pages_lds_limit);                                               \
+  if (col_tiles == 2)                                                                                        \
+    attn_mfma_prefill_kernel<DD, BIP, 2><<<grid, block, 0, stream>>>(YK_PF_ARGS);                            \
   else                                                                                                       \
-    attn_mfma_prefill_kernel<DD, BIP, 2><<<grid, block, 0, stream>>>(                                            \
-      static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),   \
-      static_cast<const bf16_t*>(v_cache), tiles, block_table, table_width, page_size, n_heads, n_kv, hpt, chunks, \
-      scale_log2, window, n_splits, ws_o, ws_ml, pages_lds_limit)
+    attn_mfma_prefill_kernel<DD, BIP, 1><<<grid, block, 0, stream>>>(YK_PF_ARGS)
   const bool bip = cache_is_tiled(YK_BF16, head_dim, page_size);
   if (head_dim == 64) {
     if (bip) { YK_PF(64, true); } else { YK_PF(64, false); }
@@ -1027,6 +1041,7 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
     if (bip) { YK_PF(128, true); } else { YK_PF(128, false); }
   }
 #undef YK_PF
+#undef YK_PF_ARGS
   if (yk_check_launch("attn_mfma_prefill")) return -1;
   if (n_splits > 1) {
     dim3 cgrid(4 * col_tiles * n_tiles, n_kv * chunks);

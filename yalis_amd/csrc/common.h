@@ -30,6 +30,23 @@ __device__ __forceinline__ float bf16_to_f32(bf16_t x) {
   return __uint_as_float(static_cast<uint32_t>(x) << 16);
 }
 
+// Over the four lanes r, r + 16, r + 32 and r + 48 (the lanes that share a column of a 16 x 16
+// matrix-core tile): the maximum, or the sum, in all four of them.  The swaps of half-waves and
+// of rows of 16 lanes move registers directly; a shuffle would go through the LDS pipe and
+// wait on its counter together with the operand reads.
+__device__ __forceinline__ float column_lanes_max(float v) {
+  const auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float column_lanes_sum(float v) {
+  const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // two floats to two bfloat16 (round to nearest even; NaN stays NaN) in one word: gfx950
 // converts in hardware (v_cvt_pk_bf16_f32), one instruction where the shifts and adds of a
 // conversion by hand take six (measured: 2 us of a 41 us product that converted its staged rows)
