@@ -425,7 +425,13 @@ static int skinny_plan(int M, int N, int K, bool gated, int* waves_out, int* k_b
   double best = 1e300;
   int best_w = 4;
   long best_s = 1;
-  for (int w : {4}) {  // measured: four waves per workgroup beat eight on every shape tried
+  // Four waves a workgroup beat eight at up to 32 rows of x on every shape tried.  With 64 rows
+  // a workgroup stages as many bytes of x as of the weight, and eight waves share one copy:
+  // measured on the 8B shapes at 64 rows (us, four / eight waves): gate/up 57.5 / 49.4, down
+  // 27.0 / 23.7, o-proj 11.3 / 10.5, but qkv 15.4 / 16.3 (its 384 workgroups of eight waves
+  // fill the compute units one and a half times); the model below tells these apart.
+  for (int w : {4, 8}) {
+    if (w == 8 && mt != 4) continue;
     const long rblocks = (ntiles + w - 1) / w;
     const double resident = std::min(20.0, static_cast<double>(160 * 1024 / skinny_lds_bytes(mt, w, SK_KC)) * w);
     for (long s = 1; s <= max_s; ++s) {
@@ -444,7 +450,7 @@ static int skinny_plan(int M, int N, int K, bool gated, int* waves_out, int* k_b
       }
     }
   }
-  if (g_force_waves) best_w = g_force_waves;
+  if (g_force_waves) best_w = g_force_waves == 8 && mt != 4 ? 4 : g_force_waves;
   if (g_force_slices) best_s = std::min<long>(g_force_slices, chunks);
   int k_block = static_cast<int>((chunks + best_s - 1) / best_s) * SK_KC;
   if (waves_out) *waves_out = best_w;
@@ -453,12 +459,12 @@ static int skinny_plan(int M, int N, int K, bool gated, int* waves_out, int* k_b
 }
 
 // For tests and measurements: force the few-row product's chunk length (128 or 256), its waves a
-// workgroup (4) and its number of K slices; 0 leaves a choice to the library.  Process-wide:
+// workgroup (4; 8 count only with more than 32 rows of x) and its number of K slices; 0 leaves a choice to the library.  Process-wide:
 // set it before the products it is meant for and clear it after (a caller that remembers
 // yk_gemm_skinny_splits must ask again).
 extern "C" int yk_gemm_skinny_force(int chunk, int waves, int slices) {
   YK_REQUIRE(chunk == 0 || chunk == 128 || chunk == 256, "gemm_skinny_force: chunks are 128 or 256 long");
-  YK_REQUIRE(waves == 0 || waves == 4, "gemm_skinny_force: a workgroup has 4 waves");
+  YK_REQUIRE(waves == 0 || waves == 4 || waves == 8, "gemm_skinny_force: a workgroup has 4 waves, or 8 (with more than 32 rows of x)");
   YK_REQUIRE(slices >= 0, "gemm_skinny_force: bad slice count");
   g_force_chunk = chunk;
   g_force_waves = waves;
@@ -508,9 +514,9 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, i
     gemm_mfma_skinny_kernel<MT_, W_, TO, G_, false, KC_><<<grid, block, lds, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block, AttnSplits{}); \
     return yk_check_launch("gemm_mfma_skinny");                                                         \
   }
-  SK_GO(1, 4, 0) SK_GO(2, 4, 0) SK_GO(4, 4, 0)
+  SK_GO(1, 4, 0) SK_GO(2, 4, 0) SK_GO(4, 4, 0) SK_GO(4, 8, 0)
   if constexpr (sizeof(TO) == 2) {  // gated results are bfloat16 only
-    SK_GO(1, 4, 1) SK_GO(2, 4, 1) SK_GO(4, 4, 1) SK_GO(1, 4, 2) SK_GO(2, 4, 2) SK_GO(4, 4, 2)
+    SK_GO(1, 4, 1) SK_GO(2, 4, 1) SK_GO(4, 4, 1) SK_GO(4, 8, 1) SK_GO(1, 4, 2) SK_GO(2, 4, 2) SK_GO(4, 4, 2) SK_GO(4, 8, 2)
   }
 #undef SK_GO
 #undef SK_GO_KC
