@@ -317,12 +317,39 @@ def test_linear_dispatch(ops):
     close(ops.linear(x[:5], w, torch.bfloat16), want[:5], 1e-2, 2**-7)
     # 65 to 192 rows where the vendor library would have few tiles: the few-row kernel, in row tiles of 64
     assert ops.few_library_tiles(100, 515) and not ops.few_library_tiles(200, 515) and not ops.few_library_tiles(128, 28672)
-    for rows in (65, 100, 192):
+    assert ops.few_library_tiles(128, 4096) and not ops.few_library_tiles(128, 6144) and not ops.few_library_tiles(160, 4096)
+    for rows in (65, 100, 128, 192):
         close(ops.linear(x[:rows], w, torch.bfloat16), want[:rows], 1e-2, 2**-7)
         part = ops.linear(x[:rows], w, torch.bfloat16, partial_ok=True)
         close(part.reduce() if hasattr(part, "reduce") else part, want[:rows], 1e-2, 2**-7)
     wf = w.float()
     close(ops.linear(x, wf, torch.bfloat16), want, 1e-2, 2**-7)
+
+
+@pytest.mark.parametrize("tuned", [False, True])
+def test_library_product(ops, tuned):
+    """The vendor library's product, called directly: rows of x and w with gaps between them,
+    both result types, shapes that are timed when first met (up to 256 rows) and shapes that are
+    not, and the same values again from the kept plan."""
+    ops.tune_library_products(tuned)
+    try:
+        for seed, (m, n, k, pad) in enumerate(((70, 520, 200, 0), (200, 1032, 136, 8), (300, 264, 512, 16), (129, 4096, 256, 0))):
+            # (other leading dimensions for the two settings, so that each makes plans of its own)
+            pad += 8 if tuned else 0
+            xs = rnd((m, k + pad), torch.bfloat16, 50 + seed)
+            wsrc = rnd((n, k + pad), torch.bfloat16, 60 + seed)
+            x, w = xs[:, :k], wsrc[:, :k]
+            want = x.double().cpu() @ w.double().cpu().T
+            first = ops.gemm_library(x, w, torch.bfloat16)
+            close(first, want, 1e-2, 2**-7)
+            assert torch.equal(first, ops.gemm_library(x, w, torch.bfloat16))
+            close(ops.gemm_library(x, w, torch.float32), want, 1e-4, 1e-5)
+    finally:
+        ops.tune_library_products(True)
+    from yalis_amd.ops.hip import KernelError
+
+    with pytest.raises(KernelError, match="gemm_library"):
+        ops.gemm_library(rnd((70, 64), torch.float32, 1), rnd((64, 64), torch.bfloat16, 2), torch.bfloat16)
 
 
 # ---------------------------------------------------------------- rotary + cache append

@@ -28,11 +28,13 @@ HOST_SOURCES = ["cache_manager.cpp"]
 # "kernels" only (so that is all a trace replay compiles), choosing tokens "sampling", the
 # benchmark's machine probes "probe".  Every library carries runtime.hip (its error slot).
 KERNEL_LIBS = {
-    "kernels": ["runtime.hip", "elementwise.hip", "gemm.hip", "attention.hip"],
+    "kernels": ["runtime.hip", "elementwise.hip", "gemm.hip", "attention.hip", "library_gemm.hip"],
     "sampling": ["runtime.hip", "sampling.hip"],
     "probe": ["runtime.hip", "probe.hip"],
 }
 HEADERS = ["common.h", "no_alloc.h"]
+# what a library links beside the HIP runtime: the vendor's matrix products for many rows
+LINK_LIBS = {"kernels": ["-lhipblaslt"]}
 
 HIPCC_FLAGS = [
     "-O3",
@@ -152,7 +154,7 @@ def build_host(force: bool = False) -> str:
 def build_kernels(name: str = "kernels", force: bool = False) -> str:
     """One library of HIP kernels for gfx950: one object per source, compiled side by side."""
     sources = KERNEL_LIBS[name]
-    digest = _digest(sources, HIPCC_FLAGS)
+    digest = _digest(sources, HIPCC_FLAGS + LINK_LIBS.get(name, []))
     bdir = build_dir()
     lib = os.path.join(bdir, f"libyalis_{name}.so")
     if not force and _is_current(lib, digest):
@@ -184,7 +186,7 @@ def build_kernels(name: str = "kernels", force: bool = False) -> str:
                 os.remove(o)
         raise errors[0]
     tmp = f"{lib}.{os.getpid()}.tmp"
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs], "link")
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs, *LINK_LIBS.get(name, [])], "link")
     for o in objs:
         os.remove(o)
     os.replace(tmp, lib)

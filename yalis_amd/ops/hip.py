@@ -4,8 +4,8 @@ Every method takes torch tensors on the GPU, checks what the kernels assume, and
 launches on torch's current stream.  There is no other implementation behind these
 methods: when the library cannot be built or loaded, constructing ``HipOps``
 raises.  Plain matrix products of many rows in bfloat16 go to the vendor library
-through ``torch.matmul`` (the reference uses cuBLAS in the same places,
-yalis/external/model.py:449,462-466,717-722); few-row products, every float32
+(hipBLASLt, called from ``csrc/library_gemm.hip``; the reference uses cuBLAS in the same
+places, yalis/external/model.py:449,462-466,717-722); few-row products, every float32
 product and everything else are the hand-written kernels.
 """
 from __future__ import annotations
@@ -61,6 +61,8 @@ _SIGNATURES = {
     ),
     "yk_gemm_skinny_splits": ([_c_int, _c_int, _c_int, _c_int], _c_int),
     "yk_gemm_skinny_force": ([_c_int, _c_int, _c_int], _c_int),
+    "yk_gemm_library": ([_vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_size_t, _vp, _vp], _c_int),
+    "yk_gemm_library_tune": ([_c_int], _c_int),
     "yk_gemm_mfma_skinny": (
         [_vp, _vp, _vp, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
         _c_int,
@@ -108,7 +110,7 @@ _LATER_SIGNATURES = {
         "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
     },
 }
-_ABI = 12
+_ABI = 13
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
 # above it the vendor library does.
@@ -220,8 +222,8 @@ class HipOps:
         # the quick way to the current stream's handle, where this torch has it
         self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
         self._workspace: Optional[torch.Tensor] = None  # attention splits, argmax parts
+        self._library_workspace: Optional[torch.Tensor] = None  # the vendor library's scratch
         self._gemm_workspace: Optional[torch.Tensor] = None  # K slices of products
-        self._mm_f32: Optional[bool] = None  # see _library_f32_out
         # page ids a workgroup of the long-span attention keeps in LDS (more: looked up in the
         # block table one by one); tests lower it to walk that path with short tables
         self.long_span_pages_in_lds = 2048
@@ -291,6 +293,11 @@ class HipOps:
         workgroup and number of K slices (0: the library decides); call without arguments to clear."""
         self._check(self.lib.yk_gemm_skinny_force(int(chunk), int(waves), int(slices)))
         self._answers = {k: v for k, v in self._answers.items() if k[0] not in ("yk_gemm_skinny_splits", "yk_gemm_skinny_from_attention_ok")}
+
+    def tune_library_products(self, on: bool = True) -> None:
+        """Whether new shapes of up to 256 rows get the fastest of the vendor library's candidates
+        (timed when first met; the default) or its first one (the same choice in every process)."""
+        self._check(self.lib.yk_gemm_library_tune(int(bool(on))))
 
     def workspaces(self):
         """The scratch buffers in use, for whoever must keep them alive (a captured graph)."""
@@ -454,23 +461,25 @@ class HipOps:
         aligned = k % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
         if x.dtype == bf and w.dtype == bf and aligned:
             if m > SKINNY_MAX_ROWS and out_dtype == bf and not self.few_library_tiles(m, n):
-                return torch.matmul(x, w.t())  # vendor library, bfloat16 in and out
-            if m > SKINNY_MAX_ROWS and out_dtype == torch.float32 and self._library_f32_out():
+                return self.gemm_library(x, w, bf)  # vendor library, bfloat16 in and out
+            if m > SKINNY_MAX_ROWS and out_dtype == torch.float32:
                 # vendor library, float32 accumulators stored as they are (the output head for
                 # more than 64 wanted rows: the few-row kernel would stream the table once per 64)
-                return torch.mm(x, w.t(), out_dtype=torch.float32)
+                return self.gemm_library(x, w, torch.float32)
             return self.gemm_mfma_skinny(x, w, out_dtype, partial_ok)
         return self.gemm_fma(x, w, out_dtype)
 
     @staticmethod
     def few_library_tiles(m: int, n: int) -> bool:
-        """Whether a product of 65 to 192 rows is still the few-row kernel's: where the vendor
-        library's output tiles (256 columns wide, one or two tiles of rows) would be too few
-        to occupy the GPU's 256 compute units, while the few-row kernel divides K among
-        workgroups.  Measured at 128 rows (us, few-row kernel / library), 8B shapes: o-proj
-        16 / 25, down-proj 48 / 76, qkv 24 / 26, gate/up 102 / 57; 3B shapes: 13 / 21, 24 / 43,
-        17 / 21, 46 / 31; 70B shapes (8,192 columns and more): the library's everywhere."""
-        return m <= 192 and -(-n // 256) < 32
+        """Whether a product of 65 to 128 rows is still the few-row kernel's: where the vendor
+        library's output tiles (256 columns wide) would be too few to occupy the GPU's 256
+        compute units, while the few-row kernel divides K among workgroups.  Measured in replayed
+        graphs with the library's fastest candidate (us, few-row kernel / library), 8B shapes at
+        128 rows: o-proj 13.8 / 15.3, down-proj 38.7 / 52.1, but qkv 23.7 / 16.6 and gate/up
+        96 / 58; at 160 rows o-proj 20.2 / 16.4, down-proj 65.6 / 58.7.  3B shapes at 128 rows:
+        o-proj 10.9 / 11.4, down-proj 20.6 / 22.9, qkv 13.7 / 13.2.  So: up to 128 rows and up to
+        4,096 columns."""
+        return m <= 128 and -(-n // 256) <= 16
 
     def _linear_from_attention(self, x: "SplitAttention", w: torch.Tensor, out_dtype, partial_ok: bool):
         """The few-row product fed by attention's unmerged splits, or None where it does not
@@ -495,15 +504,24 @@ class HipOps:
             return SplitSum(ws[: rc * m * n].view(rc, m, n), out_dtype)  # rc: the slices the launch wrote
         return y
 
-    def _library_f32_out(self) -> bool:
-        """Whether this torch's matrix product takes bfloat16 operands and gives float32."""
-        if self._mm_f32 is None:
-            try:
-                a = torch.zeros((16, 16), dtype=torch.bfloat16, device=self.device)
-                self._mm_f32 = torch.mm(a, a, out_dtype=torch.float32).dtype == torch.float32
-            except (TypeError, RuntimeError):
-                self._mm_f32 = False
-        return self._mm_f32
+    LIBRARY_WORKSPACE_BYTES = 64 << 20
+
+    def gemm_library(self, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        """x [M, K] . w [N, K]^T in the vendor library: bfloat16 operands with 16-byte aligned rows,
+        float32 accumulation, the result bfloat16 or float32.  Every shape's algorithm is chosen
+        when the shape is first met (for up to 256 rows the fastest of the library's own
+        candidates, timed then; else its first) and kept."""
+        m, k = x.shape
+        n = w.shape[0]
+        if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[1] != k or x.stride(1) != 1 or w.stride(1) != 1:
+            raise KernelError(f"gemm_library: operands {tuple(x.shape)} {x.dtype} and {tuple(w.shape)} {w.dtype}")
+        if self._library_workspace is None:
+            self._library_workspace = torch.empty(self.LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=self.device)
+        y = torch.empty((m, n), dtype=out_dtype, device=x.device)
+        self._check(self.lib.yk_gemm_library(
+            x.data_ptr(), w.data_ptr(), y.data_ptr(), _code(out_dtype), m, n, k, x.stride(0), w.stride(0), n,
+            self._library_workspace.data_ptr(), self._library_workspace.numel(), None, self._stream()))
+        return y
 
     def gemm_fma(self, x, w, out_dtype):
         m, k = x.shape
