@@ -686,7 +686,8 @@ def test_attention_long_col_tiles_policy():
     assert HipOps.attention_long_col_tiles(512, 0) == 1  # a 2,048-token prompt that starts from nothing
     assert HipOps.attention_long_col_tiles(1024, 0) == 2  # a 4,096-token one: workgroups enough to balance
     assert HipOps.attention_long_col_tiles(512, 6144) == 2  # 2,048 tokens against 6,144 cached, 8 kv heads
-    assert HipOps.attention_long_col_tiles(128, 3584) == 1  # one 512-token portion: too few workgroups
+    assert HipOps.attention_long_col_tiles(128, 3584) == 2  # one 512-token portion: few workgroups, but their keys are split
+    assert HipOps.attention_long_col_tiles(128, 512) == 1
 
 
 def test_attention_long_splits_policy():
@@ -696,6 +697,8 @@ def test_attention_long_splits_policy():
     assert HipOps.attention_long_splits(256, 64) == 3  # a 512-token portion against 4,096 keys
     assert HipOps.attention_long_splits(8, 400) == 16 and HipOps.attention_long_splits(8, 20) == 2
     assert HipOps.attention_long_splits(8, 4) == 1
+    assert HipOps.attention_long_splits(120, 64, col_tiles=2) == 4 and HipOps.attention_long_splits(240, 64, col_tiles=2) == 2
+    assert HipOps.attention_long_splits(400, 64) == 1  # two splits would start a second, nearly empty round
 
 
 def test_attention_plan_covers_the_launch():

@@ -338,14 +338,17 @@ class HipOps:
     def attention_long_col_tiles(workgroups: int, fewest_keys: int) -> int:
         """Column tiles per wave for a step's long spans.  ``workgroups``: how many the
         larger tiles (two column tiles a wave) would make; ``fewest_keys``: the fewest keys
-        any of the spans has cached before it.  Two where those workgroups are enough to fill
-        the GPU twice over, or to fill it once when no span starts from nothing (a prompt from
-        nothing has tiles with a few keys and tiles with all of them: small tiles balance
-        that better); else one.  Measured on the 8B shape (us, one / two): a whole 2,048-token
-        prompt 81 / 99, a whole 4,096-token one 272 / 242, 2,048 tokens against 6,144 cached
-        461 / 341, four 512-token portions against 3,584 cached 247 / 189, one such portion
-        73 / 80."""
-        return 2 if workgroups >= 1024 or (workgroups >= 512 and fewest_keys >= 1024) else 1
+        any of the spans has cached before it.  Two where those workgroups fill the GPU twice
+        over, or where no span starts from nothing: every block of keys staged through LDS
+        then serves twice the columns, and where the tiles are few the keys are split across
+        workgroups (``attention_long_splits``).  One for prompts from nothing: they have tiles
+        with a few keys and tiles with all of them, which small tiles balance better.
+        Measured on the 8B shape (us, one / two, each with its own splits): a whole 2,048-token
+        prompt 70 / 77, a whole 4,096-token one 232 / 204, 2,048 tokens against 6,144 cached
+        396 / 318, four 512-token portions against 3,584 cached 228 / 182, a 480-token portion
+        against 3,616 cached 72 / 65, against 7,200 cached 116 / 103, two such portions
+        124 / 111."""
+        return 2 if workgroups >= 1024 or fewest_keys >= 1024 else 1
 
     # ------------------------------------------------------------------ embedding
     def embed(self, token_ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
@@ -653,13 +656,17 @@ class HipOps:
         return 4, max(1, min(-(-par // 4), 256))
 
     @staticmethod
-    def attention_long_splits(workgroups: int, key_blocks: int) -> int:
+    def attention_long_splits(workgroups: int, key_blocks: int, col_tiles: int = 1) -> int:
         """Splits of the keys for the long-span kernel: one where the tiles alone fill the GPU
         (a prompt of a few thousand tokens); more where few tiles meet a long context (a
-        portion of a prompt whose earlier portions are cached), at least 8 key blocks a split."""
-        if workgroups >= 512:
-            return 1
-        return max(1, min(-(-768 // workgroups), key_blocks // 8, 16))
+        portion of a prompt whose earlier portions are cached): as many as still leave all
+        workgroups on the GPU at once (three a compute unit with one column tile a wave, two
+        with two; a second, partly filled round costs more than the finer split gains: a
+        480-token portion against 3,616 cached, one column tile, 3 / 4 / 5 splits 71.8 / 76.4 /
+        73.3 us; two column tiles, 3 / 4 / 5 splits 74.3 / 64.5 / 76.9), at least 8 key blocks
+        a split."""
+        slots = 768 if col_tiles == 1 else 512
+        return max(1, min(slots // max(1, workgroups), key_blocks // 8, 16))
 
     def attention_can_rotate(self, act_dtype: torch.dtype, head_dim: int) -> bool:
         """Whether ``attention`` takes ``rope=`` for such a mixer: the matrix-core kernel for
@@ -704,7 +711,7 @@ class HipOps:
             n_long = long_tiles.shape[0]
             hpt = self._ask("yk_attn_heads_per_tile", n_heads, n_kv)
             groups = n_long * n_kv * (-(-(n_heads // n_kv) // hpt))
-            long_splits = long_plan if long_plan is not None else self.attention_long_splits(groups, max(1, -(-ctx.max_ctx // 64)))
+            long_splits = long_plan if long_plan is not None else self.attention_long_splits(groups, max(1, -(-ctx.max_ctx // 64)), int(long_col_tiles))
             ws_floats = self._ask("yk_attn_mfma_workspace", 4 * long_col_tiles * n_long, n_heads, n_kv, head_dim, long_splits)
             ws = self._ws(ws_floats) if ws_floats else None
             self._check(
