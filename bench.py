@@ -365,7 +365,7 @@ def main() -> int:
     ap.add_argument("--mixed", action="store_true", help="measure mixed steps instead: 32 decode streams beside portions of 4,096-token prompts")
     ap.add_argument("--portion", type=int, default=480, help="tokens of a prompt portion in --mixed steps (with the 32 decoded tokens: 512 rows, as the scheduler cuts under a budget of 512)")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel (for hardware counters)")
-    ap.add_argument("--shape", choices=("8b", "3b", "70b"), default="8b", help="layer sizes (default: the 8B shape of the headline)")
+    ap.add_argument("--shape", choices=("8b", "3b", "1b", "70b"), default="8b", help="layer sizes (default: the 8B shape of the headline)")
     ap.add_argument("--sample", action="store_true", help="time instead the choice of a token alone (greedy and each sampling rule) at the shape's vocabulary for --batch rows")
     ap.add_argument("--probe", action="store_true", help="measure instead what a plain streaming read and a plain matrix-core loop reach on this card")
     args = ap.parse_args()

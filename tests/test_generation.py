@@ -308,7 +308,7 @@ def test_engine_over_random_weights_of_a_named_shape():
     line's --random).  The same seed gives the same tokens, another seed others."""
     from yalis_amd.models.presets import SHAPES, shape
 
-    assert {"8b", "3b", "70b", "tiny-a", "tiny-b"} <= set(SHAPES)
+    assert {"8b", "3b", "1b", "70b", "tiny-a", "tiny-b"} <= set(SHAPES)
     label, cfg = shape("tiny-b")
     ic = InferenceConfig(max_batch_size=2, max_length_of_generated_sequences=64, temperature=0.0)
 

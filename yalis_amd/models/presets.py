@@ -26,6 +26,8 @@ _LLAMA3_SCALING = {"rope_type": "llama3", "low_freq_factor": 1.0, "high_freq_fac
                    "original_max_position_embeddings": 8192}
 LLAMA32_3B = dict(LLAMA3_8B, hidden_size=3072, num_hidden_layers=28, num_attention_heads=24, intermediate_size=8192,
                   rope_scaling=dict(_LLAMA3_SCALING, factor=32.0), tie_word_embeddings=True)
+LLAMA32_1B = dict(LLAMA3_8B, hidden_size=2048, num_hidden_layers=16, num_attention_heads=32, head_dim=64, intermediate_size=8192,
+                  rope_scaling=dict(_LLAMA3_SCALING, factor=32.0), tie_word_embeddings=True)
 LLAMA31_70B = dict(LLAMA3_8B, hidden_size=8192, num_hidden_layers=80, num_attention_heads=64, intermediate_size=28672,
                    rope_scaling=dict(_LLAMA3_SCALING, factor=8.0))
 # two shapes of a few thousand parameters that differ in every size and option
@@ -47,6 +49,7 @@ TINY_B = {
 SHAPES: Dict[str, Tuple[str, dict]] = {
     "8b": ("Llama-3-8B", LLAMA3_8B),
     "3b": ("Llama-3.2-3B", LLAMA32_3B),
+    "1b": ("Llama-3.2-1B", LLAMA32_1B),
     "70b": ("Llama-3.1-70B", LLAMA31_70B),
     "tiny-a": ("tiny Llama A", TINY_A),
     "tiny-b": ("tiny Llama B", TINY_B),
