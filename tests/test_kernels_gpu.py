@@ -183,6 +183,33 @@ def test_gemm_mfma_skinny_chunk_lengths(ops, chunk, forced):
         assert torch.equal(got, ops.gated_act(ops.linear(x, packed, torch.bfloat16), "silu", torch.bfloat16, group=group))
 
 
+def test_gemm_mfma_skinny_eight_waves(ops, forced):
+    """With more than 32 rows of x a workgroup may have eight waves (128 weight rows on one
+    staged copy of x): the same sums in the same order as with four, so the same bits, on
+    sizes that are no multiples of the workgroup's rows or of the chunk, split and unsplit,
+    plain and with the activation in the epilogue.  Eight waves asked for with fewer rows of
+    x are four."""
+    for m, n, k in [(64, 200, 4096), (50, 515, 328), (40, 1040, 2056), (33, 96, 1000)]:
+        x = rnd((m, k), torch.bfloat16, 6)
+        w = rnd((n, k), torch.bfloat16, 7)
+        for slices in (1, 3):
+            forced(waves=4, slices=slices)
+            four = ops.gemm_mfma_skinny(x, w, torch.float32)
+            forced(waves=8, slices=slices)
+            eight = ops.gemm_mfma_skinny(x, w, torch.float32)
+            assert torch.equal(four, eight), (m, n, k, slices)
+            close(eight, x.double().cpu() @ w.double().cpu().T, 2e-5 * math.sqrt(k), 1e-5)
+    x = rnd((64, 1024), torch.bfloat16, 30, 0.7)
+    packed, group = ops.pack_gate_up(rnd((264, 1024), torch.bfloat16, 31, 0.05), rnd((264, 1024), torch.bfloat16, 32, 0.05))
+    forced(waves=8)
+    got = ops.gate_up_act(x, packed, group, "silu", torch.bfloat16)
+    assert torch.equal(got, ops.gated_act(ops.linear(x, packed, torch.bfloat16), "silu", torch.bfloat16, group=group))
+    few = rnd((8, 1024), torch.bfloat16, 33)
+    eight = ops.gemm_mfma_skinny(few, packed, torch.float32)
+    forced(waves=4)
+    assert torch.equal(eight, ops.gemm_mfma_skinny(few, packed, torch.float32))
+
+
 def test_forced_slice_counts_reach_the_consumers(ops, forced):
     """The number of K slices a product leaves behind is what the launch says it wrote, also
     when the plan is forced after the library was first asked about the shape."""
