@@ -322,6 +322,37 @@ def test_long_spans_that_look_pages_up_in_the_block_table(mode):
 
 
 @pytest.mark.gpu
+def test_portions_behind_a_long_cached_context():
+    """A prompt of 1,400 tokens in portions of 1,100, 170, 100 and 30: the later portions are long
+    spans behind more than 1,024 cached keys, which the attention part gives two column tiles a
+    wave with the keys split across workgroups, by its own choice; the first one starts from
+    nothing and gets one.  Every row's logits are the plain implementation's."""
+    cfg = dict(ALL["D"], max_position_embeddings=2048)
+    weights = P.random_weights(cfg, seed=21)
+    reqs = C.make_requests(cfg, [1400], seed=22)
+    want = C.plain_logits(cfg, weights, reqs, True)
+    steps = C.trace_portions(reqs, sizes=(1100, 170, 100, 30))
+    assert [len(s["entries"][0]["tokens"]) for s in steps] == [1100, 170, 100, 30]
+    ops = ops_for("cuda:0")
+    chosen = []
+    kept = ops.attention
+
+    def spy(*a, **k):
+        chosen.append((k.get("long_col_tiles", 1), None if a[12] is None else int(a[12].shape[0])))
+        return kept(*a, **k)
+
+    ops.attention = spy
+    try:
+        runner = C.make_runner(cfg, weights, "bfloat16", "cuda:0", ops, 64, C.pages_needed(steps, reqs, 64))
+        got, _ = C.run_trace(runner, steps)
+    finally:
+        del ops.attention
+    C.assert_matches(got, want, True, "portions behind a long cached context")
+    layers = cfg["num_hidden_layers"]
+    assert [c[0] for c in chosen[::layers]] == [1, 2, 2, 2], chosen[::layers]
+
+
+@pytest.mark.gpu
 def test_full_width_replay_eight_layers_float32(capsys):
     """The widths of the 8B shape at a quarter of its depth, true float32: the largest
     difference from the plain implementation over whole prompts and over single tokens stays
