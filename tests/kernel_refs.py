@@ -45,10 +45,10 @@ def rmsnorm(x, weight, eps, unit_offset, out_dtype):
 
 
 def linear(x, w, out_dtype, partial_ok=False, bias=None):
-    y = (x.to(torch.float32) @ w.to(torch.float32).T).to(out_dtype)
-    if bias is not None:  # the product is rounded first, then the bias is added and the sum rounded
-        y = (y.to(torch.float32) + bias.to(torch.float32)).to(out_dtype)
-    return y
+    y = x.to(torch.float32) @ w.to(torch.float32).T
+    if bias is not None:  # added to the float32 product, one rounding (torch's addmm, the reference's biased Linear)
+        y = y + bias.to(torch.float32)
+    return y.to(out_dtype)
 
 
 def rope_append(qkv, n_heads, n_kv, head_dim, positions, cos, sin, rotary_dim, interleaved,

@@ -15,10 +15,10 @@ from yalis_amd.models.llama import LlamaConfig
 from yalis_amd.weights.loader import TensorSpec, WeightsError, open_tensors, target_dtype
 
 
-def load_tensors(folder, specs, engine_dtype, device):
+def load_tensors(folder, specs, engine_dtype, device, wide_tensors="auto"):
     """Every tensor of ``specs`` through the loader that generation uses (``open_tensors``:
     the folder is checked as a whole, then each tensor is read when asked for)."""
-    source = open_tensors(folder, specs, {n: 1 for n in specs}, engine_dtype, device)
+    source = open_tensors(folder, specs, {n: 1 for n in specs}, engine_dtype, device, wide_tensors=wide_tensors)
     return {n: source[n] for n in specs}
 from yalis_amd.weights.random_init import write_random_model
 from yalis_amd.weights.safetensors_io import SafetensorsError, index_folder, read_tensor, write_dict
@@ -151,6 +151,7 @@ def test_precision_rule():
     assert target_dtype("F16", "float", "bfloat16") == torch.bfloat16
     assert target_dtype("F32", "float", "bfloat16") == torch.float32, "a tensor stored in 32 bits stays so"
     assert target_dtype("BF16", "float", "float32") == torch.float32
+    assert target_dtype("F32", "float", "bfloat16", keep_wide=False) == torch.bfloat16
     assert target_dtype("I64", "int", "bfloat16") == torch.int32
 
 
@@ -170,10 +171,8 @@ def test_random_folder_loads_back_bit_exact(tmp_path):
     assert abs(w.std().item() - 0.02) < 0.002 and abs(w.mean().item()) < 0.002
     n = loaded["model.norm.weight"].float()
     assert abs(n.mean().item() - 1.0) < 0.05 and 0.05 < n.std().item() < 0.15
-    # the 32-bit engine widens; a 32-bit folder stays 32-bit in a bfloat16 engine
+    # the 32-bit engine widens
     assert load_tensors(folder, specs, "float32", "cpu")["model.norm.weight"].dtype == torch.float32
-    f32 = write_random_model(str(tmp_path / "a32"), TINY_A, seed=0, dtype="float32")
-    assert load_tensors(f32, tensor_specs_for(TINY_A), "bfloat16", "cpu")["model.norm.weight"].dtype == torch.float32
     assert json.load(open(os.path.join(folder, "config.json")))["architectures"] == ["LlamaForCausalLM"]
 
 
@@ -198,11 +197,37 @@ def test_sixteen_bit_floats_of_the_other_kind_and_wide_matrices(tmp_path, caplog
     log.propagate = True  # (the package's loggers keep to themselves; the test listens in)
     try:
         with caplog.at_level(logging.WARNING, logger="yalis_amd"):
-            got = load_tensors(f32, specs, "bfloat16", "cpu")
+            got = load_tensors(f32, specs, "bfloat16", "cpu", wide_tensors="keep")
     finally:
         log.propagate = False
     assert got["lm_head.weight"].dtype == torch.float32
     assert sum("stored in 32 bits" in r.getMessage() for r in caplog.records) == 1
+
+
+def test_tensors_stored_in_32_bits(tmp_path):
+    """The bfloat16 engine: a checkpoint stored wholly in 32 bits is narrowed (the reference
+    casts every tensor to its parameter's dtype, yalis/model_loading.py:172-173), rounding to
+    nearest even; single 32-bit tensors inside a 16-bit checkpoint stay 32-bit; "keep" and
+    "cast" override both ways; the float32 engine is not affected."""
+    specs = tensor_specs_for(TINY_A)
+    f32 = write_random_model(str(tmp_path / "w"), TINY_A, seed=0, dtype="float32")
+    stored = {n: read_tensor(e) for n, e in index_folder(f32).items()}
+    got = load_tensors(f32, specs, "bfloat16", "cpu")
+    assert all(t.dtype == torch.bfloat16 for t in got.values())
+    assert torch.equal(got["lm_head.weight"], stored["lm_head.weight"].to(torch.bfloat16))
+    assert all(t.dtype == torch.float32 for t in load_tensors(f32, specs, "bfloat16", "cpu", wide_tensors="keep").values())
+    assert all(torch.equal(t, stored[n]) for n, t in load_tensors(f32, specs, "float32", "cpu").items())
+    # a 16-bit checkpoint whose norm weights are stored wide
+    mixed = {n: (t if n.endswith("norm.weight") else t.to(torch.bfloat16)) for n, t in stored.items()}
+    os.makedirs(tmp_path / "m")
+    json.dump(TINY_A, open(tmp_path / "m" / "config.json", "w"))
+    write_dict(str(tmp_path / "m" / "model.safetensors"), mixed)
+    got = load_tensors(str(tmp_path / "m"), specs, "bfloat16", "cpu")
+    assert got["model.norm.weight"].dtype == torch.float32 and torch.equal(got["model.norm.weight"], stored["model.norm.weight"])
+    assert got["lm_head.weight"].dtype == torch.bfloat16
+    assert load_tensors(str(tmp_path / "m"), specs, "bfloat16", "cpu", wide_tensors="cast")["model.norm.weight"].dtype == torch.bfloat16
+    with pytest.raises(ValueError, match="wide_tensors"):
+        load_tensors(f32, specs, "bfloat16", "cpu", wide_tensors="sometimes")
 
 
 def test_one_error_lists_everything_wrong(tmp_path):

@@ -69,11 +69,14 @@ def test_replay_modes(backend, name, mode):
         first_owner = {}
         reused = False
         for held in rp.page_log:
-            for rid, pages in held.items():
-                for p in pages:
-                    if p in first_owner and first_owner[p] != rid:
-                        reused = True
-                    first_owner.setdefault(p, rid)
+            for rid, tables in held.items():
+                for g, pages in enumerate(tables):
+                    for p in pages:
+                        if p < 0:
+                            continue
+                        if (g, p) in first_owner and first_owner[(g, p)] != rid:
+                            reused = True
+                        first_owner.setdefault((g, p), rid)
         assert reused, "the trace was meant to reuse pages"
 
 
@@ -134,6 +137,74 @@ def test_full_width_replay(dtype):
         C.assert_matches(got, want, bf16, f"full width/{mode}", f32_tol=1e-4)
         runner.pages.audit()
         assert runner.pages.live_requests() == 0
+
+
+# The widths of the other published shapes, one layer each and a small vocabulary (the 128k
+# head is covered by FULL_WIDTH): rows of weights 4, 6 and 16 KiB apart, K slices of 2,048 and
+# more in the few-row product, 65- to 128-row products on 2,048- and 3,072-column matrices,
+# three and eight query heads a kv head, head size 64.
+def _width_cfg(hidden, heads, kv, head_dim, inter, vocab, scaling_factor, tied):
+    return {
+        "architectures": ["LlamaForCausalLM"], "hidden_size": hidden, "num_hidden_layers": 1,
+        "num_attention_heads": heads, "num_key_value_heads": kv, "head_dim": head_dim, "intermediate_size": inter,
+        "vocab_size": vocab, "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
+        "rope_scaling": {"rope_type": "llama3", "factor": scaling_factor, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                         "original_max_position_embeddings": 8192},
+        "max_position_embeddings": 1024, "tie_word_embeddings": tied,
+    }
+
+
+OTHER_WIDTHS = {
+    "1b": _width_cfg(2048, 32, 8, 64, 8192, 1000, 32.0, True),
+    "3b": _width_cfg(3072, 24, 8, 128, 8192, 1003, 32.0, True),
+    "70b": _width_cfg(8192, 64, 8, 128, 28672, 520, 8.0, False),
+}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", ["1b", "3b", "70b"])
+def test_other_widths_replay(shape, dtype):
+    """Whole prompts (37 to 100 rows a product), bulk + single tokens, and mixed steps at the
+    layer widths of the Llama-3.2-1B, -3B and Llama-3.1-70B shapes."""
+    cfg = OTHER_WIDTHS[shape]
+    bf16 = dtype == "bfloat16"
+    weights = P.random_weights(cfg, seed=31)
+    reqs = C.make_requests(cfg, [100, 37, 70, 5, 66], seed=32)
+    want = C.plain_logits(cfg, weights, reqs, bf16)
+    for mode, make in (("whole", C.trace_whole), ("tail", lambda r: C.trace_tail(r, tail=6)), ("mixed", C.trace_mixed)):
+        steps = make(reqs)
+        runner = C.make_runner(cfg, weights, dtype, "cuda:0", ops_for("cuda:0"), 64, C.pages_needed(steps, reqs, 64))
+        got, _ = C.run_trace(runner, steps)
+        C.assert_matches(got, want, bf16, f"{shape} widths/{mode}", f32_tol=1e-4)
+        runner.pages.audit()
+        assert runner.pages.live_requests() == 0
+        del runner
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replayed_decode_crosses_context_buckets(dtype):
+    """Captured decode steps are keyed by the power-of-two bucket of the longest context, which
+    sizes the attention's splits.  One request decodes from 250 to 270 cached tokens, another
+    from 1,020 to 1,030: each crosses a bucket's edge (256, 1,024) with graphs on, so each is
+    served by two graphs, and every step's logits are the plain implementation's."""
+    cfg = dict(ALL["D"], max_position_embeddings=2048)
+    bf16 = dtype == "bfloat16"
+    weights = P.random_weights(cfg, seed=23)
+    reqs = C.make_requests(cfg, [270, 1030], seed=24)
+    want = C.plain_logits(cfg, weights, reqs, bf16)
+    for rid, first in (("r0", 250), ("r1", 1020)):
+        toks = reqs[rid]
+        steps = [{"step": 0, "entries": [{"id": rid, "tokens": toks[:first], "want": []}], "end": []}]
+        steps += [{"step": 1 + j - first, "entries": [{"id": rid, "tokens": [toks[j]], "want": [0]}], "end": []} for j in range(first, len(toks))]
+        runner = C.make_runner(cfg, weights, dtype, "cuda:0", ops_for("cuda:0"), 64, -(-len(toks) // 64))
+        assert runner.use_graphs
+        got, _ = C.run_trace(runner, steps)
+        assert runner.graph_replays == len(toks) - first
+        assert sorted(runner._graphs) == [(1, 256 if first == 250 else 1024), (1, 512 if first == 250 else 2048)], sorted(runner._graphs)
+        C.assert_matches({rid: got[rid]}, {rid: want[rid][first:]}, bf16, f"decode across a bucket's edge from {first}")
+        del runner
 
 
 @pytest.mark.gpu

@@ -301,6 +301,18 @@ def test_reset_kv_cache_rebuilds_the_pool(tmp_path):
     assert eng.runner.config.max_num_seqs == 4
     with pytest.raises(ValueError):
         eng.reset_kv_cache(0)
+    # after a call that went through, the old pool is gone once the new one is made: nothing
+    # (the last call's scheduler included) keeps the old runner or its pages alive
+    import gc
+    import weakref
+
+    old_runner, old_pages = weakref.ref(eng.runner), weakref.ref(eng.runner.memory.keys[0])
+    eng.reset_kv_cache(2)
+    gc.collect()
+    assert old_runner() is None and old_pages() is None
+    assert eng.runner.config.max_num_seqs == 2 and eng.runner.pages.free_pages(0) == 8
+    out, _ = eng.generate(prompts[:2], tokens_to_generate=3)
+    assert out.tolist() == [P.greedy_generate(cfg, weights, p, 3) for p in prompts[:2]]
 
 
 def test_engine_over_random_weights_of_a_named_shape():

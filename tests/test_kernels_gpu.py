@@ -372,7 +372,7 @@ def test_library_product(ops, tuned):
             assert torch.equal(first, ops.gemm_library(x, w, torch.bfloat16))
             close(ops.gemm_library(x, w, torch.float32), want, 1e-4, 1e-5)
     finally:
-        ops.tune_library_products(True)
+        ops.tune_library_products(False)
     from yalis_amd.ops.hip import KernelError
 
     with pytest.raises(KernelError, match="gemm_library"):
@@ -582,21 +582,36 @@ def _bits(t):
     return t.contiguous().view(torch.int16)
 
 
-@pytest.mark.parametrize("plan", [None, (1, 1), (4, 1), (4, 3), (1, 4)])
-@pytest.mark.parametrize("slices", [1, 3])
-@pytest.mark.parametrize("h,g,d,rd,page,inter", [
-    (32, 8, 128, 128, 64, False), (6, 2, 128, 128, 64, False), (6, 3, 64, 32, 16, False), (8, 1, 64, 64, 128, True),
-    (32, 1, 128, 64, 32, False), (24, 8, 128, 128, 64, False), (4, 4, 64, 0, 64, False),
-])
-def test_attention_rotates_and_appends_in_its_launch(ops, plan, slices, h, g, d, rd, page, inter):
+def _rotary_inside_cases():
+    shapes = [(32, 8, 128, 128, 64, False), (6, 2, 128, 128, 64, False), (6, 3, 64, 32, 16, False), (8, 1, 64, 64, 128, True),
+              (32, 1, 128, 64, 32, False), (24, 8, 128, 128, 64, False), (4, 4, 64, 0, 64, False)]
+    for shape in shapes:
+        for slices in (1, 3):
+            for plan in (None, (1, 1), (4, 1), (4, 3), (1, 4)):
+                yield (*shape, slices, plan, 0)
+    # a window: its edge inside the block that holds the token, in an earlier block, in a split
+    # that another workgroup owns; pages below it given back
+    for shape in shapes[:4] + shapes[6:]:
+        for window in (24, 100):
+            for slices, plan in ((1, None), (3, (4, 3)), (1, (1, 4)), (3, (4, 1))):
+                yield (*shape, slices, plan, window)
+
+
+@pytest.mark.parametrize("h,g,d,rd,page,inter,slices,plan,window", list(_rotary_inside_cases()))
+def test_attention_rotates_and_appends_in_its_launch(ops, plan, slices, h, g, d, rd, page, inter, window):
     """A step of single tokens: rotary + append inside the attention launch give the bits of
     rotary + append followed by attention, in the output and in the pages, whether the
     projection comes as bfloat16 rows or as float32 K slices, however the keys are divided,
     with the token's own key first, last or in the middle of a block of 64 (the slot it goes to
-    holds NaN before), in tiled and in plain pages; and both agree with the plain reference."""
+    holds NaN before), in tiled and in plain pages; and both agree with the plain reference.
+    With a window: contexts one short of it, equal to it and beyond, the pages that lie wholly
+    below the window given back (-1 in the block table, NaN where they were), and the key just
+    outside the window made large, so that a window off by one would let it take the output."""
     from yalis_amd.ops.hip import RopeInLaunch, SplitSum
 
     cached = [0, 1, 31, 32, 63, 64, 65, 700, 1500, 127, 190]
+    if window:
+        cached += [window - 1, window, window + 1]
     n = len(cached)
     gen = torch.Generator().manual_seed(31)
     n_pages = sum(-(-(c + 1) // page) for c in cached) + 3
@@ -610,9 +625,14 @@ def test_attention_rotates_and_appends_in_its_launch(ops, plan, slices, h, g, d,
         used += n_p
         k = torch.randn((c, g, d), generator=gen).to(torch.bfloat16)
         v = torch.randn((c, g, d), generator=gen).to(torch.bfloat16)
+        first_seen = max(0, c - window + 1) if window else 0  # the oldest key the token at position c sees
+        if window and first_seen > 0:
+            k[first_seen - 1] *= 40.0  # just outside: were it seen, it would take half the heads' outputs
+            table[: first_seen // page] = -1  # pages wholly below the window: given back, never filled
         for pos in range(c):
-            kc[table[pos // page], :, pos % page, :] = k[pos]
-            vc[table[pos // page], :, :, pos % page] = v[pos]
+            if table[pos // page] >= 0:
+                kc[table[pos // page], :, pos % page, :] = k[pos]
+                vc[table[pos // page], :, :, pos % page] = v[pos]
         seqs.append(SeqSpan(tokens=[0], first_position=c, block_tables=[table], state_slot=0))
     hb = build_host_batch(seqs, 1, page)
     tpt, big = ops.attention_tokens_per_tile(h, g), ops.attention_long_span_tile(h, g)
@@ -634,10 +654,10 @@ def test_attention_rotates_and_appends_in_its_launch(ops, plan, slices, h, g, d,
     # rotary + append, then attention
     kc_a, vc_a = device_cache(ops, kc.clone(), vc.clone())
     q = ops.rope_append(give(), h, g, d, positions, cos, sin, rd, inter, kc_a, vc_a, slots, page)
-    out_a = ops.attention(q, h, g, d, kc_a, vc_a, page, scale, 0, ctx, 0, dev["tiles"], plan=plan)
+    out_a = ops.attention(q, h, g, d, kc_a, vc_a, page, scale, window, ctx, 0, dev["tiles"], plan=plan)
     # both in one launch
     kc_b, vc_b = device_cache(ops, kc.clone(), vc.clone())
-    out_b = ops.attention(give(), h, g, d, kc_b, vc_b, page, scale, 0, ctx, 0, dev["tiles"], plan=plan,
+    out_b = ops.attention(give(), h, g, d, kc_b, vc_b, page, scale, window, ctx, 0, dev["tiles"], plan=plan,
                           rope=RopeInLaunch(cos, sin, rd, inter, True))
     assert torch.isfinite(out_b.float()).all()
     assert torch.equal(_bits(out_a), _bits(out_b))
@@ -646,7 +666,7 @@ def test_attention_rotates_and_appends_in_its_launch(ops, plan, slices, h, g, d,
     # that reads another entry's cache)
     q_rows = give()
     q_rows = SplitSum(q_rows.tensor[:, :, : h * d].contiguous(), torch.bfloat16) if slices > 1 else q_rows[:, : h * d].contiguous()
-    out_c = ops.attention(q_rows, h, g, d, kc_b, vc_b, page, scale, 0, ctx, 0, dev["tiles"], plan=plan,
+    out_c = ops.attention(q_rows, h, g, d, kc_b, vc_b, page, scale, window, ctx, 0, dev["tiles"], plan=plan,
                           rope=RopeInLaunch(cos, sin, rd, inter, False))
     assert torch.equal(_bits(out_a), _bits(out_c))
     # the plain reference
@@ -656,7 +676,7 @@ def test_attention_rotates_and_appends_in_its_launch(ops, plan, slices, h, g, d,
     R.rope_append(qkv_r, h, g, d, cpu["positions"], None if cos is None else cos.cpu(), None if sin is None else sin.cpu(), rd, inter, kc_r, vc_r, cpu["slots_g0"], page)
     kc_r, vc_r = kc_r.to(torch.bfloat16).float(), vc_r.to(torch.bfloat16).float()
     q_r = qkv_r.view(n, -1, d)[:, :h].reshape(n, h * d).to(torch.bfloat16).float()
-    want = R.attention(q_r, h, g, d, kc_r, vc_r, page, scale, 0, types.SimpleNamespace(arrays=cpu), 0, None)
+    want = R.attention(q_r, h, g, d, kc_r, vc_r, page, scale, window, types.SimpleNamespace(arrays=cpu), 0, None)
     close(out_b, want, 2e-2, 2**-6)
 
 
@@ -707,37 +727,59 @@ def test_attention_long_spans_with_split_keys(ops, splits, h, g, d, page, col_ti
         close(got, want, 2e-2, 2**-6)
 
 
-def test_attention_long_col_tiles_policy():
+def test_attention_policies_keep_their_invariants():
+    """What the launch policies must hold whatever their constants are: a plan has one or four
+    waves and at least one split, never more waves than key blocks could feed; the long-span
+    kernel gets one or two column tiles, and splits only as far as all workgroups stay on the
+    GPU at once."""
     from yalis_amd.ops.hip import HipOps
-
-    assert HipOps.attention_long_col_tiles(512, 0) == 1  # a 2,048-token prompt that starts from nothing
-    assert HipOps.attention_long_col_tiles(1024, 0) == 2  # a 4,096-token one: workgroups enough to balance
-    assert HipOps.attention_long_col_tiles(512, 6144) == 2  # 2,048 tokens against 6,144 cached, 8 kv heads
-    assert HipOps.attention_long_col_tiles(128, 3584) == 2  # one 512-token portion: few workgroups, but their keys are split
-    assert HipOps.attention_long_col_tiles(128, 512) == 1
-
-
-def test_attention_long_splits_policy():
-    from yalis_amd.ops.hip import HipOps
-
-    assert HipOps.attention_long_splits(1024, 32) == 1  # a whole prompt: tiles fill the GPU
-    assert HipOps.attention_long_splits(256, 64) == 3  # a 512-token portion against 4,096 keys
-    assert HipOps.attention_long_splits(8, 400) == 16 and HipOps.attention_long_splits(8, 20) == 2
-    assert HipOps.attention_long_splits(8, 4) == 1
-    assert HipOps.attention_long_splits(120, 64, col_tiles=2) == 4 and HipOps.attention_long_splits(240, 64, col_tiles=2) == 2
-    assert HipOps.attention_long_splits(400, 64) == 1  # two splits would start a second, nearly empty round
-
-
-def test_attention_plan_covers_the_launch():
-    from yalis_amd.ops.hip import ATTN_TARGET_WAVES, HipOps
 
     for groups in (1, 8, 64, 512, 5000):
         for key_blocks in (1, 2, 5, 16, 128, 2048):
             waves, splits = HipOps.attention_plan(groups, key_blocks)
             assert waves in (1, 4) and 1 <= splits <= 256
-            if key_blocks == 1 or groups >= ATTN_TARGET_WAVES:
-                assert (waves, splits) == (1, 1)
-            assert waves * splits < 2 * 8 + max(key_blocks, 1) * 2
+            assert key_blocks > 1 or (waves, splits) == (1, 1)
+            assert waves * splits < 2 * 8 + key_blocks * 2
+    for workgroups in (1, 8, 120, 256, 400, 1024, 5000):
+        for fewest in (0, 512, 1024, 7000):
+            assert HipOps.attention_long_col_tiles(workgroups, fewest) in (1, 2)
+        for key_blocks in (1, 4, 20, 64, 400):
+            for col_tiles in (1, 2):
+                splits = HipOps.attention_long_splits(workgroups, key_blocks, col_tiles)
+                assert 1 <= splits <= 16
+                assert splits == 1 or (splits * workgroups <= (768 if col_tiles == 1 else 512) and key_blocks // splits >= 8)
+
+
+@pytest.mark.parametrize("h,g,d,page", [(32, 8, 128, 64), (24, 8, 128, 64), (32, 8, 64, 64)])
+def test_attention_gives_one_result_under_every_plan_its_policies_choose(ops, h, g, d, page):
+    """The policies decide from the batch how the keys are divided (waves, splits, column tiles of
+    the long-span kernel).  For workloads on which they decide differently, the result under the
+    policy's own choice is, within rounding, the result with nothing divided and the plain
+    reference's: retuning a policy can change speed only."""
+    from yalis_amd.ops.hip import HipOps
+
+    workloads = {
+        "single tokens behind long contexts": [(2000, 1), (900, 1), (64, 1)],
+        "a few tokens each": [(1500, 3), (0, 2), (700, 4)],
+        "a portion behind a long cached context": [(1400, 200)],
+        "a prompt from nothing": [(0, 300)],
+        "portions beside single tokens": [(1100, 150), (600, 1), (0, 90), (1300, 1)],
+    }
+    seen = set()
+    for what, spans in workloads.items():
+        n_pages = sum(-(-(c + n) // page) for c, n in spans) + 2
+        chosen, want = _attention_case(ops, torch.bfloat16, h, g, d, page, spans, 0, seed=30, n_pages=n_pages)
+        undivided, _ = _attention_case(ops, torch.bfloat16, h, g, d, page, spans, 0, seed=30, n_pages=n_pages, plan=(1, 1), long_plan=1)
+        two, _ = _attention_case(ops, torch.bfloat16, h, g, d, page, spans, 0, seed=30, n_pages=n_pages, col_tiles=2)
+        close(chosen, want, 2e-2, 2**-6)
+        close(undivided, want, 2e-2, 2**-6)
+        close(two, want, 2e-2, 2**-6)
+        # (the parts of a division are merged in float32 and rounded once: what a division can
+        # change is the order of float32 sums, a unit of bfloat16 at most)
+        close(chosen, undivided.float().cpu(), 2e-2, 2**-7)
+        longest = max(c + n for c, n in spans)
+        seen.add(HipOps.attention_plan(len(spans) * g, -(-longest // 64)))
+    assert len(seen) > 1, "the workloads were meant to make the policy choose differently"
 
 
 def test_attention_far_key_stands_out(ops):

@@ -82,6 +82,64 @@ def test_llama3_scaling_regimes():
     assert torch.allclose(P.rope_inv_freq(d, theta, one), plain), "factor 1 changes nothing"
 
 
+def _is_the_reference_table(inv: torch.Tensor, d: int, base: float) -> bool:
+    """What yalis/external/model.py:786-789 says of the unscaled table, stated without the
+    function under test: d/2 frequencies, the first 1, the last base^-((d-2)/d), each a
+    constant factor base^(-2/d) below the one before (theta_i = base^(-2i/d))."""
+    if inv.shape != (d // 2,) or inv.dtype != torch.float32:
+        return False
+    v = inv.double()
+    step = base ** (-2.0 / d)
+    return bool(
+        v[0] == 1.0
+        and abs(v[-1].item() / base ** (-(d - 2.0) / d) - 1) < 1e-5
+        and ((v[1:] / v[:-1]) / step - 1).abs().max().item() < 1e-5
+    )
+
+
+@pytest.mark.parametrize("d,base", [(16, 1e4), (128, 5e5)])
+def test_rope_frequency_table_is_geometric(d, base):
+    """Pins every frequency, not only the first: an exponent i/d or 2i/(d-2) in place of
+    2i/d passes the rotation tests (which build both sides from one table) and fails here."""
+    assert _is_the_reference_table(P.rope_inv_freq(d, base, None), d, base)
+    i = torch.arange(d // 2, dtype=torch.float32)
+    assert not _is_the_reference_table(base ** -(i / d), d, base), "exponent i/d"
+    assert not _is_the_reference_table(base ** -(2 * i / (d - 2)), d, base), "exponent 2i/(d-2)"
+    assert not _is_the_reference_table(base ** -(2 * (i + 1) / d), d, base), "first frequency below 1"
+    # the engine's own table is built apart from the plain one: the same pin holds it
+    from yalis_amd.parts.rotary import inverse_frequencies
+
+    assert _is_the_reference_table(inverse_frequencies(d, base, None), d, base)
+
+
+def test_llama3_middle_regime_by_hand():
+    """yalis/external/model.py:790-807 on a table made so that one wavelength is known: head
+    size 4 has theta = (1, base^(-1/2)); with base = (orig / 4 pi)^2 the second wavelength is
+    orig / 2, so ratio = 2, smooth = (2 - 1) / (4 - 1) = 1/3 and the adjusted frequency is
+    theta * (2/3 / factor + 1/3).  The first (wavelength 2 pi < orig / 4) stays."""
+    orig, factor = 64, 8.0
+    base = (orig / (4 * math.pi)) ** 2
+    s = {"factor": factor, "low_freq_factor": 1.0, "high_freq_factor": 4.0, "original_max_position_embeddings": orig}
+    theta1 = 4 * math.pi / orig
+    got = P.rope_inv_freq(4, base, s)
+    assert got[0].item() == 1.0
+    assert abs(got[1].item() / (theta1 * (2.0 / 3.0 / factor + 1.0 / 3.0)) - 1) < 1e-5
+    # mistakes this separates: interpolating wavelengths instead of frequencies, smooth and
+    # 1 - smooth exchanged, the ratio taken as wavelen / orig
+    assert abs(got[1].item() / (theta1 / (2.0 / 3.0 * factor + 1.0 / 3.0)) - 1) > 0.1
+    assert abs(got[1].item() / (theta1 * (1.0 / 3.0 / factor + 2.0 / 3.0)) - 1) > 0.1
+    # a wavelength of exactly orig / low and beyond: divided by the factor; orig / high and
+    # below: unchanged (the clamps)
+    long_base = (2 * orig / (2 * math.pi)) ** 2  # second wavelength 2 orig
+    assert abs(P.rope_inv_freq(4, long_base, s)[1].item() / (math.pi / orig / factor) - 1) < 1e-5
+    short_base = (orig / 8 / (2 * math.pi)) ** 2  # second wavelength orig / 8
+    assert abs(P.rope_inv_freq(4, short_base, s)[1].item() / (16 * math.pi / orig) - 1) < 1e-5
+    from yalis_amd.parts.rotary import inverse_frequencies
+
+    mine = inverse_frequencies(4, base, dict(s, kind="llama3"))
+    assert abs(mine[1].item() / (theta1 * (2.0 / 3.0 / factor + 1.0 / 3.0)) - 1) < 1e-5
+
+
 def test_attention_is_the_library_routine():
     t, h, g, d = 9, 4, 2, 16
     q, k, v = torch.randn(t, h, d), torch.randn(t, g, d), torch.randn(t, g, d)

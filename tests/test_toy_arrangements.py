@@ -214,8 +214,8 @@ def toy2_plain(weights, tokens, rounder=P._identity):
         return rounder(P.rms_norm(x, w(name), c.eps))
 
     def lin(x, name, bias=False):
-        y = rounder(x @ w(name + ".weight").T)
-        return rounder(y + w(name + ".bias")) if bias else y
+        y = x @ w(name + ".weight").T
+        return rounder(y + w(name + ".bias")) if bias else rounder(y)
 
     def attention(h, p, bias):
         q = rounder(P.apply_rope(lin(h, p + ".q_proj", bias).view(t, c.heads, c.head_dim), cos, sin))

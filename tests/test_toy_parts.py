@@ -319,23 +319,5 @@ def test_toy_model_replays(backend, mode):
 
 
 def _window_tables(rp):
-    return rp.window_tables
-
-
-@pytest.fixture(autouse=True)
-def _log_window_tables(monkeypatch):
-    """Record the windowed group's block tables after every step of a replay."""
-    from yalis_amd.engine.replay import Replayer
-
-    orig = Replayer.run_step
-
-    def run_step(self, step):
-        out = orig(self, step)
-        if not hasattr(self, "window_tables"):
-            self.window_tables = []
-        if len(self.runner.pages.groups) > 1:
-            for h in self.handles.values():
-                self.window_tables.append(self.runner.pages.block_table(h, 1).tolist())
-        return out
-
-    monkeypatch.setattr(Replayer, "run_step", run_step)
+    """The windowed group's block tables after every step of a replay."""
+    return [tables[1] for held in rp.page_log for tables in held.values()]

@@ -19,9 +19,11 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def run_cli(model, dtype, out, steps, max_tokens, extra=()):
+    """``model``: a folder, or ("shape", seed) for --random."""
     text = "".join(json.dumps(s) + "\n" for s in steps)
+    which = ["--model", model] if isinstance(model, str) else ["--random", model[0], "--seed", str(model[1])]
     proc = subprocess.run(
-        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model, "--dtype", dtype,
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), *which, "--dtype", dtype,
          "--out", out, "--max-tokens", str(max_tokens), *extra],
         input=text, capture_output=True, text=True, timeout=600,
     )
@@ -34,8 +36,8 @@ def run_cli(model, dtype, out, steps, max_tokens, extra=()):
 @pytest.mark.gpu
 @pytest.mark.parametrize("stored,dtype", [("bfloat16", "bfloat16"), ("bfloat16", "float32"), ("float32", "bfloat16")])
 def test_trace_run_cli(tmp_path, stored, dtype):
-    """Also covers a folder stored in 32 bits under the bfloat16 engine: such tensors stay
-    32-bit and the products run through the float32 kernels on bfloat16 activations."""
+    """Also covers a folder stored wholly in 32 bits under the bfloat16 engine (narrowed to
+    bfloat16 at load), the files per request and the log of pages."""
     cfg = TINY_C
     folder = write_random_model(str(tmp_path / "m"), cfg, seed=4, dtype=stored)
     weights = {n: read_tensor(e).float() for n, e in index_folder(folder).items()}
@@ -65,6 +67,40 @@ def test_trace_run_cli(tmp_path, stored, dtype):
                 assert (got[r] - ref).abs().max() <= tol, (s["step"], e["id"], base + w)
                 r += 1
             cached[e["id"]] = base + len(e["tokens"])
+    # the same rows again, gathered per request, with their positions and the pages in the log
+    log = [json.loads(l) for l in open(os.path.join(out, "pages.jsonl"))]
+    assert [l["step"] for l in log] == [s["step"] for s in steps]
+    for rid, toks in reqs.items():
+        pos = [p for l in log for p in l["positions"].get(rid, [])]
+        rows = np.fromfile(os.path.join(out, "requests", f"{rid}.f32"), dtype="<f4").reshape(-1, cfg["vocab_size"])
+        assert len(pos) == rows.shape[0] and pos == sorted(pos)
+        assert (torch.from_numpy(rows) - want[rid][pos]).abs().max() <= C.tolerance(want[rid], bf16)
+    owners = {}
+    for l in log:
+        held = [p for tables in l["pages"].values() for p in tables[0] if p >= 0]
+        assert len(held) == len(set(held)), "no page is held twice"
+        for rid, tables in l["pages"].items():
+            for p in tables[0]:
+                owners.setdefault(p, set()).add(rid)
+    assert any(len(o) > 1 for o in owners.values()), "the pool is small enough that pages are used again"
+
+
+@pytest.mark.gpu
+def test_trace_run_cli_with_a_named_shape_and_a_seed(tmp_path):
+    """--random SHAPE --seed S is the model that the random-weights mode writes as a folder
+    from the same configuration and seed: the same logits, bit for bit."""
+    from yalis_amd.models.presets import shape
+
+    cfg = shape("tiny-b")[1]
+    folder = write_random_model(str(tmp_path / "m"), cfg, seed=3, dtype="bfloat16")
+    reqs = C.make_requests(cfg, [40, 130, 1], seed=9)
+    steps = C.trace_portions(reqs)
+    run_cli(folder, "bfloat16", str(tmp_path / "a"), steps, 512, extra=["--page-size", "32"])
+    run_cli(("tiny-b", 3), "bfloat16", str(tmp_path / "b"), steps, 512, extra=["--page-size", "32"])
+    for s in steps:
+        a = np.fromfile(str(tmp_path / "a" / f"{s['step']}.f32"), dtype="<f4")
+        b = np.fromfile(str(tmp_path / "b" / f"{s['step']}.f32"), dtype="<f4")
+        assert a.size == len(s["entries"][0]["want"]) * cfg["vocab_size"] and np.array_equal(a, b)
 
 
 @pytest.mark.gpu

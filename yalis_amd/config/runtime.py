@@ -135,6 +135,7 @@ class EngineConfig:
     decode_graphs: replay steps that hold single tokens only from captured HIP graphs
         (the reference's YALIS_DISABLE_DECODE_CUDAGRAPHS switches the same off,
         yalis/engine.py:44-48).
+    graph_memory_bytes, wide_tensors, tune_library_products: see the fields.
     """
 
     page_size: int = 64
@@ -147,6 +148,17 @@ class EngineConfig:
     # capture steps of single tokens as HIP graphs; YALIS_DISABLE_DECODE_CUDAGRAPHS=1 turns the
     # default off, as it does in the reference
     decode_graphs: bool = field(default_factory=lambda: os.environ.get("YALIS_DISABLE_DECODE_CUDAGRAPHS", "0") != "1")
+    # device memory that captured graphs may hold together (their logits, integer buffers and
+    # private pools); the least recently replayed ones are dropped beyond it
+    graph_memory_bytes: int = 1 << 30
+    # "auto": a checkpoint stored wholly in 32 bits is narrowed to bfloat16 by the bfloat16
+    # engine, as the reference casts every tensor to its parameter's dtype
+    # (yalis/model_loading.py:172-173), while single tensors stored in 32 bits inside a 16-bit
+    # checkpoint stay 32-bit; "keep": every tensor stored in 32 bits stays so; "cast": none does
+    wide_tensors: str = "auto"
+    # time the vendor library's candidates for new product shapes of up to 256 rows and keep the
+    # fastest (the choice then depends on the run); off: its first candidate, the same everywhere
+    tune_library_products: bool = False
 
     def __post_init__(self) -> None:
         self.dtype = canonical_dtype(self.dtype)
@@ -160,6 +172,10 @@ class EngineConfig:
             raise ValueError("max_num_batched_tokens must be positive")
         if self.num_pages is not None and self.num_pages <= 0:
             raise ValueError("num_pages must be positive")
+        if self.wide_tensors not in ("auto", "keep", "cast"):
+            raise ValueError(f"wide_tensors must be 'auto', 'keep' or 'cast', got {self.wide_tensors!r}")
+        if self.graph_memory_bytes < 0:
+            raise ValueError("graph_memory_bytes must not be negative")
 
     def pages_per_request(self) -> int:
         return -(-self.max_model_len // self.page_size)

@@ -694,34 +694,41 @@ extern "C" int yk_gated_act(const void* gu, int src_dtype, int n_splits, int rou
 }
 
 // ------------------------------------------------------------------------------- bias
-// y[m, :] += bias (float32 sum, rounded once to y's dtype).  Llama has no biases; parts
-// offer them as an option, and this is all that option costs the kernel library.
-template <typename TY, typename TB>
-__global__ void add_bias_kernel(TY* __restrict__ y, const TB* __restrict__ bias, size_t total, int cols, int ldy) {
+// y[m, :] = src[m, :] + bias, the sum in float32 and rounded once to y's dtype (src may be y
+// itself).  A projection with a bias takes its product in float32 and comes here, so that the
+// result is rounded once, as a product that adds the bias to its accumulators would round it
+// (the reference's biased Linear does: yalis/external/model.py:449, torch's addmm).  Llama has no
+// biases; parts offer them as an option, and this is all that option costs the kernel library.
+template <typename TS, typename TY, typename TB>
+__global__ void add_bias_kernel(const TS* __restrict__ src, int lds, TY* __restrict__ y, const TB* __restrict__ bias,
+                                size_t total, int cols, int ldy) {
   for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total;
        i += static_cast<size_t>(gridDim.x) * blockDim.x) {
     const size_t m = i / cols;
     const int n = static_cast<int>(i % cols);
-    TY* p = y + m * ldy + n;
-    *p = from_f32<TY>(to_f32<TY>(*p) + to_f32<TB>(bias[n]));
+    y[m * ldy + n] = from_f32<TY>(to_f32<TS>(src[m * lds + n]) + to_f32<TB>(bias[n]));
   }
 }
 
-extern "C" int yk_add_bias(void* y, int y_dtype, const void* bias, int bias_dtype, int rows, int cols, int ldy,
-                           hipStream_t stream) {
-  YK_REQUIRE(rows >= 0 && cols > 0 && ldy >= cols, "add_bias: bad sizes");
+extern "C" int yk_add_bias(const void* src, int src_dtype, int lds, void* y, int y_dtype, int ldy, const void* bias,
+                           int bias_dtype, int rows, int cols, hipStream_t stream) {
+  YK_REQUIRE(rows >= 0 && cols > 0 && ldy >= cols && lds >= cols, "add_bias: bad sizes");
+  YK_REQUIRE(src != y || (src_dtype == y_dtype && lds == ldy), "add_bias: in place needs one dtype and one stride");
   if (rows == 0) return 0;
   const size_t total = static_cast<size_t>(rows) * cols;
   const int grid = static_cast<int>(std::min<size_t>((total + 255) / 256, 65535));
-#define YK_CASE(YD, TY, BD, TB)                                                              \
-  if (y_dtype == YD && bias_dtype == BD) {                                                  \
-    add_bias_kernel<TY, TB><<<grid, 256, 0, stream>>>(static_cast<TY*>(y), static_cast<const TB*>(bias), total, cols, ldy); \
+#define YK_CASE(SD, TS, YD, TY, BD, TB)                                                      \
+  if (src_dtype == SD && y_dtype == YD && bias_dtype == BD) {                               \
+    add_bias_kernel<TS, TY, TB><<<grid, 256, 0, stream>>>(static_cast<const TS*>(src), lds, static_cast<TY*>(y), \
+                                                          static_cast<const TB*>(bias), total, cols, ldy);       \
     return yk_check_launch("add_bias");                                                     \
   }
-  YK_CASE(YK_F32, float, YK_F32, float)
-  YK_CASE(YK_F32, float, YK_BF16, bf16_t)
-  YK_CASE(YK_BF16, bf16_t, YK_F32, float)
-  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t)
+  YK_CASE(YK_F32, float, YK_F32, float, YK_F32, float)
+  YK_CASE(YK_F32, float, YK_F32, float, YK_BF16, bf16_t)
+  YK_CASE(YK_F32, float, YK_BF16, bf16_t, YK_F32, float)
+  YK_CASE(YK_F32, float, YK_BF16, bf16_t, YK_BF16, bf16_t)
+  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t, YK_F32, float)
+  YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t, YK_BF16, bf16_t)
 #undef YK_CASE
   return yk_fail("add_bias: unsupported dtype combination");
 }

@@ -3,11 +3,13 @@
 // 462-466, 717-722).  What this file adds to a plain library call: the descriptors and the
 // chosen algorithm of every shape are kept, so that a call costs the host a few microseconds
 // (through torch's matrix product it is about 19, four times a layer, which is what bounds a
-// step of a prompt portion at the smaller shapes), and for up to 256 rows of x the algorithm is
-// the fastest of the library's own candidates for that shape, timed once when the shape is first
-// met: there the library's first candidate is often not its best (128 rows at the 8B shapes, us,
-// first / fastest: down-proj 58 / 39, o-proj 20 / 15, qkv 20 / 18), while from 512 rows on the
-// first is as fast as any (and is what torch's product runs: the results are the same bits).
+// step of a prompt portion at the smaller shapes).  By default the algorithm is the library's
+// first candidate, the same in every process, so that a step's bits do not depend on the run.
+// On request (yk_gemm_library_tune) the candidates of a shape of up to 256 rows of x are timed
+// once when the shape is first met and the fastest is kept: there the first is often not the best
+// (128 rows at the 8B shapes, us, first / fastest: down-proj 58 / 39, o-proj 20 / 15, qkv 20 / 18),
+// while from 512 rows on the first is as fast as any (and is what torch's product runs: the results
+// are the same bits); the choice then depends on timing noise and may differ between two runs.
 #include <hipblaslt/hipblaslt.h>
 
 #include <map>
@@ -23,6 +25,7 @@ struct LtPlan {
   hipblasLtMatmulDesc_t desc = nullptr;
   hipblasLtMatrixLayout_t a = nullptr, b = nullptr, c = nullptr;
   hipblasLtMatmulAlgo_t algo;
+  size_t workspace_need = 0;  // scratch the chosen algorithm asks for
   int candidates = 0, chosen = 0;
 };
 
@@ -34,7 +37,7 @@ struct LtDevice {
 
 std::mutex g_lt_mutex;
 std::map<int, LtDevice> g_lt_devices;
-int g_lt_tune = 1;
+int g_lt_tune = 0;
 constexpr int LT_TUNE_MAX_ROWS = 256;
 
 const char* lt_status(hipblasStatus_t s) {
@@ -57,7 +60,7 @@ const char* lt_status(hipblasStatus_t s) {
 
 }  // namespace
 
-// 0: take the library's first candidate for every new shape; 1 (the default): for shapes of up to
+// 0 (the default): take the library's first candidate for every new shape; 1: for shapes of up to
 // 256 rows of x, time its candidates once and keep the fastest.  Shapes already met keep what
 // they have.
 extern "C" int yk_gemm_library_tune(int on) {
@@ -68,7 +71,7 @@ extern "C" int yk_gemm_library_tune(int on) {
 // y [M, N] (bfloat16, or float32 with y_dtype YK_F32) = x [M, K] . w [N, K]^T, bfloat16 operands,
 // float32 accumulation.  `workspace` is the library's scratch (it may be null with 0 bytes).
 // *info, when given, receives candidates * 256 + the index of the one in use.
-// Not for captured graphs: a new shape is timed with events on `stream`.
+// Under a graph capture nothing is timed: a shape first met there gets the first candidate.
 extern "C" int yk_gemm_library(const void* x, const void* w, void* y, int y_dtype, int M, int N, int K, int ldx,
                                int ldw, int ldy, void* workspace, size_t workspace_bytes, int* info,
                                hipStream_t stream) {
@@ -139,9 +142,14 @@ extern "C" int yk_gemm_library(const void* x, const void* w, void* y, int y_dtyp
       (void)hipGetLastError();  // a candidate that failed to launch is simply not chosen
     }
     plan.algo = found[plan.chosen].algo;
+    plan.workspace_need = found[plan.chosen].workspaceSize;
     it = dev.plans.emplace(key, plan).first;
   }
   const LtPlan& plan = it->second;
+  // (the plan was made with the workspace of the call that first met the shape)
+  if (plan.workspace_need > workspace_bytes)
+    return yk_fail("gemm_library: the algorithm kept for this shape needs " + std::to_string(plan.workspace_need) +
+                   " bytes of workspace, this call brings " + std::to_string(workspace_bytes));
   if (info) *info = plan.candidates * 256 + plan.chosen;
   LT_TRY(hipblasLtMatmul(dev.handle, plan.desc, &alpha, w, plan.a, x, plan.b, &beta, y, plan.c, y, plan.c, &plan.algo,
                          workspace, workspace_bytes, stream),

@@ -21,20 +21,15 @@ from .step import ModelRunner
 
 
 class _ShapeOnlyOps:
-    """Stands in for the kernel library where parts are built only to ask them
-    which tensors they need (no kernel is ever called)."""
+    """Stands in for the kernel library where parts are built only to ask them which
+    tensors they need: no kernel is ever called, and whatever a part's constructor asks the
+    library (a tile size, whether a fused path exists, a packed layout's group) is answered
+    with 1, a value that is a valid size and a true flag.  A new part needs no entry here."""
 
-    def check_attention_sizes(self, *a):
-        pass
-
-    def attention_tokens_per_tile(self, *a):
-        return 1
-
-    def attention_long_span_tile(self, *a):
-        return 4
-
-    def attention_long_col_tiles(self, *a):
-        return 1
+    def __getattr__(self, name):
+        if name.startswith("__"):
+            raise AttributeError(name)
+        return lambda *a, **k: 1
 
 
 def spec_from_config(config_dict: dict):
@@ -66,10 +61,13 @@ def build_model(
         raise ValueError(
             f"max_model_len={engine.max_model_len} exceeds the model's max_position_embeddings={spec.max_positions}"
         )
+    if ops is None:
+        ops = default_ops(engine.device)
+        ops.tune_library_products(engine.tune_library_products)
     rt = Runtime(
         device=engine.device,
         engine_dtype=engine.dtype,
-        ops=ops if ops is not None else default_ops(engine.device),
+        ops=ops,
         max_positions=engine.max_model_len,
         page_size=engine.page_size,
     )
@@ -79,7 +77,8 @@ def build_model(
 def load_runner(model_dir: str, engine: EngineConfig, ops=None, progress=None) -> ModelRunner:
     """A runner over the checkpoint in ``model_dir``."""
     model = build_model(read_config_json(model_dir), engine, ops)
-    model.load(open_tensors(model_dir, model.tensor_specs(), model.tensor_uses(), engine.dtype, engine.device, progress))
+    model.load(open_tensors(model_dir, model.tensor_specs(), model.tensor_uses(), engine.dtype, engine.device, progress,
+                            wide_tensors=engine.wide_tensors))
     return ModelRunner(model, engine)
 
 

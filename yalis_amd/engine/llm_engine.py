@@ -342,8 +342,13 @@ class LLMEngine:
         old = runner.config
         pages = None if old.num_pages is None else max(1, old.num_pages * max_batch_size // old.max_num_seqs)
         new_config = dataclasses.replace(old, max_num_seqs=max_batch_size, num_pages=pages)
+        # the old pool is freed before the new one is made: nothing else may hold the old runner
+        # (the last call's scheduler does) or what its captured graphs keep alive
+        runner.drop_graphs()
+        if self.last_scheduler is not None:
+            self.last_scheduler.runner = None
         self.runner = None
-        del runner  # the old pool is freed before the new one is made
+        del runner
         self.runner = ModelRunner(self.model, new_config)
         self.engine_config = new_config
         self.inference_config.max_batch_size = max_batch_size

@@ -15,6 +15,7 @@ import json
 import os
 import sys
 from typing import Dict, Iterable, List, Optional
+from urllib.parse import quote
 
 import torch
 
@@ -30,7 +31,8 @@ class Replayer:
         self.runner = runner
         self.handles: Dict[str, int] = {}
         self._next = 0
-        self.page_log: List[Dict[str, List[int]]] = []  # per step: id -> pages held (group 0)
+        # per step that ran: id -> the pages held after it, one list per cache group
+        self.page_log: List[Dict[str, List[List[int]]]] = []
 
     def run_step(self, step: dict) -> Optional[torch.Tensor]:
         """Runs one step; returns float32 logits [wanted, vocab] or None when
@@ -61,10 +63,9 @@ class Replayer:
         logits = None
         if entries:
             logits = self.runner.step(entries)
-            if self.runner.pages.groups:
-                self.page_log.append(
-                    {rid: self.runner.pages.block_table(h, 0).tolist() for rid, h in self.handles.items()}
-                )
+            self.page_log.append(
+                {rid: [t.tolist() for t in self.runner.pages.block_tables(h)] for rid, h in self.handles.items()}
+            )
         for rid in step.get("end", []):
             rid = str(rid)
             if rid not in self.handles:
@@ -75,22 +76,60 @@ class Replayer:
         return logits
 
 
+def _file_name(request_id: str) -> str:
+    """A request id as a file name (ids are arbitrary strings)."""
+    return quote(request_id, safe="") or "_"
+
+
 def replay_stream(runner: ModelRunner, lines: Iterable[str], out_dir: str, out=sys.stdout) -> None:
-    """Read steps (one JSON object a line), write ``out_dir/<step>.f32`` for steps
-    in which something is wanted, print ``done <step>`` after each."""
+    """Read steps (one JSON object a line); for steps in which something is wanted write
+    ``out_dir/<step>.f32`` (float32 [wanted, vocab], little-endian, in the order of the entries
+    and of ``want``); print ``done <step>`` after each.
+
+    Beside that, for whoever compares runs request by request: ``out_dir/requests/<id>.f32``
+    gathers every wanted row of one request in the order they were computed (its absolute
+    positions are in the log), and ``out_dir/pages.jsonl`` has one line a step:
+    ``{"step": k, "positions": {id: [absolute positions of its wanted rows]}, "pages": {id:
+    [[page ids of cache group 0], [group 1], ...]}}``, the pages every live request held
+    after the step (-1: a logical page a window has given back)."""
     os.makedirs(out_dir, exist_ok=True)
+    req_dir = os.path.join(out_dir, "requests")
+    os.makedirs(req_dir, exist_ok=True)
     rp = Replayer(runner)
-    for line in lines:
-        line = line.strip()
-        if not line:
-            continue
-        step = json.loads(line)
-        logits = rp.run_step(step)
-        if logits is not None:
-            arr = logits.detach().to(torch.float32).cpu().numpy().astype("<f4", copy=False)
-            tmp = os.path.join(out_dir, f".{step['step']}.f32.tmp")
-            arr.tofile(tmp)
-            os.replace(tmp, os.path.join(out_dir, f"{step['step']}.f32"))
-        elif torch.cuda.is_available():
-            torch.cuda.synchronize()
-        print(f"done {step['step']}", file=out, flush=True)
+    cached: Dict[str, int] = {}
+    started = set()
+    with open(os.path.join(out_dir, "pages.jsonl"), "w", encoding="utf-8") as page_log:
+        for line in lines:
+            line = line.strip()
+            if not line:
+                continue
+            step = json.loads(line)
+            ran = len(rp.page_log)
+            logits = rp.run_step(step)
+            positions: Dict[str, List[int]] = {}
+            for e in step.get("entries", []):
+                rid = str(e["id"])
+                base = cached.get(rid, 0)
+                positions[rid] = [base + int(w) for w in e.get("want", [])]
+                cached[rid] = base + len(e["tokens"])
+            if logits is not None:
+                arr = logits.detach().to(torch.float32).cpu().numpy().astype("<f4", copy=False)
+                tmp = os.path.join(out_dir, f".{step['step']}.f32.tmp")
+                arr.tofile(tmp)
+                os.replace(tmp, os.path.join(out_dir, f"{step['step']}.f32"))
+                row = 0
+                for rid, pos in positions.items():
+                    if pos:
+                        with open(os.path.join(req_dir, _file_name(rid) + ".f32"), "ab" if rid in started else "wb") as f:
+                            arr[row : row + len(pos)].tofile(f)
+                        started.add(rid)
+                        row += len(pos)
+            elif torch.cuda.is_available():
+                torch.cuda.synchronize()
+            held = rp.page_log[-1] if len(rp.page_log) > ran else {}
+            page_log.write(json.dumps({"step": step["step"], "positions": positions, "pages": held}) + "\n")
+            page_log.flush()
+            for rid in step.get("end", []):
+                cached.pop(str(rid), None)
+                started.discard(str(rid))
+            print(f"done {step['step']}", file=out, flush=True)

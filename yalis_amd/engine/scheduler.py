@@ -106,18 +106,33 @@ class Scheduler:
         room = self.cfg.max_model_len - len(prompt)
         if params.max_tokens > room:
             params = SamplingParams(**{**params.__dict__, "max_tokens": room})
-        pool_tokens = min(
-            (g.num_pages * self.runner.page_size for g in self.runner.group_shapes), default=1 << 60
-        )
         # the last sampled token is never written to the cache
-        if len(prompt) + params.max_tokens - 1 > pool_tokens:
-            raise ValueError(
-                f"request needs {len(prompt) + params.max_tokens - 1} cached tokens, the whole pool holds {pool_tokens}"
-            )
+        total = len(prompt) + params.max_tokens - 1
+        for g, shape in enumerate(self.runner.group_shapes):
+            need = self.pages_a_request_needs(total, shape.window)
+            if need > shape.num_pages:
+                kept = "all of them" if shape.window is None else f"a window of {shape.window}"
+                raise ValueError(
+                    f"request needs {total} cached tokens ({need} pages of cache group {g}, which keeps {kept}), "
+                    f"the group's whole pool holds {shape.num_pages} pages of {self.runner.page_size} tokens"
+                )
         req = Request(self._next_rid, prompt, params)
         self._next_rid += 1
         self.waiting.append(req)
         return req
+
+    def pages_a_request_needs(self, total_tokens: int, window: Optional[int]) -> int:
+        """The most pages of one cache group a request of ``total_tokens`` cached tokens ever
+        holds at once.  A group that keeps everything: all its pages.  A windowed group: while a
+        step adds n tokens behind c cached ones, positions c - window + 1 .. c + n - 1 are
+        held, window + n - 1 tokens that touch one page more than they fill; n is at most the
+        step's token budget."""
+        page = self.runner.page_size
+        full = -(-total_tokens // page)
+        if window is None:
+            return full
+        n = min(self.cfg.max_num_batched_tokens, total_tokens)
+        return min(full, -(-(int(window) + n - 1) // page) + 1)
 
     def has_work(self) -> bool:
         return bool(self.waiting or self.running)

@@ -11,6 +11,7 @@ the head runs on the wanted rows only.
 """
 from __future__ import annotations
 
+from collections import OrderedDict
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -36,12 +37,15 @@ class Site:
             return None, None
         return self._memory.kv(self.group, self.info.index_in_group)
 
-    def state(self) -> Optional[torch.Tensor]:
-        """Per-request state of this entry: [num_slots, ...]; rows are chosen by
-        ``StepContext.arrays['state_slots']``."""
-        if self.info.state_index is None:
+    def state(self, which: int = 0) -> Optional[torch.Tensor]:
+        """Per-request state of this entry, the ``which``-th of the mixer's needs:
+        [num_slots, ...]; rows are chosen by ``StepContext.arrays['state_slots']``."""
+        if not self.info.state_indices:
             return None
-        return self._memory.states[self.info.state_index]
+        return self._memory.states[self.info.state_indices[which]]
+
+    def states(self) -> Tuple[torch.Tensor, ...]:
+        return tuple(self._memory.states[i] for i in self.info.state_indices)
 
 
 class StepContext:
@@ -106,12 +110,13 @@ class _DecodeGraph:
     """One captured decode step: the graph, the integer buffer its kernels read, the
     logits it writes, and what must stay alive while it may be replayed."""
 
-    def __init__(self, graph, ints, layout, logits, keep):
+    def __init__(self, graph, ints, layout, logits, keep, nbytes=0):
         self.graph = graph
         self.ints = ints
         self.layout = layout
         self.logits = logits
         self.keep = keep
+        self.nbytes = nbytes  # device memory the graph holds (its pool, logits, integer buffer)
 
 
 # Decode steps of up to this many requests are captured as graphs (larger batches run
@@ -147,7 +152,11 @@ class ModelRunner:
         self.use_graphs = (
             torch.device(config.device).type == "cuda" and config.decode_graphs and model.graph_capturable
         )
-        self._graphs: Dict[Tuple, _DecodeGraph] = {}
+        # captured graphs, least recently replayed first; together they hold at most
+        # ``config.graph_memory_bytes`` of device memory (beyond it the oldest are dropped and
+        # captured again when their shape of step returns)
+        self._graphs: "OrderedDict[Tuple, _DecodeGraph]" = OrderedDict()
+        self.graphs_dropped = 0
         self._table_widths = [-(-config.max_model_len // self.page_size) for _ in self.group_shapes]
         self.graph_replays = 0
 
@@ -244,6 +253,24 @@ class ModelRunner:
             self.pages.advance(e.request, self.cached[e.request])
         return logits
 
+    def graph_bytes(self) -> int:
+        return sum(g.nbytes for g in self._graphs.values())
+
+    def _drop_graphs_beyond(self, limit: int, keep=None) -> None:
+        """Drop the least recently replayed graphs until what is left holds at most ``limit``
+        bytes (the one named ``keep`` always stays)."""
+        while len(self._graphs) > 1 and self.graph_bytes() > limit:
+            oldest = next(k for k in self._graphs if k != keep)
+            torch.cuda.synchronize()  # nothing of it may still be running when its memory goes back
+            del self._graphs[oldest]
+            self.graphs_dropped += 1
+
+    def drop_graphs(self) -> None:
+        """Forget every captured graph (they are captured again when needed)."""
+        if self._graphs:
+            torch.cuda.synchronize()
+        self._graphs.clear()
+
     @staticmethod
     def _views(dev: torch.Tensor, layout) -> Dict[str, torch.Tensor]:
         return {
@@ -286,17 +313,21 @@ class ModelRunner:
             self._feed_tokens(ints, layout, len(spans), token_source, token_index is not None)
             ctx = StepContext(hb, self._views(ints, layout), self.sites, self.rt)
             ops = self.rt.ops
-            # every weight matrix a part holds, as (rows, columns): the products of the step
-            products = sorted({tuple(t.shape) for p in self.model.all_parts() for t in vars(p).values()
-                               if isinstance(t, torch.Tensor) and t.dim() == 2})
+            # the products of the step, as the parts declare them: (rows, columns) of each weight
+            products = sorted({tuple(int(v) for v in nk) for p in self.model.all_parts() for nk in p.products()})
             ops.reserve_workspaces(hb.n_seqs, products)
             torch.cuda.synchronize()
+            reserved = torch.cuda.memory_reserved(self.config.device)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 logits = self.model.forward(ctx)
-            entry = _DecodeGraph(graph, ints, layout, logits, ops.workspaces())
+            held = max(torch.cuda.memory_reserved(self.config.device) - reserved, 0)
+            held = max(held, logits.numel() * logits.element_size()) + ints.numel() * 4
+            entry = _DecodeGraph(graph, ints, layout, logits, ops.workspaces(), held)
             self._graphs[key] = entry
+            self._drop_graphs_beyond(self.config.graph_memory_bytes, keep=key)
         else:
+            self._graphs.move_to_end(key)
             if layout != entry.layout:
                 raise RuntimeError("a decode step's integer arrays changed shape under a captured graph")
             self._uploader.upload(buf, into=entry.ints)

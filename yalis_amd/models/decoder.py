@@ -37,7 +37,11 @@ class SiteInfo:
     group: Optional[int]  # cache group read by this entry (None: the mixer caches nothing)
     index_in_group: Optional[int]  # which of the group's caches
     owns_cache: bool  # False: reads another entry's cache and writes none
-    state_index: Optional[int]  # which per-request state tensor (None: no state)
+    state_indices: Tuple[int, ...]  # which per-request state tensors, in the order of the mixer's needs
+
+    @property
+    def state_index(self) -> Optional[int]:
+        return self.state_indices[0] if self.state_indices else None
 
 
 class DecoderModel:
@@ -111,10 +115,12 @@ class DecoderModel:
             elif e.cache_from is not None:
                 raise ValueError(f"run_order[{i}] names cache_from but its mixer keeps no cache")
             sneed = None if mixer is None else mixer.state_need()
-            sidx = None
-            if sneed is not None:
-                sidx = len(states)
-                states.append(sneed)
+            if sneed is None:
+                sneed = ()
+            elif isinstance(sneed, StateNeed):
+                sneed = (sneed,)
+            sidx = tuple(range(len(states), len(states) + len(sneed)))
+            states.extend(sneed)
             sites.append(SiteInfo(i, e.layer, group, index, owns, sidx))
         cache_groups = [CacheGroup(n, tuple(m)) for n, m in groups]
         return cache_groups, states, sites

@@ -28,6 +28,11 @@ class KernelError(RuntimeError):
     pass
 
 
+class StaleWorkspace(KernelError):
+    """A result that lives in the library's workspace was consumed after the workspace had
+    been handed to a later launch."""
+
+
 def _code(dtype: torch.dtype) -> int:
     if dtype == torch.float32:
         return _F32
@@ -53,7 +58,7 @@ _SIGNATURES = {
          _c_int, _c_int, _c_int, _vp, _vp, _vp, _c_int, _vp],
         _c_int,
     ),
-    "yk_add_bias": ([_vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _vp], _c_int),
+    "yk_add_bias": ([_vp, _c_int, _c_int, _vp, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_gated_act": ([_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_gemm_fma": (
         [_vp, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
@@ -110,7 +115,7 @@ _LATER_SIGNATURES = {
         "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
     },
 }
-_ABI = 13
+_ABI = 14
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
 # above it the vendor library does.
@@ -133,10 +138,13 @@ class SplitSum:
     of its own.  ``out_dtype`` is the dtype the product was asked for: the consumers round
     the sum to it, so that a value does not depend on whether its product came reduced or
     as slices.  It lives in the library's workspace: consume it before the next product
-    is launched."""
+    is launched.  One that the library made carries the workspace's generation number, and
+    the library refuses (``StaleWorkspace``) to consume it once a later product has taken
+    the workspace."""
 
-    def __init__(self, tensor: torch.Tensor, out_dtype: torch.dtype = torch.float32):
+    def __init__(self, tensor: torch.Tensor, out_dtype: torch.dtype = torch.float32, owner=None, generation: int = 0):
         self.tensor = tensor
+        self.owner, self.generation = owner, generation
         self.shape = tuple(tensor.shape[1:])
         self.n_splits = tensor.shape[0]
         self.out_dtype = out_dtype
@@ -147,8 +155,16 @@ class SplitSum:
     def round_sum(self) -> int:
         return int(self.out_dtype == torch.bfloat16)
 
+    def check_live(self) -> None:
+        if self.owner is not None and self.generation != self.owner._gemm_gen:
+            raise StaleWorkspace(
+                "a product's unreduced slices (SplitSum) were consumed after a later product had been launched: the "
+                "library's workspace holds that product's slices now.  Consume a linear(..., partial_ok=True) result "
+                "(norm, rotary + append, gated activation, .reduce()) before the next linear, or ask without partial_ok")
+
     def reduce(self) -> torch.Tensor:
         """The product itself, float32 (for code that does not add the slices itself)."""
+        self.check_live()
         return self.tensor.sum(0).to(self.out_dtype).float()
 
     def float(self) -> torch.Tensor:
@@ -179,17 +195,26 @@ class SplitAttention:
     it stands for a bfloat16 tensor [tokens, heads * head_dim].  ``HipOps.linear`` merges the
     splits while it stages them as its input where its kernel can (up to 16 tokens), which
     saves the merging kernel; ``merge()`` gives the tensor itself.  It lives in the library's
-    workspace: consume it before the next attention is launched."""
+    workspace: consume it before the next attention (or anything else that takes that
+    workspace: choosing tokens) is launched; the library refuses a stale one."""
 
     def __init__(self, ops, workspace, tiles, token_cols, n_tokens, n_heads, n_kv, head_dim, n_splits):
         self.ops, self.workspace, self.tiles, self.token_cols = ops, workspace, tiles, token_cols
+        self.generation = ops._ws_gen
         self.n_heads, self.n_kv, self.head_dim, self.n_splits = n_heads, n_kv, head_dim, n_splits
         self.shape = (n_tokens, n_heads * head_dim)
         self.dtype = torch.bfloat16
         self.device = workspace.device
 
+    def check_live(self) -> None:
+        if self.generation != self.ops._ws_gen:
+            raise StaleWorkspace(
+                "an attention's unmerged splits (SplitAttention) were consumed after a later launch had taken the "
+                "library's workspace; hand them to linear() or merge() before the next attention")
+
     def merge(self) -> torch.Tensor:
         ops = self.ops
+        self.check_live()
         out = torch.empty(self.shape, dtype=self.dtype, device=self.device)
         ops._check(
             ops.lib.yk_attn_combine(
@@ -224,6 +249,10 @@ class HipOps:
         self._workspace: Optional[torch.Tensor] = None  # attention splits, argmax parts
         self._library_workspace: Optional[torch.Tensor] = None  # the vendor library's scratch
         self._gemm_workspace: Optional[torch.Tensor] = None  # K slices of products
+        # how often each workspace has been handed out: what lives in one (SplitSum,
+        # SplitAttention) remembers the number and is refused once it has moved on
+        self._ws_gen = 0
+        self._gemm_gen = 0
         # page ids a workgroup of the long-span attention keeps in LDS (more: looked up in the
         # block table one by one); tests lower it to walk that path with short tables
         self.long_span_pages_in_lds = 2048
@@ -269,10 +298,12 @@ class HipOps:
     def _ws(self, floats: int) -> torch.Tensor:
         """Float32 scratch that grows and is reused (stream order keeps uses apart)."""
         self._workspace = self._grown(self._workspace, floats)
+        self._ws_gen += 1
         return self._workspace
 
     def _gemm_ws(self, floats: int) -> torch.Tensor:
         self._gemm_workspace = self._grown(self._gemm_workspace, floats)
+        self._gemm_gen += 1
         return self._gemm_workspace
 
     def reserve_workspaces(self, rows: int, products=()) -> None:
@@ -295,8 +326,9 @@ class HipOps:
         self._answers = {k: v for k, v in self._answers.items() if k[0] not in ("yk_gemm_skinny_splits", "yk_gemm_skinny_from_attention_ok")}
 
     def tune_library_products(self, on: bool = True) -> None:
-        """Whether new shapes of up to 256 rows get the fastest of the vendor library's candidates
-        (timed when first met; the default) or its first one (the same choice in every process)."""
+        """Whether new shapes of up to 256 rows get the vendor library's first candidate (the
+        default: the same choice, and the same bits, in every process) or the fastest of its
+        candidates, timed when the shape is first met (the choice then depends on the run)."""
         self._check(self.lib.yk_gemm_library_tune(int(bool(on))))
 
     def workspaces(self):
@@ -378,6 +410,7 @@ class HipOps:
         if isinstance(x, SplitAttention):
             x = src = x.merge()
         if isinstance(x, SplitSum):
+            x.check_live()
             n_splits, round_sum, src = x.n_splits, x.round_sum, x.tensor
         else:
             self._rows(x, "norm input")
@@ -413,6 +446,7 @@ class HipOps:
                 raise KernelError("the embedding table must be contiguous and the token ids int32")
             table_rows = delta.shape[0]
         elif isinstance(delta, SplitSum):
+            delta.check_live()
             n_splits, round_sum, delta = delta.n_splits, delta.round_sum, delta.tensor
             if tuple(delta.shape[1:]) != tuple(residual.shape):
                 raise KernelError(f"delta {tuple(delta.shape[1:])} does not match the residual {tuple(residual.shape)}")
@@ -440,12 +474,16 @@ class HipOps:
         """x [M, K] . w [N, K]^T (+ bias [N]) -> [M, N].  With ``partial_ok`` (and no bias) the
         result may come as a ``SplitSum`` for a consumer that adds the slices itself."""
         if bias is not None:
-            y = self.linear(x, w, out_dtype, partial_ok=False)
-            if bias.numel() != y.shape[1] or not bias.is_contiguous():
-                raise KernelError(f"linear: bias has {bias.numel()} elements, the product {y.shape[1]} columns")
+            # the product in float32, the bias added there, one rounding (as a product that adds
+            # the bias to its accumulators rounds: the reference's biased Linear)
+            acc = self.linear(x, w, torch.float32, partial_ok=False)
+            if bias.numel() != acc.shape[1] or not bias.is_contiguous():
+                raise KernelError(f"linear: bias has {bias.numel()} elements, the product {acc.shape[1]} columns")
+            y = acc if out_dtype == torch.float32 else torch.empty(acc.shape, dtype=out_dtype, device=acc.device)
             if y.shape[0]:
-                self._check(self.lib.yk_add_bias(y.data_ptr(), _code(y.dtype), bias.data_ptr(), _code(bias.dtype),
-                                                 y.shape[0], y.shape[1], y.stride(0), self._stream()))
+                self._check(self.lib.yk_add_bias(acc.data_ptr(), _code(acc.dtype), acc.stride(0), y.data_ptr(), _code(y.dtype),
+                                                 y.stride(0), bias.data_ptr(), _code(bias.dtype), y.shape[0], y.shape[1],
+                                                 self._stream()))
             return y
         if isinstance(x, SplitAttention):
             y = self._linear_from_attention(x, w, out_dtype, partial_ok)
@@ -487,6 +525,7 @@ class HipOps:
     def _linear_from_attention(self, x: "SplitAttention", w: torch.Tensor, out_dtype, partial_ok: bool):
         """The few-row product fed by attention's unmerged splits, or None where it does not
         apply (the caller then merges them first)."""
+        x.check_live()
         m, k = x.shape
         n = w.shape[0]
         if (w.dim() != 2 or w.dtype != torch.bfloat16 or w.shape[1] != k or w.stride(1) != 1 or w.stride(0) % 8
@@ -504,7 +543,7 @@ class HipOps:
         if rc < 0:
             raise KernelError(self.lib.yk_last_error().decode())
         if keep:
-            return SplitSum(ws[: rc * m * n].view(rc, m, n), out_dtype)  # rc: the slices the launch wrote
+            return SplitSum(ws[: rc * m * n].view(rc, m, n), out_dtype, self, self._gemm_gen)  # rc: the slices the launch wrote
         return y
 
     LIBRARY_WORKSPACE_BYTES = 64 << 20
@@ -512,8 +551,8 @@ class HipOps:
     def gemm_library(self, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
         """x [M, K] . w [N, K]^T in the vendor library: bfloat16 operands with 16-byte aligned rows,
         float32 accumulation, the result bfloat16 or float32.  Every shape's algorithm is chosen
-        when the shape is first met (for up to 256 rows the fastest of the library's own
-        candidates, timed then; else its first) and kept."""
+        when the shape is first met (the library's first candidate, or with
+        ``tune_library_products`` the fastest for up to 256 rows) and kept."""
         m, k = x.shape
         n = w.shape[0]
         if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[1] != k or x.stride(1) != 1 or w.stride(1) != 1:
@@ -595,7 +634,7 @@ class HipOps:
         if rc < 0:
             raise KernelError(self.lib.yk_last_error().decode())
         if keep:
-            return SplitSum(ws[: rc * m * n].view(rc, m, n), out_dtype)  # rc: the slices the launch wrote
+            return SplitSum(ws[: rc * m * n].view(rc, m, n), out_dtype, self, self._gemm_gen)  # rc: the slices the launch wrote
         return y
 
     # ------------------------------------------------- rotary + append to the cache
@@ -607,6 +646,7 @@ class HipOps:
         n_splits, round_sum = 1, 0
         src = qkv
         if isinstance(qkv, SplitSum):
+            qkv.check_live()
             n_splits, round_sum, src = qkv.n_splits, qkv.round_sum, qkv.tensor
             n, cols = qkv.shape
             act = k_cache.dtype if n_kv else torch.bfloat16
@@ -667,6 +707,15 @@ class HipOps:
         a split."""
         slots = 768 if col_tiles == 1 else 512
         return max(1, min(slots // max(1, workgroups), key_blocks // 8, 16))
+
+    @staticmethod
+    def rope_in_launch(rotation, append: bool) -> "RopeInLaunch":
+        """What ``attention(rope=)`` takes, from a position encoding's ``Rotation`` (None: no
+        rotation, the launch only appends) and whether the projection's rows hold keys and
+        values to append."""
+        if rotation is None:
+            return RopeInLaunch(None, None, 0, False, append)
+        return RopeInLaunch(rotation.cos, rotation.sin, rotation.rotary_dim, rotation.interleaved, append)
 
     def attention_can_rotate(self, act_dtype: torch.dtype, head_dim: int) -> bool:
         """Whether ``attention`` takes ``rope=`` for such a mixer: the matrix-core kernel for
@@ -759,6 +808,7 @@ class HipOps:
                         ctx, group, tiles, plan, token_cols, rope: "RopeInLaunch"):
         n_splits_src, round_sum, src = 1, 0, qkv
         if isinstance(qkv, SplitSum):
+            qkv.check_live()
             n_splits_src, round_sum, src = qkv.n_splits, qkv.round_sum, qkv.tensor
             n, cols = qkv.shape
             src_stride = cols
@@ -810,6 +860,7 @@ class HipOps:
         n_splits, round_sum = 1, 0
         src = gu
         if isinstance(gu, SplitSum):
+            gu.check_live()
             n_splits, round_sum, src = gu.n_splits, gu.round_sum, gu.tensor
             rows, cols = gu.shape
             out_dtype = out_dtype or torch.bfloat16

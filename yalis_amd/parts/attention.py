@@ -70,14 +70,7 @@ class Attention(Mixer):
         can = getattr(rt.ops, "attention_can_rotate", None)
         self.rotates_in_launch = bool(can is not None and can(rt.act_dtype, self.head_dim))
         if self.rotates_in_launch:
-            from ..ops.hip import RopeInLaunch
-
-            p = self.rotation
-            self.rope_in_launch = {
-                append: RopeInLaunch(None if p is None else p.cos, None if p is None else p.sin,
-                                     0 if p is None else p.rotary_dim, False if p is None else p.interleaved, append)
-                for append in (False, True)
-            }
+            self.rope_in_launch = {append: rt.ops.rope_in_launch(self.rotation, append) for append in (False, True)}
         self.b_qkv = self.b_q = self.b_o = None
 
     # ---- what it needs
@@ -119,6 +112,10 @@ class Attention(Mixer):
 
     def kv_need(self) -> KVNeed:
         return KVNeed(self.n_kv, self.head_dim, self.window)
+
+    def products(self):
+        hd, kd = self.n_heads * self.head_dim, self.n_kv * self.head_dim
+        return ((hd + 2 * kd if self.projects_kv else hd, self.hidden), (self.hidden, hd))
 
     def long_col_tiles(self, hb) -> int:
         """Column tiles per wave for this step's long spans (1 or 2), from what the host

@@ -11,7 +11,7 @@ Adding a part means: subclass the interface, decorate it with the matching
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Callable, Dict, Mapping, Optional, Tuple
+from typing import Any, Callable, Dict, Mapping, Optional, Tuple, Union
 
 import torch
 
@@ -97,6 +97,14 @@ class Part:
         step's single upload and arrive as ``StepContext.arrays[name]``."""
         return {}
 
+    def products(self) -> Tuple[Tuple[int, int], ...]:
+        """The (rows, columns) of every weight matrix this part hands to ``ops.linear`` or
+        ``ops.gate_up_act``.  A product of few rows may be computed in slices of K that live
+        in the kernel library's scratch; the library sizes that scratch from this list before
+        a step is captured as a graph (a buffer cannot grow during a capture).  A part that
+        leaves a product out gets an error at the capture, never a wrong result."""
+        return ()
+
 
 class Mixer(Part):
     """Mixes information across the tokens of a request (attention here)."""
@@ -104,7 +112,10 @@ class Mixer(Part):
     def kv_need(self) -> Optional[KVNeed]:
         return None
 
-    def state_need(self) -> Optional[StateNeed]:
+    def state_need(self) -> Union[None, StateNeed, Tuple[StateNeed, ...]]:
+        """Per-request state of fixed size: nothing, one ``StateNeed``, or several (of
+        different shapes and dtypes: a short window of inputs beside a running sum, say).
+        ``site.state(i)`` gives the i-th during a step."""
         return None
 
     def forward(self, h: torch.Tensor, ctx: Any, site: Any) -> torch.Tensor:

@@ -73,5 +73,8 @@ class LMHead(Part):
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.weight = tensors[self.tied_to if self.tied_to is not None else self.name]
 
+    def products(self):
+        return ((self.vocab, self.hidden),)
+
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         return self.rt.ops.linear(h, self.weight, torch.float32)

@@ -67,6 +67,9 @@ class GatedMLP(FeedForward):
             return
         self.w_gate_up, self.gate_up_group = self.rt.ops.pack_gate_up(tensors[self.names["gate"]], tensors[self.names["up"]])
 
+    def products(self):
+        return ((2 * self.inter, self.hidden), (self.hidden, self.inter))
+
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
         ops = self.rt.ops
         if self.bias:

@@ -6,14 +6,18 @@ lists every missing tensor, every unexpected tensor and every wrong shape (the
 reference gets the same from ``load_state_dict(strict=True)``,
 yalis/model_loading.py:201-249).
 
-Precision rule: a floating tensor stored in 16 bits is kept in bfloat16, a tensor
-stored in 32 bits stays in 32 bits (such tensors are stored wide because they need
-it), integer tables become int32.  In the 32-bit mode of the engine every floating
-tensor is widened to float32 (exact).  A checkpoint stored in float16 is refused by the
-bfloat16 engine: rounding it to bfloat16 would silently drop three bits of every weight (the
-reference runs such checkpoints in float16, a precision this engine does not have); the
-float32 engine takes it.  Matrices stored in 32 bits stay so in the bfloat16 engine, which
-then runs their products on the float32 kernels: that is said once, loudly, when it happens.
+Precision rule: a floating tensor stored in 16 bits is kept in bfloat16, integer tables
+become int32, and in the 32-bit mode of the engine every floating tensor is widened to float32
+(exact).  A tensor stored in 32 bits inside a 16-bit checkpoint stays in 32 bits in the bfloat16
+engine (such tensors are stored wide because they need it).  A checkpoint stored WHOLLY in 32
+bits is a 32-bit copy of the model, not a statement about single tensors: the bfloat16 engine
+narrows it to bfloat16, as the reference casts every tensor to its parameter's dtype
+(yalis/model_loading.py:172-173).  ``wide_tensors`` overrides the rule: "keep" leaves every
+32-bit tensor wide (a float32 matrix in the bfloat16 engine then runs on the float32 kernels,
+which is said once, loudly), "cast" narrows all of them.  A checkpoint stored in float16 is
+refused by the bfloat16 engine: rounding it to bfloat16 would silently drop three bits of every
+weight (the reference runs such checkpoints in float16, a precision this engine does not
+have); the float32 engine takes it.
 """
 from __future__ import annotations
 
@@ -70,14 +74,26 @@ _INT_TAGS = {"I64", "I32", "I16", "I8", "U8"}
 IGNORED_SUFFIXES = ("rotary_emb.inv_freq",)
 
 
-def target_dtype(storage_tag: str, kind: str, engine_dtype: str) -> torch.dtype:
+def target_dtype(storage_tag: str, kind: str, engine_dtype: str, keep_wide: bool = True) -> torch.dtype:
+    """``keep_wide``: whether a tensor stored in 32 bits stays so in the bfloat16 engine."""
     if kind == "int":
         return torch.int32
     if engine_dtype == "float32":
         return torch.float32
-    if storage_tag in ("F32", "F64"):
+    if storage_tag in ("F32", "F64") and keep_wide:
         return torch.float32
     return torch.bfloat16
+
+
+def keeps_wide(entries: Dict[str, TensorEntry], wanted: Dict[str, "TensorSpec"], wide_tensors: str) -> bool:
+    """The precision rule's decision for a checkpoint: True when tensors stored in 32 bits
+    stay in 32 bits in the bfloat16 engine."""
+    if wide_tensors not in ("auto", "keep", "cast"):
+        raise ValueError(f"wide_tensors must be 'auto', 'keep' or 'cast', got {wide_tensors!r}")
+    if wide_tensors != "auto":
+        return wide_tensors == "keep"
+    tags = {entries[n].dtype for n, sp in wanted.items() if sp.kind == "float" and n in entries}
+    return not tags <= {"F32", "F64"}  # a checkpoint wholly in 32 bits is narrowed
 
 
 def check_against(entries: Dict[str, TensorEntry], wanted: Dict[str, TensorSpec], where: str, engine_dtype: Optional[str] = None) -> None:
@@ -139,22 +155,28 @@ def open_tensors(
     engine_dtype: str,
     device: str,
     progress: Optional[Callable[[str], None]] = None,
+    wide_tensors: str = "auto",
 ) -> TensorSource:
     """Check the folder against ``wanted`` (the one error lists everything that is wrong)
     and return a source that reads each tensor onto ``device`` when it is asked for."""
     entries = index_folder(model_dir)
     check_against(entries, wanted, model_dir, engine_dtype)
+    keep_wide = keeps_wide(entries, wanted, wide_tensors)
     if engine_dtype == "bfloat16":
-        wide = [n for n, sp in wanted.items() if sp.kind == "float" and len(sp.shape) >= 2 and entries[n].dtype in ("F32", "F64")]
-        if wide:
+        wide = [n for n, sp in wanted.items() if sp.kind == "float" and entries[n].dtype in ("F32", "F64")]
+        matrices = [n for n in wide if len(wanted[n].shape) >= 2]
+        if wide and not keep_wide:
+            logger.info("%s: %d tensors stored in 32 bits are narrowed to bfloat16 for the bfloat16 engine "
+                        "(wide_tensors='keep' leaves them wide)", model_dir, len(wide))
+        elif matrices:
             logger.warning(
                 "%d matrices of %s are stored in 32 bits and stay so: the bfloat16 engine runs their products on its "
-                "float32 kernels (twice the memory, far slower than the matrix cores); first: %s", len(wide), model_dir, wide[0])
+                "float32 kernels (twice the memory, far slower than the matrix cores); first: %s", len(matrices), model_dir, matrices[0])
     done = [0]
 
     def make(name: str) -> torch.Tensor:
         e = entries[name]
-        dt = target_dtype(e.dtype, wanted[name].kind, engine_dtype)
+        dt = target_dtype(e.dtype, wanted[name].kind, engine_dtype, keep_wide)
         t = read_tensor(e).to(device=device, dtype=dt).contiguous()
         done[0] += 1
         if progress is not None and done[0] % 32 == 1:
