@@ -256,6 +256,9 @@ def test_split_sums_feed_their_consumers(ops):
     part = ops.linear(x, w, torch.bfloat16, partial_ok=True)
     assert isinstance(part, SplitSum) and part.n_splits > 1, "this shape was meant to split K"
     assert part.out_dtype == torch.bfloat16
+    # (the slices live in the library's workspace until the next product; a copy of this test's
+    # own can be fed to every consumer below)
+    part = SplitSum(part.tensor.clone(), part.out_dtype)
     full = part.tensor.sum(0)
     assert (full.cpu() - (x.double().cpu() @ w.double().cpu().T).float()).abs().max() < 1e-3
     reduced = ops.linear(x, w, torch.bfloat16)  # the same slices, summed and rounded by the product
@@ -555,11 +558,12 @@ def test_attention_splits_merged_by_the_product(ops, plan, h, g, d, page, monkey
 
     monkeypatch.setattr(hip_ops, "MERGE_IN_PRODUCT_MAX_TOKENS", 16)  # as far as the kernel goes, not as far as it pays
     spans = [(700, 1), (64, 2), (300, 1), (0, 3), (1500, 1), (63, 2)]
+    plain, _ = _attention_case(ops, torch.bfloat16, h, g, d, page, spans, 0, seed=21, n_pages=2700 // page + 8, plan=plan)
+    # (the unmerged splits live in the library's workspace until the next attention: made last)
     got, want = _attention_case(ops, torch.bfloat16, h, g, d, page, spans, 0, seed=21, n_pages=2700 // page + 8, plan=plan, with_cols=True)
     assert isinstance(got, SplitAttention) and got.n_splits == plan[1] and got.shape == (10, h * d)
     merged = got.merge()
     close(merged, want, 2e-2, 2**-6)
-    plain, _ = _attention_case(ops, torch.bfloat16, h, g, d, page, spans, 0, seed=21, n_pages=2700 // page + 8, plan=plan)
     assert torch.equal(plain, merged)
     fed = 0
     for n_out, out_dtype, partial_ok in ((h * d, torch.bfloat16, True), (515, torch.float32, False), (48, torch.bfloat16, True)):

@@ -46,7 +46,7 @@ def test_trace_run_cli(tmp_path, stored, dtype):
     for s in steps[::4]:  # some steps want nothing: no file then
         for e in s["entries"]:
             e["want"] = []
-    max_tokens = sum(-(-len(t) // 64) * 64 for t in list(reqs.values())[:4]) + 64
+    max_tokens = 64 * C.pages_needed(steps, reqs, 64)  # the most live requests ever hold: pages are used again
     out = str(tmp_path / "out")
     run_cli(folder, dtype, out, steps, max_tokens)
     bf16 = dtype == "bfloat16"

@@ -10,7 +10,7 @@
 // Page layout: keys [page][kv_head][page_size][head_dim], values transposed
 // [page][kv_head][head_dim][page_size].  Pages are never cleared, so nothing beyond a
 // request's token count is ever read as a number: invisible scores are replaced, and
-// values of tokens that do not exist yet are zeroed before they meet a probability.
+// values of tokens that do not exist yet, or that lie below a window, are zeroed before they meet a probability.
 //
 // Two kernels:
 //  * attn_generic: one wave per (token, head), float32 arithmetic throughout, any
@@ -540,8 +540,9 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) acc[dt] *= alpha;
     }
-    // values of keys that do not exist yet may be anything: zero them (last block only)
-    if (kb * 64 + 64 > hi) {
+    // values of keys that do not exist yet, or that lie below the window (their pages may have
+    // been given back), may be anything: zero them (the last and the first block only)
+    if (kb * 64 + 64 > hi || kb * 64 < lo) {
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         const int key = kb * 64 + 32 * u + 8 * gq;
@@ -549,7 +550,7 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
           for (int e = 0; e < 8; ++e)
-            if (key + e >= hi) vf[u][dt].h[e] = 0;
+            if (key + e >= hi || key + e < lo) vf[u][dt].h[e] = 0;
       }
     }
     if (ROPE && makes_kv && kb == kb_new && gq == new_gq) {
@@ -808,12 +809,12 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
       {
         u32x4_t v = vreg[p];
         const int key = kb * 64 + v_key[p];
-        if (key + 8 > hi) {  // values of keys that do not exist yet may be anything
+        if (key + 8 > hi || key < lo) {  // values of keys that do not exist yet, or below the window, may be anything
           AFrag8 f;
           f.u = v;
 #pragma unroll
           for (int i = 0; i < 8; ++i)
-            if (key + i >= hi) f.h[i] = 0;
+            if (key + i >= hi || key + i < lo) f.h[i] = 0;
           v = f.u;
         }
         *reinterpret_cast<u32x4_t*>(&vs[v_dim[p]][v_key[p]]) = v;
