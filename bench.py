@@ -15,9 +15,13 @@ stops.
 Beside the headline the one JSON line holds: ``roofline`` (the bytes a decode step has to
 read, every weight once and the cache of the live requests, over its time, against 8 TB/s);
 ``prefill`` (2,048 tokens, the mean of three timed runs, with its fraction of 2.5 PFLOP/s);
-``points``: decode at batch 1 and 64 with the same roofline fraction each, and mixed steps at
-the Llama-3.2-3B shape (32 decode streams beside 480-token portions of 4,096-token prompts)
-with their bound max(bytes / 8 TB/s, flops / 2.5 PFLOP/s); ``breakdown``: the time of a
+``points``: decode at batch 1 and 64 with the same roofline fraction each; TTFT and TBT of the
+same workload as ``LLMEngine.generate`` itself reports them; prefill of 512 and 8,192 tokens,
+decode at batch 8 behind 8,000-token prompts and at batch 64 behind 4,000-token ones; mixed
+steps at the Llama-3.2-3B shape (32 decode streams beside 480-, 992- and 2,016-token portions
+of 4,096-token prompts) with their bound max(bytes / 8 TB/s, flops / 2.5 PFLOP/s); decode at
+batch 1 / 8 / 64 behind 2,048-token prompts at the Llama-3.1-70B shape (``--no-70b`` leaves
+it out); ``breakdown``: the time of a
 decode step and of the prefill by kind of work (products, attention, output head, norms),
 each with the fraction of the peak that bounds it.
 """
@@ -146,17 +150,39 @@ class Shape:
         return self.layers * (2 * t * self.layer_params + 2 * self.h * self.d * t * t) + 2 * self.vocab * self.c
 
 
-def make_runner(cfg: dict, max_batch: int, ctx_cap: int, graphs: bool = True, page: int = 64):
+def make_engine(cfg: dict, max_batch: int, ctx_cap: int, graphs: bool = True, page: int = 64, pool_tokens: int = 0):
+    """The engine as a user builds it over random weights of a shape (``LLMEngine.from_random``):
+    its runner is what the step-level measurements drive, its ``generate`` what the
+    generate-level ones call.  ``pool_tokens``: the pool's size when it is not ``max_batch``
+    requests of ``ctx_cap`` tokens."""
+    from yalis_amd import InferenceConfig, LLMEngine
     from yalis_amd.config.runtime import EngineConfig
-    from yalis_amd.engine.factory import random_runner
 
     pages_per_req = -(-ctx_cap // page)
+    max_len = min(cfg["max_position_embeddings"], pages_per_req * page)
     engine = EngineConfig(
-        page_size=page, num_pages=pages_per_req * max_batch, max_num_seqs=max_batch,
-        max_model_len=min(cfg["max_position_embeddings"], pages_per_req * page),
-        max_num_batched_tokens=8192, dtype="bfloat16", decode_graphs=graphs,
+        page_size=page, num_pages=-(-pool_tokens // page) if pool_tokens else pages_per_req * max_batch, max_num_seqs=max_batch,
+        max_model_len=max_len, max_num_batched_tokens=8192, dtype="bfloat16", decode_graphs=graphs,
     )
-    return random_runner(cfg, engine, seed=0)
+    ic = InferenceConfig(max_batch_size=max_batch, max_length_of_generated_sequences=max_len, temperature=0.0)
+    return LLMEngine.from_random(cfg, ic, precision="bf16", seed=0, engine_config=engine)
+
+
+def make_runner(cfg: dict, max_batch: int, ctx_cap: int, graphs: bool = True, page: int = 64):
+    return make_engine(cfg, max_batch, ctx_cap, graphs, page).runner
+
+
+def generate_metrics(engine, vocab: int, gen, batch: int, prompt_len: int, n_tokens: int):
+    """TTFT and TBT as ``LLMEngine.generate`` itself reports them (the reference's definitions,
+    yalis/engine.py:531-557) for ``batch`` prompts of ``prompt_len`` tokens; the second of two
+    calls (the first captures the decode graphs)."""
+    import torch
+
+    prompts = [torch.randint(0, vocab, (prompt_len,), generator=gen).tolist() for _ in range(batch)]
+    metrics = None
+    for _ in range(2):
+        _, metrics = engine.generate(prompts, tokens_to_generate=n_tokens, ignore_eos=True)
+    return metrics
 
 
 def decode_run(runner, vocab: int, gen, batch: int, prompt_len: int, steps: int, warmup: int):
@@ -367,6 +393,7 @@ def main() -> int:
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel (for hardware counters)")
     ap.add_argument("--shape", choices=("8b", "3b", "1b", "70b"), default="8b", help="layer sizes (default: the 8B shape of the headline)")
     ap.add_argument("--sample", action="store_true", help="time instead the choice of a token alone (greedy and each sampling rule) at the shape's vocabulary for --batch rows")
+    ap.add_argument("--no-70b", action="store_true", help="leave out the points at the Llama-3.1-70B shape (decode at batch 1 / 8 / 64 behind 2,048-token prompts; 141 GB of weights)")
     ap.add_argument("--probe", action="store_true", help="measure instead what a plain streaming read and a plain matrix-core loop reach on this card")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -401,7 +428,16 @@ def main() -> int:
 
     max_batch = max(args.batch, 1 if args.no_points else 64)
     total_steps = args.steps + args.warmup + 8
-    runner = make_runner(cfg, max_batch, max(args.prompt_len + total_steps + 1, args.prefill_len), graphs=not args.no_graphs)
+    ctx_cap = max(args.prompt_len + total_steps + 1, args.prefill_len)
+    pool_tokens = 0
+    further = not args.no_points and args.shape == "8b" and args.layers is None and not args.only_prefill
+    if further:
+        # further sizes: prompts of 8,192 tokens, batch 8 behind 8,000-token prompts, batch 64
+        # behind 4,000-token ones (the pool holds the largest of them)
+        ctx_cap = cfg["max_position_embeddings"]
+        pool_tokens = 64 * (4000 + 64 + 64)
+    engine = make_engine(cfg, max_batch, ctx_cap, graphs=not args.no_graphs, pool_tokens=pool_tokens)
+    runner = engine.runner
 
     if args.only_prefill:
         _, times = prefill_run(runner, shape.vocab, gen, args.prefill_len, runs=3)
@@ -456,20 +492,56 @@ def main() -> int:
             points[name] = round(b * steps / dtb, 2)
             # the same roofline as the headline: bytes the step has to read / its time / 8 TB/s
             points[name + "_frac"] = round(shape.decode_bytes(b, ctx_b) / (dtb / steps) / (HBM_GBPS * 1e9), 4)
+        # the same workload through LLMEngine.generate itself: its own TTFT and TBT (scheduler,
+        # sampler and the host's share included; the step-level figures above leave them out)
+        gm = generate_metrics(engine, shape.vocab, gen, args.batch, args.prompt_len, args.steps + 1)
+        points["generate_tbt_ms"] = round(gm["TBT"], 4)
+        points["generate_ttft_ms"] = round(gm["TTFT"], 3)
+        points["generate_tok_s"] = round(gm["Throughput"], 1)
+        if further:
+            for t2 in (512, 8192):
+                pf2, _ = prefill_run(runner, shape.vocab, gen, t2, runs=3)
+                points[f"prefill_{t2}_tok_s"] = round(t2 / pf2, 1)
+                points[f"prefill_{t2}_frac"] = round(shape.prefill_flops(t2) / pf2 / BF16_FLOPS, 4)
+            for b, plen, name in ((8, 8000, "decode_b8_ctx8k"), (64, 4000, "decode_b64_ctx4k")):
+                dtb, ctx_b = decode_run(runner, shape.vocab, gen, b, plen, 8, 2)
+                points[name] = round(b * 8 / dtb, 2)
+                points[name + "_frac"] = round(shape.decode_bytes(b, ctx_b) / (dtb / 8) / (HBM_GBPS * 1e9), 4)
         result["breakdown"] = breakdown(runner, shape, gen, args.batch, args.prompt_len, t)
-        del runner
+        del runner, engine
         torch.cuda.empty_cache()
-        # mixed steps at the Llama-3.2-3B shape: 32 decode streams beside 480-token portions of
-        # 4,096-token prompts (only with the headline's own shape and all its layers)
+        # mixed steps at the Llama-3.2-3B shape: 32 decode streams beside portions of 4,096-token
+        # prompts, 512, 1,024 and 2,048 rows a step (only with the headline's own shape and all
+        # its layers)
         if args.shape == "8b" and args.layers is None:
             name3, cfg3 = SHAPES["3b"]
             shape3 = Shape(cfg3)
-            ms3, bound3, _ = mixed_run(make_runner(dict(cfg3), 34, 4096 + 64), shape3, gen, args.prompt_len, 480)
-            points["mixed_3b_ms_per_step"] = round(ms3, 3)
-            points["mixed_3b_decode_tok_s"] = round(32 / ms3 * 1e3, 1)
-            points["mixed_3b_prefill_tok_s"] = round(480 / ms3 * 1e3, 1)
-            points["mixed_3b_bound_ms"] = round(bound3, 3)  # max(bytes / 8 TB/s, flops / 2.5 PFLOP/s)
-            points["mixed_3b_frac"] = round(bound3 / ms3, 4)
+            runner3 = make_runner(dict(cfg3), 34, 4096 + 64)
+            for portion, tag in ((480, "mixed_3b"), (992, "mixed_3b_p992"), (2016, "mixed_3b_p2016")):
+                ms3, bound3, _ = mixed_run(runner3, shape3, gen, args.prompt_len, portion)
+                if portion == 480:
+                    points["mixed_3b_ms_per_step"] = round(ms3, 3)
+                    points["mixed_3b_decode_tok_s"] = round(32 / ms3 * 1e3, 1)
+                    points["mixed_3b_prefill_tok_s"] = round(480 / ms3 * 1e3, 1)
+                    points["mixed_3b_bound_ms"] = round(bound3, 3)  # max(bytes / 8 TB/s, flops / 2.5 PFLOP/s)
+                else:
+                    points[tag + "_ms_per_step"] = round(ms3, 3)
+                    points[tag + "_prefill_tok_s"] = round(portion / ms3 * 1e3, 1)
+                points[tag + "_frac"] = round(bound3 / ms3, 4)
+            del runner3
+            torch.cuda.empty_cache()
+            if not args.no_70b and torch.cuda.mem_get_info()[0] > 200e9:
+                # BASELINE's fifth configuration: the Llama-3.1-70B shape (141 GB of weights on the
+                # one GPU), decode at batch 1, 8 and 64 behind 2,048-token prompts
+                name70, cfg70 = SHAPES["70b"]
+                shape70 = Shape(cfg70)
+                runner70 = make_runner(dict(cfg70), 64, 2048 + 64)
+                for b in (1, 8, 64):
+                    dtb, ctx_b = decode_run(runner70, shape70.vocab, gen, b, 2048, 6, 2)
+                    points[f"decode70b_b{b}"] = round(b * 6 / dtb, 2)
+                    points[f"decode70b_b{b}_frac"] = round(shape70.decode_bytes(b, ctx_b) / (dtb / 6) / (HBM_GBPS * 1e9), 4)
+                del runner70
+                torch.cuda.empty_cache()
         result["points"] = points
 
     print(json.dumps(result))

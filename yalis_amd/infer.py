@@ -28,7 +28,7 @@ def parse_args(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--model", "--model-path", dest="model_path", default=None, help="folder with config.json, model.safetensors (and a tokenizer for text prompts)")
     ap.add_argument("--random", dest="random_shape", default=None, metavar="SHAPE",
-                    help="no folder: random weights (seed: --random-weights-seed, default 0) of a named shape: 8b, 3b, 70b, tiny-a, tiny-b")
+                    help="no folder: random weights (seed: --random-weights-seed, default 0) of a named shape: 8b, 3b, 1b, 70b, tiny-a, tiny-b")
     ap.add_argument("--model-name", default=None)
     ap.add_argument("--precision", "--dtype", dest="precision", default="bf16", choices=["bf16", "fp32", "bfloat16", "float32"])
     ap.add_argument("--prompt", action="append", default=[], help="a text prompt (repeatable; needs a tokenizer)")
