@@ -210,6 +210,54 @@ def test_gemm_mfma_skinny_eight_waves(ops, forced):
     assert torch.equal(eight, ops.gemm_mfma_skinny(few, packed, torch.float32))
 
 
+@pytest.mark.parametrize("chunk", [128, 256])
+@pytest.mark.parametrize("waves", [4, 8])
+def test_gemm_mfma_skinny_wide_form(ops, forced, chunk, waves):
+    """33 to 64 rows of x in the wide form (32 x 32 x 16 products, a wave owns 32 weight rows),
+    forced here on every shape: sizes that are no multiples of a wave's 32 rows, of the chunk or
+    of 64 rows of x, one-hot operands that name the element every lane must hold, split and
+    unsplit, float32 and bfloat16 results, the activation in the epilogue (with a last tile
+    that holds one gate/up pair only); by the library's own rule it is taken at an unsliced K of 8,192."""
+    try:
+        ops.wide_skinny_products(2)
+        forced(chunk=chunk, waves=waves)
+        for m, n, k in [(64, 200, 4096), (50, 515, 328), (40, 1040, 2056), (33, 96, 1000), (100, 72, 520)]:
+            x = rnd((m, k), torch.bfloat16, 6)
+            w = rnd((n, k), torch.bfloat16, 7)
+            want = x.double().cpu() @ w.double().cpu().T
+            for slices in (1, 3):
+                forced(chunk=chunk, waves=waves, slices=slices)
+                close(ops.gemm_mfma_skinny(x, w, torch.float32), want, 2e-5 * math.sqrt(k), 1e-5)
+                part = ops.linear(x, w, torch.bfloat16, partial_ok=True)
+                close(part.reduce() if hasattr(part, "reduce") else part, want, 2e-2, 2**-7)
+            forced(chunk=chunk, waves=waves)
+        m, n, k = 40, 48, 64
+        for kk in (0, 7, 8, 15, 16, 40, 63):
+            x = torch.zeros((m, k), dtype=torch.bfloat16, device=DEV)
+            w = torch.zeros((n, k), dtype=torch.bfloat16, device=DEV)
+            x[:, kk] = torch.arange(1, m + 1, dtype=torch.bfloat16)
+            w[:, kk] = torch.arange(1, n + 1, dtype=torch.bfloat16) * 0.5
+            got = ops.gemm_mfma_skinny(x, w, torch.float32).cpu()
+            assert torch.equal(got, torch.outer(torch.arange(1, m + 1).float(), torch.arange(1, n + 1).float() * 0.5)), f"k={kk}"
+        for inter in (264, 512, 40):  # 528, 1024 and 80 rows of gate/up: the last tile is half, none, half
+            x = rnd((64, 1024), torch.bfloat16, 30, 0.7)
+            packed, group = ops.pack_gate_up(rnd((inter, 1024), torch.bfloat16, 31, 0.05), rnd((inter, 1024), torch.bfloat16, 32, 0.05))
+            got = ops.gate_up_act(x[:50], packed, group, "silu", torch.bfloat16)
+            plain = ops.gated_act(ops.linear(x[:50], packed, torch.bfloat16), "silu", torch.bfloat16, group=group)
+            assert torch.equal(got, plain), inter
+            ops.wide_skinny_products(0)
+            assert torch.equal(got, ops.gate_up_act(x[:50], packed, group, "silu", torch.bfloat16))
+            ops.wide_skinny_products(2)
+        ops.wide_skinny_products(1)
+        forced()
+        forced(slices=1)
+        x, w = rnd((48, 8192), torch.bfloat16, 8, 0.3), rnd((136, 8192), torch.bfloat16, 9, 0.05)
+        by_rule = ops.gemm_mfma_skinny(x, w, torch.float32)
+        close(by_rule, x.double().cpu() @ w.double().cpu().T, 2e-5 * math.sqrt(8192), 1e-5)
+    finally:
+        ops.wide_skinny_products(1)
+
+
 def test_forced_slice_counts_reach_the_consumers(ops, forced):
     """The number of K slices a product leaves behind is what the launch says it wrote, also
     when the plan is forced after the library was first asked about the shape."""

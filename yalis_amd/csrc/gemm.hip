@@ -156,6 +156,18 @@ static size_t skinny_lds_bytes(int mt, int waves, int kc) {
 // short chunks for slices of up to 1,792, up to 4,096 with 64 rows of x.
 // What yk_gemm_skinny_force set (0: the library decides): for tests and measurements only.
 static int g_force_chunk = 0, g_force_waves = 0, g_force_slices = 0;
+// 33 to 64 rows of x against a K of 8,192 and more that one workgroup walks whole (no K slices:
+// in practice gate/up with the activation in its epilogue): the wide form (32 x 32 x 16
+// products, two waves of 32 weight rows a workgroup).  Measured (us, 16-row form / wide form):
+// the 70B shape's gate/up (57,344 x 8,192) at 64 / 48 / 33 rows of x 200 / 186, 191 / 167,
+// 187 / 161.  Elsewhere it does not pay: the same shape's sliced products at 64 rows, down-proj
+// 97.4 / 98.4, qkv 33.8 / 43.5, o-proj 33.6 / 36.5; at a K of 4,096 (the 8B shape at 64 rows)
+// gate/up 50.2 / 52.2 with four waves of 32 rows and 57.4 with two, down-proj 23.7 / 26.1, qkv
+// 14.2 / 15.9.  The wide form halves the reads of x from LDS per weight byte, but a workgroup
+// has half the waves to keep loads in flight, which counts for more wherever a workgroup's walk
+// over K is short.  yk_gemm_skinny_wide: 0 never, 1 by this rule, 2 always (tests, measurements).
+static int g_wide = 1;
+constexpr int SK_WIDE_MIN_K = 8192;
 
 static int skinny_chunk(int mt, int k_block) {
   if (g_force_chunk) return g_force_chunk;
@@ -386,6 +398,162 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
   }
 }
 
+// The wide form, for 33 to 64 rows of x: v_mfma_f32_32x32x16_bf16 (64 lanes, c = lane % 32,
+// hl = lane / 32):
+//   A (32 x 16): lane holds A[c][8 hl .. 8 hl + 7];  B (16 x 32): lane holds B[8 hl .. 8 hl + 7][c];
+//   C (32 x 32): lane holds C[8 (v / 4) + 4 hl + v % 4][c] in accumulator v = 0 .. 15.
+// A = 32 rows of the weight, B = 32 rows of x, two B tiles a wave: every weight fragment read
+// from LDS meets two fragments of x, where the 16-row form reads four (and half as large a
+// piece of the weight) - at 64 rows of x those reads are what the workgroup's time goes to.
+// A workgroup of W waves owns 32 W weight rows and 64 rows of x over one slice of K; all else
+// (chunks, loads of two rows x 512 bytes or four x 256, parking in wave-private LDS, x staged
+// once a workgroup, clamped addresses instead of conditions) is the 16-row form's.
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+template <int W, typename TO, int GATED, int KC>
+__global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_wide_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, float* __restrict__ part,
+    TO* __restrict__ y, int M, int N, int K, int ldx, int ldw, int ldy, int k_block) {
+  extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
+  constexpr int STEPS = KC / 16;               // matrix-core steps per chunk
+  constexpr int ROW = KC + SK_PAD;             // an LDS row
+  constexpr int LOADS = KC / 16;               // 16-byte loads a lane makes for a chunk of the wave's 32 rows
+  constexpr int LPR = KC / 8, RPL = 64 / LPR;  // lanes that load one weight row's chunk; rows per load
+  constexpr int XB = skinny_x_buffers(4, KC);
+  bf16_t(*xs0)[ROW] = reinterpret_cast<bf16_t(*)[ROW]>(lds);  // XB x [64][ROW]
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  bf16_t(*wl)[ROW] = reinterpret_cast<bf16_t(*)[ROW]>(lds + static_cast<size_t>(64 * XB) * ROW + static_cast<size_t>(32 * wave) * ROW);
+  const int c = lane % 32, hl = lane / 32;
+  const int n0 = (blockIdx.x * W + wave) * 32;
+  const int m0 = blockIdx.y * 64;
+  const int kb0 = blockIdx.z * k_block;
+  const int kb1 = min(K, kb0 + k_block);
+
+  f32x16_t acc[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+
+  const int half = lane / LPR, l32 = lane % LPR;
+  const bf16_t* wrow[LOADS];
+#pragma unroll
+  for (int j = 0; j < LOADS; ++j) wrow[j] = w + static_cast<size_t>(min(n0 + RPL * j + half, N - 1)) * ldw;
+  const int k_last = K - 8;
+  u32x4_t regs[LOADS];
+#define SKW_LOAD_W(KC0)                                                                     \
+  {                                                                                          \
+    const int kk_ = min((KC0) + 8 * l32, k_last);                                            \
+    _Pragma("unroll") for (int j = 0; j < LOADS; ++j)                                        \
+        regs[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wrow[j] + kk_)); \
+  }
+  constexpr int XP = 64 * (KC / 8) / (W * 64);
+  static_assert(XP * W * 64 == 64 * (KC / 8), "x pieces must divide evenly over the threads");
+  const u32x4_t zero = {0u, 0u, 0u, 0u};
+  u32x4_t xr[XP];
+#pragma unroll
+  for (int p = 0; p < XP; ++p) xr[p] = zero;
+#define SKW_LOAD_X(KC0)                                                                     \
+  _Pragma("unroll") for (int p = 0; p < XP; ++p) {                                           \
+    const int e_ = threadIdx.x + p * W * 64;                                                 \
+    const int m_ = m0 + e_ / (KC / 8), k_ = (KC0) + 8 * (e_ % (KC / 8));                     \
+    if (m_ < M) xr[p] = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(m_) * ldx + min(k_, k_last)); \
+  }
+  const int n_chunks = (kb1 - kb0 + KC - 1) / KC;
+  SKW_LOAD_W(kb0)
+  SKW_LOAD_X(kb0)
+  int turn = 0;
+  for (int ci = 0; ci < n_chunks; ++ci, turn ^= 1) {
+    const int kc = kb0 + ci * KC;
+    if (XB == 1) __syncthreads();
+    bf16_t(*xs)[ROW] = xs0 + (XB == 2 ? turn * 64 : 0);
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j) *reinterpret_cast<u32x4_t*>(&wl[RPL * j + half][8 * l32]) = regs[j];
+#pragma unroll
+    for (int p = 0; p < XP; ++p) {
+      const int e = threadIdx.x + p * W * 64;
+      const bool outside = m0 + e / (KC / 8) >= M || kc + 8 * (e % (KC / 8)) >= kb1;
+      *reinterpret_cast<u32x4_t*>(&xs[e / (KC / 8)][8 * (e % (KC / 8))]) = outside ? zero : xr[p];
+    }
+    if (ci + 1 < n_chunks) {
+      SKW_LOAD_W(kc + KC)
+      SKW_LOAD_X(kc + KC)
+    }
+    __syncthreads();
+    constexpr int AHEAD = 3;
+    Frag8 a[STEPS], b[STEPS][2];
+#define SKW_READ(U)                                                                         \
+  {                                                                                          \
+    a[U].u = *reinterpret_cast<const u32x4_t*>(&wl[c][16 * (U) + 8 * hl]);                   \
+    b[U][0].u = *reinterpret_cast<const u32x4_t*>(&xs[c][16 * (U) + 8 * hl]);                \
+    b[U][1].u = *reinterpret_cast<const u32x4_t*>(&xs[32 + c][16 * (U) + 8 * hl]);           \
+  }
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) SKW_READ(u)
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < STEPS; ++u) {
+      if (u + AHEAD < STEPS) {
+        SKW_READ(u + AHEAD)
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[u].v, b[u][0].v, acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[u].v, b[u][1].v, acc[1], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#undef SKW_READ
+  }
+#undef SKW_LOAD_W
+#undef SKW_LOAD_X
+
+  if (GATED) {
+    // The weight's rows alternate 8 gate rows / their 8 up rows: of a wave's 32 rows, 0-7 and
+    // 16-23 are gates, 8-15 and 24-31 their ups.  Accumulators 0-3 of a lane are four gate
+    // features (4 hl .. 4 hl + 3) of one token, accumulators 4-7 the up features that belong
+    // to them; 8-11 and 12-15 the second pair of groups.
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int m = m0 + 32 * t + c;
+      if (m >= M) continue;
+#pragma unroll
+      for (int pair = 0; pair < 2; ++pair) {
+        if (n0 + 16 * pair >= N) continue;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          y[static_cast<size_t>(m) * ldy + n0 / 2 + 8 * pair + 4 * hl + e] =
+              from_f32<TO>(act_apply(as_output(acc[t][8 * pair + e], 1), GATED - 1) * as_output(acc[t][8 * pair + 4 + e], 1));
+      }
+    }
+    return;
+  }
+  const bool to_part = part != nullptr;
+  float* pout = to_part ? part + static_cast<size_t>(blockIdx.z) * M * N : nullptr;
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int m = m0 + 32 * t + c;
+    if (m >= M) continue;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int n = n0 + 8 * q + 4 * hl;
+      if (n >= N) continue;
+      if (to_part && n + 3 < N && N % 4 == 0) {
+        *reinterpret_cast<f32x4_t*>(pout + static_cast<size_t>(m) * N + n) =
+            f32x4_t{acc[t][4 * q], acc[t][4 * q + 1], acc[t][4 * q + 2], acc[t][4 * q + 3]};
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (n + e < N) {
+            if (to_part)
+              pout[static_cast<size_t>(m) * N + n + e] = acc[t][4 * q + e];
+            else
+              y[static_cast<size_t>(m) * ldy + n + e] = from_f32<TO>(acc[t][4 * q + e]);
+          }
+        }
+      }
+    }
+  }
+}
+
 // y[m][n] = sum over splits of part[s][m][n], in the order of s
 template <typename TO>
 __global__ void reduce_splits_kernel(const float* __restrict__ part, TO* __restrict__ y, int M,
@@ -472,6 +640,12 @@ extern "C" int yk_gemm_skinny_force(int chunk, int waves, int slices) {
   return 0;
 }
 
+extern "C" int yk_gemm_skinny_wide(int mode) {
+  YK_REQUIRE(mode >= 0 && mode <= 2, "gemm_skinny_wide: 0 never, 1 by the library's rule, 2 always");
+  g_wide = mode;
+  return 0;
+}
+
 // gated != 0: the plan of a product with the activation in its epilogue (1: it can be fused).
 extern "C" int yk_gemm_skinny_splits(int M, int N, int K, int gated) { return skinny_plan(M, N, K, gated != 0, nullptr, nullptr); }
 
@@ -501,6 +675,34 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, i
   dim3 block(waves * 64);
   const int kc = skinny_chunk(mt, k_block);
   const size_t lds = skinny_lds_bytes(mt, waves, kc);
+  if (mt == 4 && (g_wide == 2 || (g_wide == 1 && K >= SK_WIDE_MIN_K && splits == 1))) {
+    // waves of 32 weight rows: two of them (64 rows a workgroup) by the rule, half the plan's
+    // number (the plan's rows a workgroup) when forced
+    const int ww = g_wide == 2 ? waves / 2 : 2;
+    dim3 wblock(ww * 64);
+    grid.x = (N + 32 * ww - 1) / (32 * ww);
+    const size_t lds = skinny_lds_bytes(mt, 2 * ww, kc);
+#define SKW_GO(W_, G_) SKW_GO_KC(W_, G_, 128) SKW_GO_KC(W_, G_, 256)
+#define SKW_GO_KC(W_, G_, KC_)                                                                          \
+  if (ww == W_ && gated == G_ && kc == KC_) {                                                           \
+    static bool raised = false;                                                                         \
+    if (!raised) {                                                                                      \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_wide_kernel<W_, TO, G_, KC_>), \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)    \
+        return yk_fail("gemm_mfma_skinny: cannot raise the LDS limit");                                 \
+      raised = true;                                                                                    \
+    }                                                                                                   \
+    gemm_mfma_skinny_wide_kernel<W_, TO, G_, KC_><<<grid, wblock, lds, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block); \
+    return yk_check_launch("gemm_mfma_skinny (wide)");                                                  \
+  }
+    SKW_GO(2, 0) SKW_GO(4, 0)
+    if constexpr (sizeof(TO) == 2) {
+      SKW_GO(2, 1) SKW_GO(4, 1) SKW_GO(2, 2) SKW_GO(4, 2)
+    }
+#undef SKW_GO
+#undef SKW_GO_KC
+    return yk_fail("gemm_mfma_skinny: no wide kernel for this plan");
+  }
 #define SK_GO(MT_, W_, G_) SK_GO_KC(MT_, W_, G_, 128) SK_GO_KC(MT_, W_, G_, 256)
 #define SK_GO_KC(MT_, W_, G_, KC_)                                                                       \
   if (mt == MT_ && waves == W_ && gated == G_ && kc == KC_) {                                           \

@@ -66,6 +66,7 @@ _SIGNATURES = {
     ),
     "yk_gemm_skinny_splits": ([_c_int, _c_int, _c_int, _c_int], _c_int),
     "yk_gemm_skinny_force": ([_c_int, _c_int, _c_int], _c_int),
+    "yk_gemm_skinny_wide": ([_c_int], _c_int),
     "yk_gemm_library": ([_vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_size_t, _vp, _vp], _c_int),
     "yk_gemm_library_tune": ([_c_int], _c_int),
     "yk_gemm_mfma_skinny": (
@@ -115,7 +116,7 @@ _LATER_SIGNATURES = {
         "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
     },
 }
-_ABI = 14
+_ABI = 15
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
 # above it the vendor library does.
@@ -324,6 +325,12 @@ class HipOps:
         workgroup and number of K slices (0: the library decides); call without arguments to clear."""
         self._check(self.lib.yk_gemm_skinny_force(int(chunk), int(waves), int(slices)))
         self._answers = {k: v for k, v in self._answers.items() if k[0] not in ("yk_gemm_skinny_splits", "yk_gemm_skinny_from_attention_ok")}
+
+    def wide_skinny_products(self, mode: int = 1) -> None:
+        """For tests and measurements: when few-row products of 33 to 64 rows run in the wide form
+        (32 x 32 x 16 matrix-core products): 0 never, 1 where the library's rule says so (the
+        default: an unsliced K of 8,192 and more), 2 always."""
+        self._check(self.lib.yk_gemm_skinny_wide(int(mode)))
 
     def tune_library_products(self, on: bool = True) -> None:
         """Whether new shapes of up to 256 rows get the vendor library's first candidate (the
