@@ -258,6 +258,59 @@ def test_gemm_mfma_skinny_wide_form(ops, forced, chunk, waves):
         ops.wide_skinny_products(1)
 
 
+def test_gemm_tile(ops):
+    """The product in tiles of 128 x 128 for some dozens to a few hundred rows: sizes that are no
+    multiples of the tile or of the step of 64 along K, one-hot operands, K cut into 1 to 8 slices
+    (an odd number of steps in a slice, a last slice shorter than the others), float32 and
+    bfloat16 results, slices kept for a consumer; and where ``linear`` takes it by itself."""
+    from yalis_amd.ops.hip import SplitSum
+
+    try:
+        for m, n, k in [(65, 200, 4096), (128, 128, 64), (130, 515, 328), (256, 1040, 2056), (200, 96, 1000), (300, 136, 8192), (1, 8, 8)]:
+            x = rnd((m, k), torch.bfloat16, 6)
+            w = rnd((n, k), torch.bfloat16, 7)
+            want = x.double().cpu() @ w.double().cpu().T
+            for slices in (0, 1, 2, 3, 8):
+                ops.force_tile_slices(slices)
+                close(ops.gemm_tile(x, w, torch.float32), want, 2e-5 * math.sqrt(k), 1e-5)
+                part = ops.gemm_tile(x, w, torch.bfloat16, partial_ok=True)
+                if isinstance(part, SplitSum):
+                    assert part.out_dtype == torch.bfloat16 and 1 < part.n_splits <= max(slices, 8)
+                    close(part.reduce(), want, 2e-2, 2**-7)
+                    res = rnd((m, n), torch.float32, 8)
+                    got = ops.add_rmsnorm(res.clone(), part, torch.ones(n, device=DEV), 1e-5, False, torch.float32)
+                    part = ops.gemm_tile(x, w, torch.bfloat16, partial_ok=True)
+                    summed = part.tensor[0].clone()  # the consumers add the slices one after the other
+                    for sl in range(1, part.n_splits):
+                        summed += part.tensor[sl]
+                    plain = ops.add_rmsnorm(res.clone(), summed.to(torch.bfloat16), torch.ones(n, device=DEV), 1e-5, False, torch.float32)
+                    assert torch.equal(got, plain), "the slices' consumers round their sum as the product's output would have been"
+                else:
+                    close(part, want, 2e-2, 2**-7)
+        ops.force_tile_slices(0)
+        m, n, k = 150, 140, 128
+        for kk in (0, 7, 8, 15, 16, 63, 64, 127):
+            x = torch.zeros((m, k), dtype=torch.bfloat16, device=DEV)
+            w = torch.zeros((n, k), dtype=torch.bfloat16, device=DEV)
+            x[:, kk] = torch.arange(1, m + 1, dtype=torch.bfloat16)
+            w[:, kk] = torch.arange(1, n + 1, dtype=torch.bfloat16) * 0.5
+            got = ops.gemm_tile(x, w, torch.float32).cpu()
+            assert torch.equal(got, torch.outer(torch.arange(1, m + 1).float(), torch.arange(1, n + 1).float() * 0.5)), f"k={kk}"
+        # rows of x and w with gaps between them
+        xs, wsrc = rnd((100, 4096 + 16), torch.bfloat16, 9), rnd((72, 4096 + 8), torch.bfloat16, 10)
+        close(ops.gemm_tile(xs[:, :4096], wsrc[:, :4096], torch.float32), xs[:, :4096].double().cpu() @ wsrc[:, :4096].double().cpu().T, 2e-5 * 64, 1e-5)
+        # a down projection of 65 to 256 rows is this kernel's by linear's own choice
+        assert ops.long_matrix_tiles(128, 4096, 14336) and not ops.long_matrix_tiles(64, 4096, 14336)
+        assert not ops.long_matrix_tiles(300, 4096, 14336) and not ops.long_matrix_tiles(128, 4096, 4096)
+        x, w = rnd((100, 4096), torch.bfloat16, 11, 0.3), rnd((520, 4096), torch.bfloat16, 12, 0.05)
+        y = ops.linear(x, w, torch.bfloat16, partial_ok=True)
+        assert isinstance(y, SplitSum)
+        close(y.reduce(), x.double().cpu() @ w.double().cpu().T, 2e-2, 2**-7)
+        close(ops.linear(x, w, torch.bfloat16), x.double().cpu() @ w.double().cpu().T, 2e-2, 2**-7)
+    finally:
+        ops.force_tile_slices(0)
+
+
 def test_forced_slice_counts_reach_the_consumers(ops, forced):
     """The number of K slices a product leaves behind is what the launch says it wrote, also
     when the plan is forced after the library was first asked about the shape."""

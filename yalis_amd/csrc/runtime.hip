@@ -17,4 +17,4 @@ int yk_check_launch(const char* what) {
   return 0;
 }
 extern "C" const char* yk_last_error() { return yk_error_slot().c_str(); }
-extern "C" int yk_abi_version() { return 15; }
+extern "C" int yk_abi_version() { return 16; }

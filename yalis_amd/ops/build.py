@@ -28,7 +28,7 @@ HOST_SOURCES = ["cache_manager.cpp"]
 # "kernels" only (so that is all a trace replay compiles), choosing tokens "sampling", the
 # benchmark's machine probes "probe".  Every library carries runtime.hip (its error slot).
 KERNEL_LIBS = {
-    "kernels": ["runtime.hip", "elementwise.hip", "gemm.hip", "attention.hip", "library_gemm.hip"],
+    "kernels": ["runtime.hip", "elementwise.hip", "gemm.hip", "gemm_tile.hip", "attention.hip", "library_gemm.hip"],
     "sampling": ["runtime.hip", "sampling.hip"],
     "probe": ["runtime.hip", "probe.hip"],
 }

@@ -73,6 +73,12 @@ _SIGNATURES = {
         [_vp, _vp, _vp, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
         _c_int,
     ),
+    "yk_gemm_tile": (
+        [_vp, _vp, _vp, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
+        _c_int,
+    ),
+    "yk_gemm_tile_splits": ([_c_int, _c_int, _c_int], _c_int),
+    "yk_gemm_tile_force": ([_c_int], _c_int),
     "yk_attn_generic": (
         [_vp, _c_int, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp],
         _c_int,
@@ -116,7 +122,7 @@ _LATER_SIGNATURES = {
         "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
     },
 }
-_ABI = 15
+_ABI = 16
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
 # above it the vendor library does.
@@ -508,6 +514,8 @@ class HipOps:
         bf = torch.bfloat16
         aligned = k % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
         if x.dtype == bf and w.dtype == bf and aligned:
+            if out_dtype == bf and self.long_matrix_tiles(m, n, k):
+                return self.gemm_tile(x, w, bf, partial_ok)
             if m > SKINNY_MAX_ROWS and out_dtype == bf and not self.few_library_tiles(m, n):
                 return self.gemm_library(x, w, bf)  # vendor library, bfloat16 in and out
             if m > SKINNY_MAX_ROWS and out_dtype == torch.float32:
@@ -516,6 +524,19 @@ class HipOps:
                 return self.gemm_library(x, w, torch.float32)
             return self.gemm_mfma_skinny(x, w, out_dtype, partial_ok)
         return self.gemm_fma(x, w, out_dtype)
+
+    @staticmethod
+    def long_matrix_tiles(m: int, n: int, k: int) -> bool:
+        """Whether a product of 65 to 256 rows is ``gemm_tile``'s: where the matrix is at least twice
+        as long as it is wide (a down projection), so that tiles of 128 x 128 cut along K occupy
+        the GPU and the slices are long.  Measured in replayed graphs (us, vendor library's first
+        candidate / few-row kernel / tiles): 8B down-proj (4,096 x 14,336) at 72 rows 36.6 / 37.2 /
+        25.6, at 128 57.9 / 35.4 / 27.0, at 192 77.5 / 65.9 / 49.3, at 256 45.9 / - / 47.5; 3B
+        (3,072 x 8,192) at 128 32.9 / 19.6 / 17.7, at 192 45.3 / 27.5 / 28.5; 70B (8,192 x 28,672) at
+        128 200 / 167 / 110, at 256 314 / - / 200; 1B (2,048 x 8,192) at 192 22.9 / 19.7 / 18.2.  On
+        squarer matrices the three are within a tenth of each other up to 128 rows, and from 384
+        rows on the library wins everywhere."""
+        return SKINNY_MAX_ROWS < m <= 256 and k >= 2 * n and k >= 4096
 
     @staticmethod
     def few_library_tiles(m: int, n: int) -> bool:
@@ -571,6 +592,32 @@ class HipOps:
             x.data_ptr(), w.data_ptr(), y.data_ptr(), _code(out_dtype), m, n, k, x.stride(0), w.stride(0), n,
             self._library_workspace.data_ptr(), self._library_workspace.numel(), None, self._stream()))
         return y
+
+    def gemm_tile(self, x, w, out_dtype, partial_ok: bool = False):
+        """x [M, K] . w [N, K]^T in tiles of 128 x 128 on the matrix cores (bfloat16 operands with
+        16-byte aligned rows): the kernel for some dozens to a few hundred rows against long
+        matrices.  Where its plan cuts K the result comes as a ``SplitSum`` (with ``partial_ok``)
+        or is summed here."""
+        m, k = x.shape
+        n = w.shape[0]
+        splits = self._ask("yk_gemm_tile_splits", m, n, k)
+        ws = self._gemm_ws(splits * m * n) if splits > 1 else None
+        y = None if splits > 1 else torch.empty((m, n), dtype=out_dtype, device=x.device)
+        rc = self.lib.yk_gemm_tile(
+            x.data_ptr(), w.data_ptr(), _ptr(y), _code(out_dtype), _ptr(ws), 0 if ws is None else ws.numel(),
+            m, n, k, x.stride(0), w.stride(0), n, self._stream(),
+        )
+        if rc < 0:
+            raise KernelError(self.lib.yk_last_error().decode())
+        if rc == 0:
+            return y
+        part = SplitSum(ws[: rc * m * n].view(rc, m, n), out_dtype, self, self._gemm_gen)
+        return part if partial_ok else part.reduce().to(out_dtype)
+
+    def force_tile_slices(self, slices: int = 0) -> None:
+        """For tests and measurements: force the K slices of ``gemm_tile`` (0: the library decides)."""
+        self._check(self.lib.yk_gemm_tile_force(int(slices)))
+        self._answers = {k: v for k, v in self._answers.items() if k[0] != "yk_gemm_tile_splits"}
 
     def gemm_fma(self, x, w, out_dtype):
         m, k = x.shape
