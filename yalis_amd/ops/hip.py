@@ -642,9 +642,46 @@ class HipOps:
         inter = w_gate.shape[0]
         g = self.GATE_UP_GROUP
         if w_gate.dtype == torch.bfloat16 and w_up.dtype == torch.bfloat16 and inter % g == 0:
-            packed = torch.stack([w_gate.view(inter // g, g, -1), w_up.view(inter // g, g, -1)], dim=1)
-            return packed.reshape(2 * inter, -1).contiguous(), g
+            k = w_gate.shape[1]
+            packed = self._rows_apart(2 * inter, k, w_gate.device)
+            packed.view(inter // g, 2, g, k)[:, 0].copy_(w_gate.view(inter // g, g, k))
+            packed.view(inter // g, 2, g, k)[:, 1].copy_(w_up.view(inter // g, g, k))
+            return packed, g
         return torch.cat([w_gate, w_up], dim=0).contiguous(), 0
+
+    # Rows of a streamed bfloat16 matrix that would lie a multiple of 4 KiB apart are kept 128 bytes
+    # further apart.  Workgroups of the few-row product that walk all of K in step (gate/up, the
+    # output head: their K is not sliced) ask, at every moment, for addresses a whole number of
+    # rows apart, and rows 4 KiB apart crowd onto few memory channels.  Up to 32 rows of x the
+    # product answers that by starting its workgroups at different places of K; with more rows
+    # they must stay in step (they share the staged rows of x through L2: started apart, gate/up
+    # at 64 rows went 50 -> 64 us), and the gap between rows does it instead: 8B shape, us, rows 8 KiB
+    # apart / 128 bytes more: gate/up at 64 rows of x 52.0 / 45.6, at 48 48.0 / 42.6, the head at 64
+    # 221 / 197, at 48 212 / 184; at 32 rows and fewer no difference (42.2 / 43.3, 37.0 / 37.5).  The
+    # sliced products (qkv, o-proj, down-proj) are better off without (qkv at 64 rows 14.0 / 15.7),
+    # and so are rows of 16 KiB (the 70B shape's gate/up at 64 / 8 rows 196 / 223, 151 / 178): the
+    # gap is for rows of 4 and 8 KiB (the 1B shape's head at 64 rows 120 / 110).
+    ROW_GAP = 64  # elements
+
+    @staticmethod
+    def _rows_crowd(k: int) -> bool:
+        return 2 * k in (4096, 8192)
+
+    def _rows_apart(self, rows: int, k: int, device) -> torch.Tensor:
+        """An uninitialised bfloat16 [rows, k], its rows 128 bytes further apart where that pays."""
+        if self._rows_crowd(k):
+            return torch.empty((rows, k + self.ROW_GAP), dtype=torch.bfloat16, device=device)[:, :k]
+        return torch.empty((rows, k), dtype=torch.bfloat16, device=device)
+
+    def streamed_matrix(self, w: torch.Tensor) -> torch.Tensor:
+        """``w`` as a part should keep it when all it does with it is multiply few rows by it with
+        K unsliced (an output head): ``w`` itself, or a copy with its rows 128 bytes further apart
+        (see above)."""
+        if w.dim() != 2 or w.dtype != torch.bfloat16 or not w.is_contiguous() or not self._rows_crowd(w.shape[1]):
+            return w
+        out = self._rows_apart(w.shape[0], w.shape[1], w.device)
+        out.copy_(w)
+        return out
 
     def gate_up_act(self, x: torch.Tensor, w_gate_up: torch.Tensor, group: int, activation: str, out_dtype: torch.dtype) -> torch.Tensor:
         """act(x . gate^T) * (x . up^T) -> [M, intermediate], ``w_gate_up`` and ``group`` as

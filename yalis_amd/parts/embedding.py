@@ -72,6 +72,12 @@ class LMHead(Part):
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.weight = tensors[self.tied_to if self.tied_to is not None else self.name]
+        if self.tied_to is None:
+            # a table of its own: kept the way the kernel library streams it best (a tied table
+            # stays as the embedding gathers from it)
+            keep = getattr(self.rt.ops, "streamed_matrix", None)
+            if keep is not None:
+                self.weight = keep(self.weight)
 
     def products(self):
         return ((self.vocab, self.hidden),)
