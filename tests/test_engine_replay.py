@@ -328,6 +328,37 @@ def test_graph_replays_match_eager_steps(dtype):
     C.assert_matches({"r3": torch.cat([want["r3"][:0], outs[True]["a"]])}, {"r3": want["r3"][100:]}, dtype == "bfloat16", "graph decode")
 
 
+@pytest.mark.gpu
+def test_captured_graphs_are_bounded():
+    """Captured decode graphs are kept least recently replayed first and dropped beyond the
+    engine's bound on what they may hold: with a bound of one byte every new shape of step drops
+    the one before (and is captured again when it returns), and the logits are what they are
+    with the default bound."""
+    cfg, weights, reqs, want = setup("C", "bfloat16")
+    a, b = reqs["r3"], reqs["r2"]
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:30], "want": []}, {"id": "b", "tokens": b[:20], "want": []}], "end": []}]
+    for j in range(12):  # two requests, then one, then two again, ...: two shapes of step by turns
+        entries = [{"id": "a", "tokens": [a[30 + j]], "want": [0]}]
+        if j % 2 == 0:
+            entries.append({"id": "b", "tokens": [b[20 + j // 2]], "want": [0]})
+        steps.append({"step": 1 + j, "entries": entries, "end": []})
+    outs = {}
+    for bound in (1 << 30, 1):
+        runner = C.make_runner(cfg, weights, "bfloat16", "cuda:0", ops_for("cuda:0"), 16, 24)
+        runner.config.graph_memory_bytes = bound
+        got, _ = C.run_trace(runner, steps)
+        outs[bound] = got
+        assert runner.graph_replays == 12
+        if bound == 1:
+            assert len(runner._graphs) == 1 and runner.graphs_dropped == 11
+        else:
+            assert len(runner._graphs) == 2 and runner.graphs_dropped == 0 and 0 < runner.graph_bytes() < bound
+        runner.drop_graphs()
+        assert not runner._graphs
+    assert torch.equal(outs[1]["a"], outs[1 << 30]["a"]) and torch.equal(outs[1]["b"], outs[1 << 30]["b"])
+    C.assert_matches({"r3": outs[1]["a"]}, {"r3": want["r3"][30:42]}, True, "graphs dropped and captured again")
+
+
 def _many_requests_trace(cfg, n_live, seed):
     """``n_live`` short requests: whole prompts eight to a step, then steps that hold one token of
     every request still running; request i decodes 3 + i % 4 tokens, so that a quarter of the

@@ -275,6 +275,58 @@ def toy_plain(weights, tokens, rounder=P._identity):
     return norm(x, "toy.final") @ w("toy.head").T
 
 
+# ---------------------------------------------- a model whose only cache group has a window
+def build_window_only_spec(c: ToyConfig) -> ModelSpec:
+    spec = build_toy_spec(c)
+    import dataclasses
+
+    return dataclasses.replace(spec, architecture="ToyWindowOnlyForCausalLM", run_order=(RunEntry(2),))
+
+
+register_architecture("ToyWindowOnlyForCausalLM", ToyConfig, build_window_only_spec)
+
+
+def test_a_windowed_group_is_sized_by_its_window():
+    """A model whose every cache keeps a window of 24 tokens only: a request of 150 cached tokens
+    never holds more than the window plus one step's tokens, so a pool of 4 pages of 16 takes it
+    under a budget of 16 tokens a step (the whole length would need 10), a pool of 3 does not, and
+    the tokens generated from the small pool are those from a large one."""
+    from yalis_amd.engine.scheduler import Scheduler
+    from yalis_amd.sampling.sampler import SamplingParams
+
+    cfg = dict(TOY, architectures=["ToyWindowOnlyForCausalLM"])
+    prompt = C.make_requests({"vocab_size": TOY["vocab_size"]}, [120], seed=9)["r0"]
+    outs = {}
+    for pages in (4, 40, 3):
+        eng = EngineConfig(page_size=16, num_pages=pages, max_num_seqs=2, max_model_len=256, max_num_batched_tokens=16,
+                           dtype="float32", device="cpu")
+        model = build_model(cfg, eng, ops=RefOps())
+        model.load({k: v for k, v in random_tensors(model.tensor_specs(), 3, torch.float32)})
+        runner = ModelRunner(model, eng)
+        assert [g.window for g in runner.group_shapes] == [24]
+        sched = Scheduler(runner)
+        assert sched.pages_a_request_needs(150, 24) == 4 and sched.pages_a_request_needs(150, None) == 10
+        assert sched.pages_a_request_needs(20, 24) == 2, "a short request is sized by its length"
+        if pages == 3:
+            with pytest.raises(ValueError, match="a window of 24"):
+                sched.add(prompt, SamplingParams(temperature=0.0, max_tokens=31))
+            continue
+        req = sched.add(prompt, SamplingParams(temperature=0.0, max_tokens=31))
+        steps = 0
+        while sched.has_work():
+            plan = sched.schedule()
+            assert plan, "the scheduler made no progress"
+            logits = runner.step(sched.entries(plan))
+            sched.update(plan, logits.argmax(-1).tolist())
+            steps += 1
+            assert steps < 200
+        assert req.preemptions == 0 and len(req.output) == 31
+        runner.pages.audit()
+        assert runner.pages.live_requests() == 0 and runner.pages.free_pages(0) == pages
+        outs[pages] = req.output
+    assert outs[4] == outs[40]
+
+
 def make_toy_runner(device, dtype, num_pages):
     eng = EngineConfig(page_size=16, num_pages=num_pages, max_num_seqs=4, max_model_len=256, dtype=dtype, device=device)
     ops = RefOps() if device == "cpu" else None
