@@ -52,6 +52,12 @@ def parse_args(argv=None):
     ap.add_argument("--page-size", type=int, default=64)
     ap.add_argument("--num-pages", type=int, default=None)
     ap.add_argument("--max-num-batched-tokens", "--max-batched-tokens", dest="max_num_batched_tokens", type=int, default=2048)
+    ap.add_argument("--wide-tensors", choices=["auto", "keep", "cast"], default="auto",
+                    help="what the bf16 engine does with tensors stored in 32 bits: auto (a checkpoint wholly in 32 bits is narrowed, "
+                         "single wide tensors of a 16-bit checkpoint stay wide), keep, cast")
+    ap.add_argument("--tune-library-products", action="store_true",
+                    help="time the vendor library's candidates for new product shapes of up to 256 rows and keep the fastest "
+                         "(results may then differ in their last bits from run to run)")
     args = ap.parse_args(argv)
     if (args.model_path is None) == (args.random_shape is None):
         ap.error("give either --model DIR or --random SHAPE")
@@ -90,6 +96,8 @@ def main(argv=None) -> int:
         max_model_len=min(args.max_length_of_generated_sequences, int(raw.get("max_position_embeddings", 1 << 30))),
         max_num_batched_tokens=args.max_num_batched_tokens,
         dtype=canonical_dtype(args.precision),
+        wide_tensors=args.wide_tensors,
+        tune_library_products=args.tune_library_products,
     )
     if model_config is None:
         engine = LLMEngine.from_random(raw, inference_config, precision=args.precision, seed=args.random_weights_seed or 0,
