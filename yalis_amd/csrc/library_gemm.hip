@@ -35,6 +35,19 @@ struct LtDevice {
   std::map<std::tuple<int, int, int, int, int, int, int>, LtPlan> plans;
 };
 
+// A process that meets ever new row counts (every portion length times every matrix of the model)
+// would keep a plan for each: beyond this many the plans of a device are dropped and made again
+// as their shapes come back (a plan is host memory only; making one takes some tens of microseconds).
+constexpr size_t LT_MAX_PLANS = 4096;
+
+void destroy_plan(LtPlan& plan) {
+  if (plan.a) hipblasLtMatrixLayoutDestroy(plan.a);
+  if (plan.b) hipblasLtMatrixLayoutDestroy(plan.b);
+  if (plan.c) hipblasLtMatrixLayoutDestroy(plan.c);
+  if (plan.desc) hipblasLtMatmulDescDestroy(plan.desc);
+  plan = LtPlan();
+}
+
 std::mutex g_lt_mutex;
 std::map<int, LtDevice> g_lt_devices;
 int g_lt_tune = 0;
@@ -93,6 +106,13 @@ extern "C" int yk_gemm_library(const void* x, const void* w, void* y, int y_dtyp
     // Row-major y = x . w^T is, in the library's column-major terms, Y (N x M) = W^T . X with
     // W stored K x N (leading dimension ldw) and X stored K x M (leading dimension ldx).
     LtPlan plan;
+    struct Guard {  // a plan that fails half-made gives back what it holds
+      LtPlan& plan;
+      bool kept = false;
+      ~Guard() {
+        if (!kept) destroy_plan(plan);
+      }
+    } guard{plan};
     LT_TRY(hipblasLtMatmulDescCreate(&plan.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F), "gemm_library: descriptor");
     const hipblasOperation_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
     LT_TRY(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta)), "gemm_library: transa");
@@ -143,7 +163,12 @@ extern "C" int yk_gemm_library(const void* x, const void* w, void* y, int y_dtyp
     }
     plan.algo = found[plan.chosen].algo;
     plan.workspace_need = found[plan.chosen].workspaceSize;
+    if (dev.plans.size() >= LT_MAX_PLANS) {
+      for (auto& kept : dev.plans) destroy_plan(kept.second);
+      dev.plans.clear();
+    }
     it = dev.plans.emplace(key, plan).first;
+    guard.kept = true;
   }
   const LtPlan& plan = it->second;
   // (the plan was made with the workspace of the call that first met the shape)
