@@ -62,7 +62,8 @@ def test_embed(ops, dtype):
 
 
 # ------------------------------------------------------------------------------ norm
-@pytest.mark.parametrize("width,rows", [(192, 7), (4096, 33), (1000, 3), (6144, 2)])
+# (from 1,024 rows on a thread of the fast form holds two pieces of its row)
+@pytest.mark.parametrize("width,rows", [(192, 7), (4096, 33), (1000, 3), (6144, 2), (3080, 1030), (72, 1025)])
 @pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
 def test_add_rmsnorm(ops, width, rows, act, wdtype):
