@@ -479,3 +479,31 @@ def test_full_width_replay_eight_layers_float32(capsys):
     with capsys.disabled():
         print(f"\n[full width, 8 layers, float32] largest difference from the plain implementation: {worst:.3e} (bound 1e-4); "
               f"from its float64 form: engine {ours:.3e}, plain float32 {theirs:.3e}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_pages_beyond_two_to_the_31_elements_of_the_pool(dtype):
+    """A pool whose keys (and values) are more than 2^31 elements a layer, the low pages held by
+    a request that is never stepped: the requests of a mixed trace live wholly above them, where
+    an offset computed in 32 bits would wrap."""
+    cfg, weights, reqs, want = setup("F", dtype)
+    page = PAGE["F"]
+    per_page = cfg["num_key_value_heads"] * page * cfg["head_dim"]
+    low = (2**31 + 2**27) // per_page
+    steps = C.trace_mixed(reqs)
+    n_pages = low + C.pages_needed(steps, reqs, page)
+    need = 2 * cfg["num_hidden_layers"] * n_pages * per_page * (4 if dtype == "float32" else 2)
+    if torch.cuda.mem_get_info()[0] < 1.2 * need:
+        pytest.skip("not enough free device memory for the pool")
+    runner = C.make_runner(cfg, weights, dtype, "cuda:0", ops_for("cuda:0"), page, n_pages, max_seqs=5)
+    holder = 10**6
+    assert runner.pages.admit(holder) is not None and runner.pages.reserve(holder, low * page)
+    got, rp = C.run_trace(runner, steps)
+    lowest = min(p for held in rp.page_log for tables in held.values() for t in tables for p in t if p >= 0)
+    assert lowest * per_page > 2**31
+    C.assert_matches(got, want, dtype == "bfloat16", "pages beyond 2^31 elements")
+    runner.pages.release(holder)
+    runner.pages.audit()
+    del runner
+    torch.cuda.empty_cache()

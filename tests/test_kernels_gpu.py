@@ -554,9 +554,11 @@ def test_rope_append_prompt_portions(ops, h, g, d, rd, page):
 
 
 # ------------------------------------------------------------------------- attention
-def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True, n_pages=64, plan=None, long_plan=None, col_tiles=1, with_cols=False):
+def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True, n_pages=64, plan=None, long_plan=None, col_tiles=1, with_cols=False,
+                    pool_pages=None):
     """spans: list of (cached tokens before the step, new tokens).  Builds pages in a
-    shuffled order, fills cache for the earlier tokens, runs rope-free attention."""
+    shuffled order, fills cache for the earlier tokens, runs rope-free attention.
+    pool_pages: the pages are the last n_pages of a pool of so many (never initialised below them)."""
     gen = torch.Generator().manual_seed(seed)
     order = torch.randperm(n_pages, generator=gen).tolist()
     kc = torch.zeros((n_pages, g, page, d), dtype=dtype)
@@ -577,7 +579,7 @@ def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True,
         for pos in range(total):
             kc[table[pos // page], :, pos % page, :] = k[pos]
             vc[table[pos // page], :, :, pos % page] = v[pos]
-        seqs.append(SeqSpan(tokens=[0] * new, first_position=cached, block_tables=[table], state_slot=0))
+        seqs.append(SeqSpan(tokens=[0] * new, first_position=cached, block_tables=[table + (pool_pages - n_pages if pool_pages else 0)], state_slot=0))
     hb = build_host_batch(seqs, 1, page)
     tpt = ops.attention_tokens_per_tile(h, g)
     big = ops.attention_long_span_tile(h, g)
@@ -593,8 +595,16 @@ def _attention_case(ops, dtype, h, g, d, page, spans, window, seed, poison=True,
     q = (torch.randn((n, h * d), generator=gen) * 1.5).to(dtype)
     scale = 1.0 / math.sqrt(d)
     kc_d, vc_d = device_cache(ops, kc, vc)
+    if pool_pages:
+        pool_k = torch.empty((pool_pages,) + tuple(kc_d.shape[1:]), dtype=dtype, device=DEV)
+        pool_v = torch.empty((pool_pages,) + tuple(vc_d.shape[1:]), dtype=dtype, device=DEV)
+        pool_k[pool_pages - n_pages:] = kc_d
+        pool_v[pool_pages - n_pages:] = vc_d
+        kc_d, vc_d = pool_k, pool_v
     got = ops.attention(q.to(DEV), h, g, d, kc_d, vc_d, page, scale, window, ctx, 0, ctx.arrays["tiles"], ctx.arrays["long_tiles"], plan=plan, long_plan=long_plan, long_col_tiles=col_tiles,
                         token_cols=ctx.arrays["cols"] if with_cols else None)
+    if pool_pages:
+        return got, None  # (the plain implementation would need the pool on the host)
     want = R.attention(q.float(), h, g, d, kc.float(), vc.float(), page, scale, window, ctx_cpu, 0, None)
     return got, want
 
@@ -886,6 +896,26 @@ def test_attention_gives_one_result_under_every_plan_its_policies_choose(ops, h,
         longest = max(c + n for c, n in spans)
         seen.add(HipOps.attention_plan(len(spans) * g, -(-longest // 64)))
     assert len(seen) > 1, "the workloads were meant to make the policy choose differently"
+
+
+@pytest.mark.parametrize("dtype,h,g,d,page", [(torch.bfloat16, 32, 8, 128, 64), (torch.bfloat16, 6, 3, 64, 16), (torch.float32, 4, 2, 48, 32)])
+def test_attention_in_a_pool_beyond_4_gib(ops, dtype, h, g, d, page):
+    """Pages whose offsets in the pool do not fit 32 bits (a pool of more than 4 GiB of keys, and
+    as much of values; more than 2^31 elements): the same bits as from the same pages at the
+    start of a small pool, for single tokens, short and long spans, keys split and not."""
+    free = torch.cuda.mem_get_info()[0]
+    per_page = g * page * d * (2 if dtype == torch.bfloat16 else 4)
+    pool_pages = (2**31 + 2**28) // (g * page * d)
+    if free < 2.5 * pool_pages * per_page:
+        pytest.skip("not enough free device memory for the pool")
+    assert pool_pages * g * page * d > 2**31
+    spans = [(0, 5), (17, 1), (0, 300), (63, 2), (700, 1), (31, 34), (200, 130)]
+    for plan, long_plan in ((None, None), ((4, 3), 2)):
+        small, want = _attention_case(ops, dtype, h, g, d, page, spans, 0, seed=5, plan=plan, long_plan=long_plan, n_pages=128)
+        big, _ = _attention_case(ops, dtype, h, g, d, page, spans, 0, seed=5, plan=plan, long_plan=long_plan, n_pages=128, pool_pages=pool_pages)
+        assert torch.equal(small, big)
+        close(small, want, 2e-5 if dtype == torch.float32 else 2e-2, 0 if dtype == torch.float32 else 2**-7)
+        torch.cuda.empty_cache()
 
 
 def test_attention_far_key_stands_out(ops):
