@@ -14,10 +14,10 @@ bits is a 32-bit copy of the model, not a statement about single tensors: the bf
 narrows it to bfloat16, as the reference casts every tensor to its parameter's dtype
 (yalis/model_loading.py:172-173).  ``wide_tensors`` overrides the rule: "keep" leaves every
 32-bit tensor wide (a float32 matrix in the bfloat16 engine then runs on the float32 kernels,
-which is said once, loudly), "cast" narrows all of them.  A checkpoint stored in float16 is
-refused by the bfloat16 engine: rounding it to bfloat16 would silently drop three bits of every
-weight (the reference runs such checkpoints in float16, a precision this engine does not
-have); the float32 engine takes it.
+which is said once, loudly), "cast" narrows all of them.  Tensors stored in float16 are rounded
+to bfloat16 by the bfloat16 engine (to nearest even; every float16 value lies within bfloat16's
+range), again as the reference casts to the parameter's dtype, and a warning says that three
+bits of each such weight's fraction are dropped; the float32 engine widens them exactly.
 """
 from __future__ import annotations
 
@@ -113,8 +113,6 @@ def check_against(entries: Dict[str, TensorEntry], wanted: Dict[str, TensorSpec]
             ok = tag in (_FLOAT_TAGS if s.kind == "float" else _INT_TAGS)
             if not ok:
                 wrong_kind.append((n, tag, s.kind))
-            elif tag == "F16" and engine_dtype == "bfloat16":
-                wrong_kind.append((n, tag, "bfloat16 or float32 (this engine has no float16; run it with precision fp32 or convert the checkpoint)"))
     if missing or unexpected or wrong_shape or wrong_kind:
         raise WeightsError(where, sorted(missing), sorted(unexpected), wrong_shape, wrong_kind)
 
@@ -163,6 +161,11 @@ def open_tensors(
     check_against(entries, wanted, model_dir, engine_dtype)
     keep_wide = keeps_wide(entries, wanted, wide_tensors)
     if engine_dtype == "bfloat16":
+        halves = [n for n, sp in wanted.items() if sp.kind == "float" and entries[n].dtype == "F16"]
+        if halves:
+            logger.warning("%d tensors of %s are stored in float16: the bfloat16 engine rounds them to bfloat16 (three bits of "
+                           "each weight's fraction are dropped; precision fp32 keeps them exactly); first: %s",
+                           len(halves), model_dir, halves[0])
         wide = [n for n, sp in wanted.items() if sp.kind == "float" and entries[n].dtype in ("F32", "F64")]
         matrices = [n for n in wide if len(wanted[n].shape) >= 2]
         if wide and not keep_wide:
