@@ -507,3 +507,23 @@ def test_pages_beyond_two_to_the_31_elements_of_the_pool(dtype):
     runner.pages.audit()
     del runner
     torch.cuda.empty_cache()
+
+
+def test_an_entry_without_tokens_sits_the_step_out():
+    """An entry that brings no tokens changes nothing (its request is as if left out of the
+    step); one that wants logits of tokens it did not bring is refused."""
+    from yalis_amd.engine.replay import Replayer, ReplayError
+
+    cfg, weights, reqs, want = setup("A", "float32")
+    toks = reqs["r1"]
+    runner = C.make_runner(cfg, weights, "float32", "cpu", ops_for("cpu"), 16, 8)
+    rp = Replayer(runner)
+    assert rp.run_step({"step": 0, "entries": [{"id": "x", "tokens": [], "want": []}], "end": []}) is None
+    a = rp.run_step({"step": 1, "entries": [{"id": "x", "tokens": toks[:9], "want": [8]}, {"id": "y", "tokens": []}], "end": []})
+    b = rp.run_step({"step": 2, "entries": [{"id": "x", "tokens": [], "want": []}], "end": []})
+    c = rp.run_step({"step": 3, "entries": [{"id": "x", "tokens": toks[9:], "want": [len(toks) - 10]}], "end": ["x"]})
+    assert b is None
+    assert (a[0] - want["r1"][8]).abs().max() < 2e-5 and (c[0] - want["r1"][-1]).abs().max() < 2e-5
+    with pytest.raises(ReplayError, match="brings no tokens"):
+        rp.run_step({"step": 4, "entries": [{"id": "z", "tokens": [], "want": [0]}], "end": []})
+    assert runner.pages.live_requests() == 0
