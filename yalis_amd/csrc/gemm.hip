@@ -132,10 +132,8 @@ union Frag8 {
 // rows beyond N are read from the last row and never stored, K beyond the slice is read
 // from valid places and meets zeros of x.
 constexpr int SK_KC = 256;            // K elements per chunk
-constexpr int SK_STEPS = SK_KC / 32;  // matrix-core steps per chunk
 constexpr int SK_PAD = 8;             // bf16 elements of padding per LDS row (keeps 16-byte reads conflict-free)
 constexpr int SK_ROW = SK_KC + SK_PAD;
-constexpr int SK_MAX_WAVES = 8;
 
 // x is parked in two buffers by turns where that costs no resident workgroup (up to 16 rows
 // of x): then one barrier a chunk is enough.  Measured: 2 to 5 % on the 8B shapes.

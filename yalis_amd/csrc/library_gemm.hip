@@ -146,19 +146,18 @@ extern "C" int yk_gemm_library(const void* x, const void* w, void* y, int y_dtyp
         bool ok = true;
         float ms = 0.f;
         for (int rep = 0; rep < 4 && ok; ++rep) {  // the first run of a kernel is not counted
-          if (rep == 1) hipEventRecord(e0, stream);
-          ok = hipblasLtMatmul(dev.handle, plan.desc, &alpha, w, plan.a, x, plan.b, &beta, y, plan.c, y, plan.c,
+          if (rep == 1) ok = hipEventRecord(e0, stream) == hipSuccess;
+          ok = ok && hipblasLtMatmul(dev.handle, plan.desc, &alpha, w, plan.a, x, plan.b, &beta, y, plan.c, y, plan.c,
                                &found[c].algo, workspace, workspace_bytes, stream) == HIPBLAS_STATUS_SUCCESS;
         }
-        hipEventRecord(e1, stream);
-        if (hipEventSynchronize(e1) != hipSuccess) ok = false;
+        if (hipEventRecord(e1, stream) != hipSuccess || hipEventSynchronize(e1) != hipSuccess) ok = false;
         if (ok && hipEventElapsedTime(&ms, e0, e1) == hipSuccess && ms < best) {
           best = ms;
           plan.chosen = c;
         }
       }
-      hipEventDestroy(e0);
-      hipEventDestroy(e1);
+      (void)hipEventDestroy(e0);
+      (void)hipEventDestroy(e1);
       (void)hipGetLastError();  // a candidate that failed to launch is simply not chosen
     }
     plan.algo = found[plan.chosen].algo;
