@@ -127,9 +127,12 @@ def layer_forward(
     positions: torch.Tensor,
     rounder: Rounder = _identity,
     window: Optional[int] = None,
+    residual_rounder: Rounder = _identity,
 ) -> torch.Tensor:
     """yalis/external/model.py:414-439 (pre-norm, sequential residuals) around
-    :525-608 (attention) and :740-744 (feed-forward).  x: [T, C] residual."""
+    :525-608 (attention) and :740-744 (feed-forward).  x: [T, C] residual.
+    ``residual_rounder`` rounds the residual stream after each sum: the reference in bfloat16
+    keeps the stream in bfloat16 (every tensor of :437-438 is), an engine may keep it wider."""
     n_head = cfg["num_attention_heads"]
     n_group = cfg.get("num_key_value_heads") or n_head
     head_dim = cfg.get("head_dim") or cfg["hidden_size"] // n_head
@@ -150,12 +153,12 @@ def layer_forward(
         q, k, v, 1.0 / math.sqrt(head_dim), positions, positions, window, round_p=rounder
     )
     a = rounder(a).reshape(t, n_head * head_dim)
-    x = x + rounder(a @ w("self_attn.o_proj.weight").T)
+    x = residual_rounder(x + rounder(a @ w("self_attn.o_proj.weight").T))
 
     h = rounder(rms_norm(x, w("post_attention_layernorm.weight"), eps))
-    x = x + swiglu_mlp(
+    x = residual_rounder(x + swiglu_mlp(
         h, w("mlp.gate_proj.weight"), w("mlp.up_proj.weight"), w("mlp.down_proj.weight"), rounder
-    )
+    ))
     return x
 
 
@@ -167,6 +170,7 @@ def forward(
     first_position: int = 0,
     dtype: torch.dtype = torch.float32,
     n_layers: Optional[int] = None,
+    residual_rounder: Rounder = _identity,
 ) -> torch.Tensor:
     """yalis/external/model.py:122-197: embedding, the blocks, final norm, head.
     Returns logits [T, V].  ``first_position`` shifts every position (only
@@ -176,7 +180,7 @@ def forward(
     positions = torch.arange(first_position, first_position + len(ids))
     n = cfg["num_hidden_layers"] if n_layers is None else n_layers
     for layer in range(n):
-        x = layer_forward(cfg, weights, layer, x, positions, rounder)
+        x = layer_forward(cfg, weights, layer, x, positions, rounder, residual_rounder=residual_rounder)
     h = rounder(rms_norm(x, weights["model.norm.weight"].to(dtype), cfg["rms_norm_eps"]))
     if cfg.get("tie_word_embeddings", False):
         head = weights["model.embed_tokens.weight"]

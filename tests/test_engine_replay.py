@@ -527,3 +527,22 @@ def test_an_entry_without_tokens_sits_the_step_out():
     with pytest.raises(ReplayError, match="brings no tokens"):
         rp.run_step({"step": 4, "entries": [{"id": "z", "tokens": [], "want": [0]}], "end": []})
     assert runner.pages.live_requests() == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "F"])
+def test_bfloat16_engine_beside_a_bfloat16_residual_stream(name):
+    """The reference in bfloat16 keeps the residual stream in bfloat16 (every sum of
+    yalis/external/model.py:437-438 is rounded); this engine keeps it in float32.  The plain
+    implementation with the stream rounded after every sum, which is the reference's arithmetic,
+    and the engine agree within the tolerance of two bfloat16 implementations of one model, and
+    so do the two plain forms (the deviation is rounding noise, not another model)."""
+    cfg, weights, reqs, want_wide = setup(name, "bfloat16")
+    w16 = {k: v.to(torch.bfloat16).float() for k, v in weights.items()}
+    narrow = {rid: P.forward(cfg, w16, toks, rounder=P.bf16_round, residual_rounder=P.bf16_round) for rid, toks in reqs.items()}
+    steps = C.trace_whole(reqs)
+    page = PAGE[name]
+    runner = C.make_runner(cfg, weights, "bfloat16", "cuda:0", ops_for("cuda:0"), page, C.pages_needed(steps, reqs, page))
+    got, _ = C.run_trace(runner, steps)
+    C.assert_matches(got, narrow, True, f"{name}/bfloat16 residual stream")
+    C.assert_matches(want_wide, narrow, True, f"{name}/the two plain forms")
