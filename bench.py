@@ -531,8 +531,8 @@ def main() -> int:
             del runner3
             torch.cuda.empty_cache()
             if not args.no_70b and torch.cuda.mem_get_info()[0] > 200e9:
-                # BASELINE's fifth configuration: the Llama-3.1-70B shape (141 GB of weights on the
-                # one GPU), decode at batch 1, 8 and 64 behind 2,048-token prompts
+                # the Llama-3.1-70B shape (141 GB of weights on the one GPU), decode at batch 1, 8
+                # and 64 behind 2,048-token prompts
                 name70, cfg70 = SHAPES["70b"]
                 shape70 = Shape(cfg70)
                 runner70 = make_runner(dict(cfg70), 64, 2048 + 64)
