@@ -518,7 +518,7 @@ def test_an_entry_without_tokens_sits_the_step_out():
     toks = reqs["r1"]
     runner = C.make_runner(cfg, weights, "float32", "cpu", ops_for("cpu"), 16, 8)
     rp = Replayer(runner)
-    assert rp.run_step({"step": 0, "entries": [{"id": "x", "tokens": [], "want": []}], "end": []}) is None
+    assert rp.run_step({"step": 0, "entries": [{"id": "x", "tokens": [], "want": []}, {"id": "never", "tokens": []}], "end": ["never"]}) is None
     a = rp.run_step({"step": 1, "entries": [{"id": "x", "tokens": toks[:9], "want": [8]}, {"id": "y", "tokens": []}], "end": []})
     b = rp.run_step({"step": 2, "entries": [{"id": "x", "tokens": [], "want": []}], "end": []})
     c = rp.run_step({"step": 3, "entries": [{"id": "x", "tokens": toks[9:], "want": [len(toks) - 10]}], "end": ["x"]})

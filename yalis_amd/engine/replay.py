@@ -38,6 +38,7 @@ class Replayer:
         """Runs one step; returns float32 logits [wanted, vocab] or None when
         nothing was wanted."""
         entries = []
+        sat_out = set()  # requests named with no tokens (one that never brought any holds nothing to give back)
         for e in step.get("entries", []):
             rid = str(e["id"])
             tokens = [int(t) for t in e["tokens"]]
@@ -45,6 +46,7 @@ class Replayer:
             if not tokens:
                 if want:
                     raise ReplayError(f"step {step.get('step')}: request {rid!r} brings no tokens but wants logits at {want}")
+                sat_out.add(rid)
                 continue  # an entry without tokens: the request sits this step out
             if rid not in self.handles:
                 handle = self._next
@@ -71,6 +73,8 @@ class Replayer:
         for rid in step.get("end", []):
             rid = str(rid)
             if rid not in self.handles:
+                if rid in sat_out:
+                    continue
                 raise ReplayError(f"step {step.get('step')}: cannot end unknown request {rid!r}")
             self.runner.release(self.handles.pop(rid))
         if logits is None or logits.shape[0] == 0:
