@@ -113,4 +113,4 @@ def test_trace_run_cli_refuses_an_overfull_pool(tmp_path):
          "--out", str(tmp_path / "o"), "--max-tokens", "64"],
         input=text, capture_output=True, text=True, timeout=600,
     )
-    assert proc.returncode != 0 and "no pages left" in proc.stderr
+    assert proc.returncode != 0 and "no pages left" in proc.stderr and "Traceback" not in proc.stderr
