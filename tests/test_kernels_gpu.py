@@ -211,6 +211,24 @@ def test_gemm_mfma_skinny_eight_waves(ops, forced):
     assert torch.equal(eight, ops.gemm_mfma_skinny(few, packed, torch.float32))
 
 
+def test_gemm_mfma_skinny_two_chunks_in_flight(ops, forced):
+    """Long slices of K with 33 to 64 rows of x and eight waves walk in short chunks, two in
+    flight per wave (a register set each, by turns): the same sums in the same order as one
+    long chunk at a time, so the same bits; slices of an even and of an odd number of chunks,
+    K no multiple of the chunk, the last slice shorter, one chunk only in a slice."""
+    for m, n, k, slices in [(64, 200, 16384, 2), (48, 136, 4096 + 2600, 1), (33, 520, 3 * 4224 + 72, 3), (64, 96, 4352, 1), (40, 130, 4200, 1)]:
+        x = rnd((m, k), torch.bfloat16, 6)
+        w = rnd((n, k), torch.bfloat16, 7)
+        forced(waves=8, slices=slices)
+        two = ops.gemm_mfma_skinny(x, w, torch.float32)   # the rule's own choice for these slices
+        forced(waves=8, slices=slices, chunk=256)
+        one = ops.gemm_mfma_skinny(x, w, torch.float32)
+        forced(waves=4, slices=slices, chunk=128)
+        four = ops.gemm_mfma_skinny(x, w, torch.float32)
+        assert torch.equal(two, one) and torch.equal(two, four), (m, n, k, slices)
+        close(two, x.double().cpu() @ w.double().cpu().T, 2e-5 * math.sqrt(k), 1e-5)
+
+
 @pytest.mark.parametrize("chunk", [128, 256])
 @pytest.mark.parametrize("waves", [4, 8])
 def test_gemm_mfma_skinny_wide_form(ops, forced, chunk, waves):

@@ -185,7 +185,7 @@ struct AttnSplits {
 };
 constexpr int SK_SPLITS_MAX_K_BLOCK = 1024;  // a workgroup's whole slice of x then fits beside the weights
 
-template <int MT, int W, typename TO, int GATED, bool FROM_SPLITS, int KC>
+template <int MT, int W, typename TO, int GATED, bool FROM_SPLITS, int KC, int DEPTH = 1>
 __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, float* __restrict__ part,
     TO* __restrict__ y, int M, int N, int K, int ldx, int ldw, int ldy, int k_block, AttnSplits xa) {
@@ -220,26 +220,29 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
 #pragma unroll
   for (int j = 0; j < STEPS; ++j) wrow[j] = w + static_cast<size_t>(min(n0 + RPL * j + half, N - 1)) * ldw;
   const int k_last = K - 8;
-  u32x4_t regs[STEPS];
-#define SK_LOAD_W(KC0)                                                                      \
+  // DEPTH chunks are in flight per wave, each in a register set of its own
+  u32x4_t regs[DEPTH][STEPS];
+#define SK_LOAD_W(S, KC0)                                                                   \
   {                                                                                          \
     const int kk_ = min((KC0) + 8 * l32, k_last);                                            \
     _Pragma("unroll") for (int j = 0; j < STEPS; ++j)                                     \
-        regs[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wrow[j] + kk_)); \
+        regs[S][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wrow[j] + kk_)); \
   }
   // x: the chunk's 16*MT rows x 32 pieces of 16 bytes are spread over the threads, XP each;
   // what lies outside M or the slice is loaded from a clamped address and parked as zero
   constexpr int XP = 16 * MT * (KC / 8) / (W * 64);
   static_assert(XP * W * 64 == 16 * MT * (KC / 8), "x pieces must divide evenly over the threads");
   const u32x4_t zero = {0u, 0u, 0u, 0u};
-  u32x4_t xr[XP];
+  u32x4_t xr[DEPTH][XP];
 #pragma unroll
-  for (int p = 0; p < XP; ++p) xr[p] = zero;
-#define SK_LOAD_X(KC0)                                                                      \
+  for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+    for (int p = 0; p < XP; ++p) xr[d][p] = zero;
+#define SK_LOAD_X(S, KC0)                                                                   \
   _Pragma("unroll") for (int p = 0; p < XP; ++p) {                                           \
     const int e_ = threadIdx.x + p * W * 64;                                                 \
     const int m_ = m0 + e_ / (KC / 8), k_ = (KC0) + 8 * (e_ % (KC / 8));               \
-    if (m_ < M) xr[p] = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(m_) * ldx + min(k_, k_last)); \
+    if (m_ < M) xr[S][p] = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(m_) * ldx + min(k_, k_last)); \
   }
 
   // The workgroups of a launch do not all start at the same place of their slices: workgroup b
@@ -263,7 +266,7 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
     if (j >= slots) j -= slots;
     return kb0 + j * KC;
   };
-  SK_LOAD_W(chunk_start(0))
+  SK_LOAD_W(0, chunk_start(0))
   if (FROM_SPLITS) {
     // (the first chunk of the weights is in flight meanwhile)
     const int pieces = k_block / 4;
@@ -289,10 +292,22 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
       *reinterpret_cast<u32x2_t*>(x_all + static_cast<size_t>(m) * x_all_row + kk) = piece;
     }
   } else {
-    SK_LOAD_X(chunk_start(0))
+    SK_LOAD_X(0, chunk_start(0))
   }
+#pragma unroll
+  for (int d = 1; d < DEPTH; ++d)
+    if (d < n_chunks) {
+      SK_LOAD_W(d, chunk_start(d))
+      if (!FROM_SPLITS) {
+        SK_LOAD_X(d, chunk_start(d))
+      }
+    }
   int turn = 0;
-  for (int ci = 0; ci < n_chunks; ++ci, turn ^= 1) {
+  for (int ci0 = 0; ci0 < n_chunks; ci0 += DEPTH) {
+#pragma unroll
+   for (int d = 0; d < DEPTH; ++d) {
+    const int ci = ci0 + d;
+    if (DEPTH > 1 && ci >= n_chunks) continue;  // (the same in every wave)
     const int kc = chunk_start(ci);
     // With one buffer every wave must have read the previous chunk of x before it is
     // overwritten.  With two, the buffer written now was last read two chunks ago, and every
@@ -301,7 +316,7 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
     bf16_t(*xs)[ROW] = xs0 + (XB == 2 ? turn * 16 * MT : 0);
     // park what has arrived, then put the next chunk's loads in flight
 #pragma unroll
-    for (int j = 0; j < STEPS; ++j) *reinterpret_cast<u32x4_t*>(&wl[RPL * j + half][8 * l32]) = regs[j];
+    for (int j = 0; j < STEPS; ++j) *reinterpret_cast<u32x4_t*>(&wl[RPL * j + half][8 * l32]) = regs[d][j];
     if (!FROM_SPLITS) {
 #pragma unroll
       for (int p = 0; p < XP; ++p) {
@@ -309,14 +324,14 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
         // wait for everything it has just put in flight)
         const int e = threadIdx.x + p * W * 64;
         const bool outside = m0 + e / (KC / 8) >= M || kc + 8 * (e % (KC / 8)) >= kb1;
-        *reinterpret_cast<u32x4_t*>(&xs[e / (KC / 8)][8 * (e % (KC / 8))]) = outside ? zero : xr[p];
+        *reinterpret_cast<u32x4_t*>(&xs[e / (KC / 8)][8 * (e % (KC / 8))]) = outside ? zero : xr[d][p];
       }
     }
-    if (ci + 1 < n_chunks) {
-      const int kc_next = chunk_start(ci + 1);
-      SK_LOAD_W(kc_next)
+    if (ci + DEPTH < n_chunks) {
+      const int kc_next = chunk_start(ci + DEPTH);
+      SK_LOAD_W(d, kc_next)
       if (!FROM_SPLITS) {
-        SK_LOAD_X(kc_next)
+        SK_LOAD_X(d, kc_next)
       }
     }
     __syncthreads();
@@ -348,6 +363,8 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
       __builtin_amdgcn_sched_barrier(0);
     }
 #undef SK_READ
+    turn ^= 1;
+   }
   }
 #undef SK_LOAD_W
 #undef SK_LOAD_X
@@ -671,9 +688,23 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, i
   dim3 grid((N + 16 * waves - 1) / (16 * waves), (M + 16 * mt - 1) / (16 * mt), splits);
   YK_REQUIRE(grid.y <= 65535, "gemm_mfma_skinny: too many rows for one launch");
   dim3 block(waves * 64);
-  const int kc = skinny_chunk(mt, k_block);
+  int kc = skinny_chunk(mt, k_block);
+  // Long slices with 64 rows of x and eight waves: short chunks, two of them in flight per wave
+  // (a register set each), in place of one long chunk: the same bytes in flight with half the
+  // LDS a workgroup parks them in and a finer walk.  Measured on the 70B shape's down projection
+  // (8,192 x 28,672 in four slices of 7,168; us, one long chunk / two short ones): 97.8 / 82.8 at
+  // 64 rows of x, 96.7 / 80.2 at 48.  Where the slices are short enough for short chunks anyway,
+  // a second chunk in flight costs 2 to 5 % (8B shape at 64 rows: gate/up 45.5 -> 46.6 us, down
+  // 23.5 -> 24.5, qkv 13.9 -> 15.0), and four cost 8 to 10 %: the kernel is not short of bytes in
+  // flight there.
+  const bool wide = mt == 4 && (g_wide == 2 || (g_wide == 1 && K >= SK_WIDE_MIN_K && splits == 1));
+  int depth = 1;
+  if (!wide && mt == 4 && waves == 8 && !gated && !g_force_chunk && kc == SK_KC) {
+    kc = 128;
+    depth = 2;
+  }
   const size_t lds = skinny_lds_bytes(mt, waves, kc);
-  if (mt == 4 && (g_wide == 2 || (g_wide == 1 && K >= SK_WIDE_MIN_K && splits == 1))) {
+  if (wide) {
     // waves of 32 weight rows: two of them (64 rows a workgroup) by the rule, half the plan's
     // number (the plan's rows a workgroup) when forced
     const int ww = g_wide == 2 ? waves / 2 : 2;
@@ -701,19 +732,20 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, i
 #undef SKW_GO_KC
     return yk_fail("gemm_mfma_skinny: no wide kernel for this plan");
   }
-#define SK_GO(MT_, W_, G_) SK_GO_KC(MT_, W_, G_, 128) SK_GO_KC(MT_, W_, G_, 256)
-#define SK_GO_KC(MT_, W_, G_, KC_)                                                                       \
-  if (mt == MT_ && waves == W_ && gated == G_ && kc == KC_) {                                           \
+#define SK_GO(MT_, W_, G_) SK_GO_KC(MT_, W_, G_, 128, 1) SK_GO_KC(MT_, W_, G_, 256, 1)
+#define SK_GO_KC(MT_, W_, G_, KC_, D_)                                                                   \
+  if (mt == MT_ && waves == W_ && gated == G_ && kc == KC_ && depth == D_) {                            \
     static bool raised = false; /* allow more than the default 64 KB of dynamic LDS, once */           \
     if (!raised) {                                                                                      \
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_kernel<MT_, W_, TO, G_, false, KC_>), \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_kernel<MT_, W_, TO, G_, false, KC_, D_>), \
                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)    \
         return yk_fail("gemm_mfma_skinny: cannot raise the LDS limit");                                 \
       raised = true;                                                                                    \
     }                                                                                                   \
-    gemm_mfma_skinny_kernel<MT_, W_, TO, G_, false, KC_><<<grid, block, lds, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block, AttnSplits{}); \
+    gemm_mfma_skinny_kernel<MT_, W_, TO, G_, false, KC_, D_><<<grid, block, lds, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block, AttnSplits{}); \
     return yk_check_launch("gemm_mfma_skinny");                                                         \
   }
+  SK_GO_KC(4, 8, 0, 128, 2)
   SK_GO(1, 4, 0) SK_GO(2, 4, 0) SK_GO(4, 4, 0) SK_GO(4, 8, 0)
   if constexpr (sizeof(TO) == 2) {  // gated results are bfloat16 only
     SK_GO(1, 4, 1) SK_GO(2, 4, 1) SK_GO(4, 4, 1) SK_GO(4, 8, 1) SK_GO(1, 4, 2) SK_GO(2, 4, 2) SK_GO(4, 4, 2) SK_GO(4, 8, 2)
