@@ -273,6 +273,21 @@ def test_gemm_mfma_skinny_wide_form(ops, forced, chunk, waves):
         x, w = rnd((48, 8192), torch.bfloat16, 8, 0.3), rnd((136, 8192), torch.bfloat16, 9, 0.05)
         by_rule = ops.gemm_mfma_skinny(x, w, torch.float32)
         close(by_rule, x.double().cpu() @ w.double().cpu().T, 2e-5 * math.sqrt(8192), 1e-5)
+        # with more than 48 rows of x the rule keeps two long chunks in flight per wave: the same
+        # bits as one at a time (a forced chunk length), on a K of an odd number of chunks and a tail
+        for m, k in ((64, 8192 + 256 + 72), (49, 8192)):
+            x, w = rnd((m, k), torch.bfloat16, 8, 0.3), rnd((136, k), torch.bfloat16, 9, 0.05)
+            forced(slices=1)
+            two = ops.gemm_mfma_skinny(x, w, torch.float32)
+            forced(slices=1, chunk=256)
+            assert torch.equal(two, ops.gemm_mfma_skinny(x, w, torch.float32))
+            close(two, x.double().cpu() @ w.double().cpu().T, 2e-5 * math.sqrt(k), 1e-5)
+            packed, group = ops.pack_gate_up(rnd((72, k), torch.bfloat16, 31, 0.05), rnd((72, k), torch.bfloat16, 32, 0.05))
+            forced()
+            got = ops.gate_up_act(x, packed, group, "silu", torch.bfloat16)
+            forced(chunk=256)
+            assert torch.equal(got, ops.gate_up_act(x, packed, group, "silu", torch.bfloat16))
+        forced()
     finally:
         ops.wide_skinny_products(1)
 

@@ -425,7 +425,7 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_kernel(
 // once a workgroup, clamped addresses instead of conditions) is the 16-row form's.
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
-template <int W, typename TO, int GATED, int KC>
+template <int W, typename TO, int GATED, int KC, int DEPTH = 1>
 __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_wide_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, float* __restrict__ part,
     TO* __restrict__ y, int M, int N, int K, int ldx, int ldw, int ldy, int k_block) {
@@ -455,44 +455,54 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_wide_kernel(
 #pragma unroll
   for (int j = 0; j < LOADS; ++j) wrow[j] = w + static_cast<size_t>(min(n0 + RPL * j + half, N - 1)) * ldw;
   const int k_last = K - 8;
-  u32x4_t regs[LOADS];
-#define SKW_LOAD_W(KC0)                                                                     \
+  u32x4_t regs[DEPTH][LOADS];  // DEPTH chunks in flight per wave, a register set each
+#define SKW_LOAD_W(S, KC0)                                                                  \
   {                                                                                          \
     const int kk_ = min((KC0) + 8 * l32, k_last);                                            \
     _Pragma("unroll") for (int j = 0; j < LOADS; ++j)                                        \
-        regs[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wrow[j] + kk_)); \
+        regs[S][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wrow[j] + kk_)); \
   }
   constexpr int XP = 64 * (KC / 8) / (W * 64);
   static_assert(XP * W * 64 == 64 * (KC / 8), "x pieces must divide evenly over the threads");
   const u32x4_t zero = {0u, 0u, 0u, 0u};
-  u32x4_t xr[XP];
+  u32x4_t xr[DEPTH][XP];
 #pragma unroll
-  for (int p = 0; p < XP; ++p) xr[p] = zero;
-#define SKW_LOAD_X(KC0)                                                                     \
+  for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+    for (int p = 0; p < XP; ++p) xr[d][p] = zero;
+#define SKW_LOAD_X(S, KC0)                                                                  \
   _Pragma("unroll") for (int p = 0; p < XP; ++p) {                                           \
     const int e_ = threadIdx.x + p * W * 64;                                                 \
     const int m_ = m0 + e_ / (KC / 8), k_ = (KC0) + 8 * (e_ % (KC / 8));                     \
-    if (m_ < M) xr[p] = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(m_) * ldx + min(k_, k_last)); \
+    if (m_ < M) xr[S][p] = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(m_) * ldx + min(k_, k_last)); \
   }
   const int n_chunks = (kb1 - kb0 + KC - 1) / KC;
-  SKW_LOAD_W(kb0)
-  SKW_LOAD_X(kb0)
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+    if (d < n_chunks) {
+      SKW_LOAD_W(d, kb0 + d * KC)
+      SKW_LOAD_X(d, kb0 + d * KC)
+    }
   int turn = 0;
-  for (int ci = 0; ci < n_chunks; ++ci, turn ^= 1) {
+  for (int ci0 = 0; ci0 < n_chunks; ci0 += DEPTH) {
+#pragma unroll
+   for (int d = 0; d < DEPTH; ++d) {
+    const int ci = ci0 + d;
+    if (DEPTH > 1 && ci >= n_chunks) continue;  // (the same in every wave)
     const int kc = kb0 + ci * KC;
     if (XB == 1) __syncthreads();
     bf16_t(*xs)[ROW] = xs0 + (XB == 2 ? turn * 64 : 0);
 #pragma unroll
-    for (int j = 0; j < LOADS; ++j) *reinterpret_cast<u32x4_t*>(&wl[RPL * j + half][8 * l32]) = regs[j];
+    for (int j = 0; j < LOADS; ++j) *reinterpret_cast<u32x4_t*>(&wl[RPL * j + half][8 * l32]) = regs[d][j];
 #pragma unroll
     for (int p = 0; p < XP; ++p) {
       const int e = threadIdx.x + p * W * 64;
       const bool outside = m0 + e / (KC / 8) >= M || kc + 8 * (e % (KC / 8)) >= kb1;
-      *reinterpret_cast<u32x4_t*>(&xs[e / (KC / 8)][8 * (e % (KC / 8))]) = outside ? zero : xr[p];
+      *reinterpret_cast<u32x4_t*>(&xs[e / (KC / 8)][8 * (e % (KC / 8))]) = outside ? zero : xr[d][p];
     }
-    if (ci + 1 < n_chunks) {
-      SKW_LOAD_W(kc + KC)
-      SKW_LOAD_X(kc + KC)
+    if (ci + DEPTH < n_chunks) {
+      SKW_LOAD_W(d, kc + DEPTH * KC)
+      SKW_LOAD_X(d, kc + DEPTH * KC)
     }
     __syncthreads();
     constexpr int AHEAD = 3;
@@ -517,6 +527,8 @@ __global__ __launch_bounds__(W * 64) void gemm_mfma_skinny_wide_kernel(
       __builtin_amdgcn_sched_barrier(0);
     }
 #undef SKW_READ
+    turn ^= 1;
+   }
   }
 #undef SKW_LOAD_W
 #undef SKW_LOAD_X
@@ -711,19 +723,27 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, float* part, TO* y, i
     dim3 wblock(ww * 64);
     grid.x = (N + 32 * ww - 1) / (32 * ww);
     const size_t lds = skinny_lds_bytes(mt, 2 * ww, kc);
-#define SKW_GO(W_, G_) SKW_GO_KC(W_, G_, 128) SKW_GO_KC(W_, G_, 256)
-#define SKW_GO_KC(W_, G_, KC_)                                                                          \
-  if (ww == W_ && gated == G_ && kc == KC_) {                                                           \
+#define SKW_GO(W_, G_) SKW_GO_KC(W_, G_, 128, 1) SKW_GO_KC(W_, G_, 256, 1)
+#define SKW_GO_KC(W_, G_, KC_, D_)                                                                      \
+  if (ww == W_ && gated == G_ && kc == KC_ && wdepth == D_) {                                           \
     static bool raised = false;                                                                         \
     if (!raised) {                                                                                      \
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_wide_kernel<W_, TO, G_, KC_>), \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_skinny_wide_kernel<W_, TO, G_, KC_, D_>), \
                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)    \
         return yk_fail("gemm_mfma_skinny: cannot raise the LDS limit");                                 \
       raised = true;                                                                                    \
     }                                                                                                   \
-    gemm_mfma_skinny_wide_kernel<W_, TO, G_, KC_><<<grid, wblock, lds, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block); \
+    gemm_mfma_skinny_wide_kernel<W_, TO, G_, KC_, D_><<<grid, wblock, lds, stream>>>(x, w, part, y, M, N, K, ldx, ldw, ldy, k_block); \
     return yk_check_launch("gemm_mfma_skinny (wide)");                                                  \
   }
+    // With more than 48 rows of x the rule's two waves keep two long chunks in flight each (the 70B
+    // shape's gate/up, us, one / two: 186.5 / 176 at 64 rows; 170 / 172 at 48 and 164 / 165 at 33,
+    // so not there).
+    const int wdepth = g_wide == 1 && !g_force_chunk && M > 48 && kc == SK_KC ? 2 : 1;
+    SKW_GO_KC(2, 0, 256, 2)
+    if constexpr (sizeof(TO) == 2) {
+      SKW_GO_KC(2, 1, 256, 2) SKW_GO_KC(2, 2, 256, 2)
+    }
     SKW_GO(2, 0) SKW_GO(4, 0)
     if constexpr (sizeof(TO) == 2) {
       SKW_GO(2, 1) SKW_GO(4, 1) SKW_GO(2, 2) SKW_GO(4, 2)
